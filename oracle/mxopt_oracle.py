@@ -1,0 +1,468 @@
+"""CPU oracle for the optimizer-step path of mlx-node (TEST INFRASTRUCTURE ONLY).
+
+This module restates, in NumPy float32 and one rounded operation at a time, what
+the reference's optimizer path computes.  It exists to check the HIP kernels; it is
+never imported by the product package, only by tests, the smoke check and the
+CPU-baseline leg of the benchmark.
+
+Conventions shared by every function here
+-----------------------------------------
+* The reference builds each optimizer as a chain of MLX element-wise ops, and MLX
+  rounds to float32 after every op.  Every line below is therefore exactly one
+  IEEE float32 operation on arrays (NumPy does not contract a*b+c).
+* Every host scalar reaches MLX as ``array(static_cast<float>(value))``
+  (crates/mlx-sys/src/mlx.cpp:335-338, 525-547): coefficients are evaluated in
+  float64 on the host and only then cast to float32.  ``_f32`` is that cast.
+* bfloat16 tensors are carried as ``numpy.uint16`` bit patterns.  A bf16 operand
+  combined with a float32 scalar array promotes to float32 (MLX type promotion),
+  so the optimizers below up-cast bf16 inputs, compute in float32 and return
+  float32, exactly like ``update_single`` which never casts back
+  (crates/mlx-core/src/optimizers/adamw.rs:81-142).
+
+What pins each function (see tests/test_oracle_*.py)
+----------------------------------------------------
+* SGD, SGD+momentum, L2 decay, clip-by-value, gradient norm, clip-by-norm,
+  LR schedules, gradient accumulation, apply_gradients: the closed-form
+  known-answer values held by the reference's own tests
+  (__test__/core/optimizers.test.ts, __test__/trainers/grpo-gradient-accumulation.test.ts,
+  __test__/training/basic-training.test.ts).
+* Adam/AdamW (bias correction on, one tensor), SGD, RMSprop, clip_grad_norm:
+  agreement with torch.optim / torch.nn.utils (a library that is not the
+  reference) to ~1e-6 relative, plus float64 brute force on small inputs.
+* f32<->bf16 conversion: bit-exact against torch's CPU conversion.
+
+PARITY UNPINNED (no reference test, fixture or buildable reference covers it):
+* bf16 inputs through any optimizer (promotion to float32 is MLX's documented
+  rule but no reference test runs it);
+* the order in which MLX sums squares for the global norm (the oracle uses the
+  exact float64 sum, rounded once);
+* NaN handling of ``clip`` (NaN is propagated here);
+* the per-call ``step`` quirk, Nesterov's stored state and the
+  ``(m/(sqrt(v)+eps))*lr`` association are pinned only by reading the source.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+F32 = np.float32
+
+
+def _f32(x: float) -> np.float32:
+    """float64 host scalar -> float32 MLX scalar (mlx.cpp:335-338, 531-535)."""
+    return np.float32(np.float64(x))
+
+
+# --------------------------------------------------------------------------
+# bfloat16 helpers (bit patterns in uint16)
+# --------------------------------------------------------------------------
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    """Exact widening of bf16 bit patterns to float32."""
+    bits = np.asarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit patterns, round-to-nearest-even; NaN stays a quiet NaN.
+
+    This is ``astype(bfloat16)`` of the reference (models/qwen3/model.rs:2443-2448).
+    """
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    lsb = (u >> np.uint32(16)) & np.uint32(1)
+    rounded = ((u + np.uint32(0x7FFF) + lsb) >> np.uint32(16)).astype(np.uint16)
+    nan = np.isnan(x)
+    if np.any(nan):
+        quiet = ((u >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16)
+        rounded = np.where(nan, quiet, rounded)
+    return rounded
+
+
+def as_f32(x: np.ndarray) -> np.ndarray:
+    """Promote an oracle tensor (float32, or bf16 bits as uint16) to float32."""
+    x = np.asarray(x)
+    if x.dtype == np.uint16:
+        return bf16_to_f32(x)
+    if x.dtype == np.float16:
+        return x.astype(np.float32)
+    if x.dtype != np.float32:
+        raise TypeError(f"oracle tensors are float32, float16 or uint16(bf16); got {x.dtype}")
+    return x
+
+
+def is_bf16(x: np.ndarray) -> bool:
+    return np.asarray(x).dtype == np.uint16
+
+
+# --------------------------------------------------------------------------
+# Optimizers  (crates/mlx-core/src/optimizers/{adam,adamw,sgd,rmsprop}.rs)
+# --------------------------------------------------------------------------
+
+class Adam:
+    """optimizers/adam.rs:41-153.  ``step`` counts update_single CALLS (adam.rs:73)."""
+
+    def __init__(self, learning_rate: Optional[float] = None, beta1: Optional[float] = None,
+                 beta2: Optional[float] = None, eps: Optional[float] = None,
+                 bias_correction: Optional[bool] = None):
+        self.learning_rate = 1e-3 if learning_rate is None else float(learning_rate)
+        self.beta1 = 0.9 if beta1 is None else float(beta1)
+        self.beta2 = 0.999 if beta2 is None else float(beta2)
+        self.eps = 1e-8 if eps is None else float(eps)
+        self.bias_correction = False if bias_correction is None else bool(bias_correction)
+        self.step = 0
+        self.state: Dict[str, Tuple[np.ndarray, np.ndarray]] = {}
+
+    def _decayed(self, p: np.ndarray) -> np.ndarray:
+        return p
+
+    def update_single(self, param_name: str, param: np.ndarray, grad: np.ndarray) -> np.ndarray:
+        p = as_f32(param)
+        g = as_f32(grad)
+        if param_name not in self.state:  # init_state: float32 zeros (adam.rs:148-153)
+            self.state[param_name] = (np.zeros(p.shape, F32), np.zeros(p.shape, F32))
+        self.step += 1
+        m, v = self.state[param_name]
+
+        pd = self._decayed(p)
+        beta1_m = m * _f32(self.beta1)
+        omb1_g = g * _f32(1.0 - self.beta1)
+        new_m = beta1_m + omb1_g
+        g_sq = g * g                               # mlx square
+        beta2_v = v * _f32(self.beta2)
+        omb2_g2 = g_sq * _f32(1.0 - self.beta2)
+        new_v = beta2_v + omb2_g2
+        if self.bias_correction:
+            t = float(self.step)
+            bc1 = 1.0 / (1.0 - math.pow(self.beta1, t))
+            bc2 = 1.0 / (1.0 - math.pow(self.beta2, t))
+            m_hat = new_m * _f32(bc1)
+            v_hat = new_v * _f32(bc2)
+        else:
+            m_hat, v_hat = new_m, new_v
+        sqrt_v = np.sqrt(v_hat)
+        denom = sqrt_v + _f32(self.eps)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            update = m_hat / denom
+        lr_update = update * _f32(self.learning_rate)
+        new_p = pd - lr_update
+        self.state[param_name] = (new_m, new_v)    # UNcorrected moments are stored
+        return new_p
+
+    def reset(self) -> None:
+        self.state.clear()
+        self.step = 0
+
+
+class AdamW(Adam):
+    """optimizers/adamw.rs:43-157: Adam plus the decoupled decay multiply (adamw.rs:83-84)."""
+
+    def __init__(self, learning_rate=None, beta1=None, beta2=None, eps=None,
+                 weight_decay: Optional[float] = None, bias_correction=None):
+        super().__init__(learning_rate, beta1, beta2, eps, bias_correction)
+        self.weight_decay = 0.01 if weight_decay is None else float(weight_decay)
+
+    def _decayed(self, p: np.ndarray) -> np.ndarray:
+        return p * _f32(1.0 - self.learning_rate * self.weight_decay)
+
+
+class SGD:
+    """optimizers/sgd.rs:40-159."""
+
+    def __init__(self, learning_rate: float, momentum: Optional[float] = None,
+                 weight_decay: Optional[float] = None, dampening: Optional[float] = None,
+                 nesterov: Optional[bool] = None):
+        momentum = 0.0 if momentum is None else float(momentum)
+        dampening = 0.0 if dampening is None else float(dampening)
+        nesterov = False if nesterov is None else bool(nesterov)
+        if nesterov and (momentum <= 0.0 or dampening != 0.0):     # sgd.rs:51-56
+            raise ValueError("Nesterov momentum requires momentum > 0 and dampening = 0")
+        self.learning_rate = float(learning_rate)
+        self.momentum = momentum
+        self.weight_decay = 0.0 if weight_decay is None else float(weight_decay)
+        self.dampening = dampening
+        self.nesterov = nesterov
+        self.state: Dict[str, Optional[np.ndarray]] = {}
+
+    def update_single(self, param_name: str, param: np.ndarray, grad: np.ndarray) -> np.ndarray:
+        p = as_f32(param)
+        g = as_f32(grad)
+        self.state.setdefault(param_name, None)
+        if self.weight_decay != 0.0:                                # sgd.rs:86-94
+            ge = g + p * _f32(self.weight_decay)
+        else:
+            ge = g
+        if self.momentum != 0.0:
+            v = self.state[param_name]
+            if v is not None:                                       # sgd.rs:98-106
+                new_v = v * _f32(self.momentum) + ge * _f32(1.0 - self.dampening)
+            else:                                                   # first call: copy (sgd.rs:107-114)
+                new_v = ge * _f32(1.0)
+            if self.nesterov:                                       # sgd.rs:117-125
+                final = new_v + ge
+            else:
+                final = new_v
+            self.state[param_name] = final                          # sgd.rs:130 stores final_update
+            update = final
+        else:
+            update = ge
+        return p - update * _f32(self.learning_rate)                # sgd.rs:139-140
+
+    def reset(self) -> None:
+        self.state.clear()
+
+
+class RMSprop:
+    """optimizers/rmsprop.rs:36-127."""
+
+    def __init__(self, learning_rate: Optional[float] = None, alpha: Optional[float] = None,
+                 eps: Optional[float] = None, weight_decay: Optional[float] = None):
+        self.learning_rate = 1e-2 if learning_rate is None else float(learning_rate)
+        self.alpha = 0.99 if alpha is None else float(alpha)
+        self.eps = 1e-8 if eps is None else float(eps)
+        self.weight_decay = 0.0 if weight_decay is None else float(weight_decay)
+        self.state: Dict[str, np.ndarray] = {}
+
+    def update_single(self, param_name: str, param: np.ndarray, grad: np.ndarray) -> np.ndarray:
+        p = as_f32(param)
+        g = as_f32(grad)
+        if param_name not in self.state:
+            self.state[param_name] = np.zeros(p.shape, F32)
+        v = self.state[param_name]
+        if self.weight_decay != 0.0:                                # rmsprop.rs:69-77
+            ge = g + p * _f32(self.weight_decay)
+        else:
+            ge = g
+        g_sq = ge * ge
+        new_v = v * _f32(self.alpha) + g_sq * _f32(1.0 - self.alpha)  # rmsprop.rs:80-83
+        denom = np.sqrt(new_v) + _f32(self.eps)                     # rmsprop.rs:86-88
+        with np.errstate(divide="ignore", invalid="ignore"):
+            update = ge / denom                                     # rmsprop.rs:91
+        new_p = p - update * _f32(self.learning_rate)               # rmsprop.rs:92-93
+        self.state[param_name] = new_v
+        return new_p
+
+    def reset(self) -> None:
+        self.state.clear()
+
+
+# --------------------------------------------------------------------------
+# Gradient utilities  (optimizers/mod.rs:33-227, gradients/mod.rs:233-312)
+# --------------------------------------------------------------------------
+
+def exact_sumsq(grads: Iterable[np.ndarray]) -> float:
+    """Sum of squares of the stored gradient values, accumulated in float64."""
+    total = 0.0
+    for g in grads:
+        x = as_f32(g).astype(np.float64).ravel()
+        total += float(np.dot(x, x))
+    return total
+
+
+def clip_value(grad: np.ndarray, lo: float, hi: float) -> np.ndarray:
+    """``clip`` with float32 bounds (mlx.cpp:469-481); a non-finite bound is 'no bound'.
+    Returns float32.  NaN elements stay NaN."""
+    g = as_f32(grad)
+    out = g
+    if math.isfinite(lo):
+        out = np.where(np.isnan(out), out, np.maximum(out, _f32(lo)))
+    if math.isfinite(hi):
+        out = np.where(np.isnan(out), out, np.minimum(out, _f32(hi)))
+    return out.astype(F32, copy=False)
+
+
+def norm_scale_c1(sumsq: float, max_norm: float) -> Tuple[np.float32, np.float32]:
+    """(norm, scale) of ``GradientUtils::clip_grad_norm`` (optimizers/mod.rs:87-96):
+    n = sqrt(S) in float32, scale = min(f32(max) / (n + f32(1e-6)), 1.0f)."""
+    n = np.float32(math.sqrt(sumsq))
+    with np.errstate(divide="ignore", over="ignore"):
+        scale = np.minimum(_f32(max_norm) / (n + _f32(1e-6)), F32(1.0))
+    return n, F32(scale)
+
+
+class GradientUtils:
+    """optimizers/mod.rs:33-227."""
+
+    @staticmethod
+    def compute_gradient_norm(gradients: Dict[str, np.ndarray]) -> float:
+        """optimizers/mod.rs:43-55: float64 sum of squares of the float32 read-back."""
+        return math.sqrt(exact_sumsq(gradients.values()))
+
+    @staticmethod
+    def clip_grad_norm(gradients: Dict[str, np.ndarray], max_norm: float) -> Dict[str, np.ndarray]:
+        """optimizers/mod.rs:67-107.  Every tensor is multiplied by the scale, also when it is 1."""
+        if not gradients:
+            return {}
+        _, scale = norm_scale_c1(exact_sumsq(gradients.values()), max_norm)
+        return {k: as_f32(g) * scale for k, g in gradients.items()}
+
+    @staticmethod
+    def clip_grad_norm_with_norm(gradients, max_norm):
+        """optimizers/mod.rs:116-158: also returns the float32 norm widened to float64."""
+        if not gradients:
+            return {}, 0.0
+        n, scale = norm_scale_c1(exact_sumsq(gradients.values()), max_norm)
+        return {k: as_f32(g) * scale for k, g in gradients.items()}, float(n)
+
+    @staticmethod
+    def clip_grad_value(grad: np.ndarray, min_val: float, max_val: float) -> np.ndarray:
+        """optimizers/mod.rs:164-166."""
+        return clip_value(grad, min_val, max_val)
+
+    @staticmethod
+    def clip_grad_value_and_norm(gradients, clip_val: float, max_norm: Optional[float]):
+        """optimizers/mod.rs:174-226: clamp to +-clip_val, then clip_grad_norm of the clamped values."""
+        if not gradients:
+            return {}
+        clamped = {k: clip_value(g, -clip_val, clip_val) for k, g in gradients.items()}
+        if max_norm is None:
+            return clamped
+        _, scale = norm_scale_c1(exact_sumsq(clamped.values()), max_norm)
+        return {k: g * scale for k, g in clamped.items()}
+
+
+def clip_gradients_by_global_norm(gradients: Sequence[np.ndarray], max_norm: float) -> List[np.ndarray]:
+    """gradients/mod.rs:233-285: float64 norm on the host; unchanged copies when n <= max,
+    otherwise multiply by f32(max / (n + 1e-6)) evaluated in float64."""
+    if not gradients:
+        return []
+    n = math.sqrt(exact_sumsq(gradients))
+    if n <= max_norm:
+        return [np.array(g, copy=True) for g in gradients]
+    scale = _f32(max_norm / (n + 1e-6))
+    return [as_f32(g) * scale for g in gradients]
+
+
+def clip_gradients_by_value(gradients: Sequence[np.ndarray], lo: float, hi: float) -> List[np.ndarray]:
+    """gradients/mod.rs:299-312."""
+    return [clip_value(g, lo, hi) for g in gradients]
+
+
+# --------------------------------------------------------------------------
+# Accumulation and plain-SGD apply
+# --------------------------------------------------------------------------
+
+def _add_promoted(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """MLX ``add`` of two tensors: result dtype = promote(a, b).  bf16 + bf16 is one
+    float32 add rounded to bf16; any float32 operand makes the result float32."""
+    s = as_f32(a) + as_f32(b)
+    if is_bf16(a) and is_bf16(b):
+        return f32_to_bf16(s)
+    return s
+
+
+def accumulate_gradients(accumulated: Dict[str, np.ndarray], new: Dict[str, np.ndarray]) -> Dict[str, np.ndarray]:
+    """Qwen3Model::accumulate_gradients, models/qwen3/model.rs:2217-2243 (also the engine's
+    variant, grpo/engine.rs:2632-2666, which differs only in when it evaluates)."""
+    out: Dict[str, np.ndarray] = {}
+    for name, g in new.items():
+        if name in accumulated:
+            out[name] = _add_promoted(accumulated[name], g)
+        else:
+            out[name] = np.array(g, copy=True)
+    for name, a in accumulated.items():
+        if name not in out:
+            out[name] = np.array(a, copy=True)
+    return out
+
+
+def accumulate_gradients_sft(accumulated: Optional[Dict[str, np.ndarray]], new: Dict[str, np.ndarray]):
+    """sft/engine.rs:282-290: names missing from the accumulator are silently dropped."""
+    if accumulated is None:
+        return {k: np.array(v, copy=True) for k, v in new.items()}
+    out = dict(accumulated)
+    for name, g in new.items():
+        if name in out:
+            out[name] = _add_promoted(out[name], g)
+    return out
+
+
+def accumulate_fp32(acc: Optional[np.ndarray], grad: np.ndarray) -> np.ndarray:
+    """Mixed-precision accumulation buffer: acc(float32) + widen(grad); first call = widen.
+    (The intent stated at grpo/autograd.rs:317-318; the reference itself sums in grad dtype.)"""
+    g = as_f32(grad)
+    return g.astype(F32, copy=True) if acc is None else acc + g
+
+
+def mul_scalar(x: np.ndarray, value: float) -> np.ndarray:
+    """``mul_scalar`` (mlx.cpp:531-535): promotes to float32."""
+    return as_f32(x) * _f32(value)
+
+
+def apply_gradients(params: Dict[str, np.ndarray], gradients: Dict[str, np.ndarray],
+                    learning_rate: float) -> Dict[str, np.ndarray]:
+    """Qwen3Model::apply_gradients, models/qwen3/model.rs:2409-2460: plain SGD in the
+    parameter's dtype.  lr is cast to the parameter dtype, lr*g and p-(lr*g) are each one
+    rounded op in the promoted dtype, the result is cast back to the parameter dtype."""
+    out: Dict[str, np.ndarray] = {}
+    for name, g in gradients.items():
+        if name not in params:
+            raise KeyError(f"Parameter '{name}' not found in model")   # model.rs:2427-2432
+        p = params[name]
+        lr32 = _f32(learning_rate)
+        if is_bf16(p):
+            lr_p = bf16_to_f32(f32_to_bf16(np.array([lr32], F32)))[0]
+            scaled = lr_p * as_f32(g)
+            if is_bf16(g):
+                scaled = bf16_to_f32(f32_to_bf16(scaled))              # bf16*bf16 -> bf16
+                out[name] = f32_to_bf16(bf16_to_f32(p) - scaled)       # bf16-bf16 -> bf16
+            else:
+                out[name] = f32_to_bf16(bf16_to_f32(p) - scaled)       # fp32 result cast back
+        else:
+            out[name] = as_f32(p) - lr32 * as_f32(g)
+    return out
+
+
+# --------------------------------------------------------------------------
+# Learning-rate schedules  (optimizers/mod.rs:239-292) -- host float64 closed forms
+# --------------------------------------------------------------------------
+
+def _idiv(a: int, b: int) -> int:
+    """Rust i64 division truncates toward zero."""
+    q = abs(a) // abs(b)
+    return q if (a >= 0) == (b >= 0) else -q
+
+
+class LRScheduler:
+    @staticmethod
+    def linear_decay(initial_lr: float, final_lr: float, current_step: int, total_steps: int) -> float:
+        if current_step >= total_steps:
+            return final_lr
+        return initial_lr + (final_lr - initial_lr) * (current_step / total_steps)
+
+    @staticmethod
+    def exponential_decay(initial_lr: float, decay_rate: float, current_step: int, decay_steps: int) -> float:
+        # integer division of the step counters (optimizers/mod.rs:263)
+        return initial_lr * math.pow(decay_rate, float(_idiv(current_step, decay_steps)))
+
+    @staticmethod
+    def cosine_annealing(initial_lr: float, min_lr: float, current_step: int, total_steps: int) -> float:
+        if current_step >= total_steps:
+            return min_lr
+        progress = current_step / total_steps
+        return min_lr + (initial_lr - min_lr) * 0.5 * (1.0 + math.cos(progress * math.pi))
+
+    @staticmethod
+    def step_decay(initial_lr: float, factor: float, current_step: int, step_size: int) -> float:
+        return initial_lr * (factor ** _idiv(current_step, step_size))
+
+
+# --------------------------------------------------------------------------
+# Helpers used by parity tests
+# --------------------------------------------------------------------------
+
+def ulp_diff_f32(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """Distance in float32 units-in-the-last-place (monotone integer mapping)."""
+    def key(x):
+        i = np.ascontiguousarray(x, dtype=np.float32).view(np.int32).astype(np.int64)
+        return np.where(i < 0, np.int64(-(2 ** 31)) - i, i)
+    return np.abs(key(a) - key(b))
+
+
+def ulp_diff_bf16(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    def key(x):
+        i = np.asarray(x, dtype=np.uint16).view(np.int16).astype(np.int64)
+        return np.where(i < 0, np.int64(-(2 ** 15)) - i, i)
+    return np.abs(key(a_bits) - key(b_bits))
