@@ -1,0 +1,221 @@
+/* mxopt -- MI355X (gfx950) kernels for the optimizer step of mlx-node, C ABI.
+ *
+ * This is the boundary a host (the reference's Rust crate `mlx-core`, or any other
+ * caller) binds instead of building every optimizer out of ~13 lazy MLX element-wise
+ * ops per tensor.  Every entry point takes plain pointers and sizes; device buffers
+ * are owned by the caller and are never freed or retained beyond the lifetime of the
+ * table that names them.  Nothing here allocates per call: a table (descriptors +
+ * chunk list on the device) is built once for a parameter list and reused every step.
+ *
+ * All arithmetic is IEEE float32, one rounding per reference op, in the reference's
+ * op order, so results are bit-identical to the reference's float32 op chain.
+ * 16-bit tensors (bf16, f16) are widened on load and rounded to nearest-even once on
+ * store.  Hyper-parameters cross the boundary ALREADY CAST to float32 the way the
+ * reference casts them: evaluated in float64 on the host, then static_cast<float>
+ * (crates/mlx-sys/src/mlx.cpp:335-338, 531-535); the *_hp_from_f64 helpers do that.
+ *
+ * Error convention: every call returns an int status (0 = ok), never throws or aborts
+ * across the boundary, and leaves a message readable with mxopt_last_error()
+ * (mirrors the reference's "null handle => Err(message)" idiom,
+ * crates/mlx-core/src/array/handle.rs:4-16, and napi Status::{InvalidArg,GenericFailure}).
+ *
+ * Threading: calls on one context are serialised by the caller; different contexts
+ * may be used from different threads.  Kernels are enqueued on the context's stream;
+ * no call synchronises with the host except mxopt_synchronize / mxopt_read_*.
+ */
+#ifndef MXOPT_H
+#define MXOPT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes = the reference's DType enum (crates/mlx-core/src/array/mod.rs:17-26,
+ * crates/mlx-sys/src/mlx.cpp:152-157).  Only the floating types are accepted. */
+enum { MXOPT_F32 = 0, MXOPT_I32 = 1, MXOPT_F16 = 2, MXOPT_BF16 = 3, MXOPT_U32 = 4 };
+
+enum {
+  MXOPT_OK = 0,
+  MXOPT_ERR_INVALID_ARG = 1, /* napi Status::InvalidArg (sgd.rs:51-56) */
+  MXOPT_ERR_FAILURE = 2,     /* napi Status::GenericFailure (model.rs:2427-2432) */
+  MXOPT_ERR_HIP = 3,         /* a HIP runtime call failed; message carries hipGetErrorString */
+  MXOPT_ERR_OOM = 4
+};
+
+typedef struct mxopt_ctx mxopt_ctx;
+typedef struct mxopt_table mxopt_table;
+
+/* ---- context -------------------------------------------------------------------- */
+
+/* One context per optimizer object / engine.  `hip_stream` is a hipStream_t (NULL = the
+ * device's default stream).  Replaces nothing in the reference: MLX owns one implicit
+ * device stream (crates/mlx-core/src/stream.rs). */
+int mxopt_create(int device, void* hip_stream, mxopt_ctx** out);
+void mxopt_destroy(mxopt_ctx* ctx);
+/* Last error message of `ctx` (or of the calling thread when ctx is NULL). Never NULL. */
+const char* mxopt_last_error(const mxopt_ctx* ctx);
+/* Waits for everything enqueued on the context's stream (the reference's eval(),
+ * crates/mlx-sys/src/mlx.cpp:189-209). */
+int mxopt_synchronize(mxopt_ctx* ctx);
+/* Tuning knobs, by name: "grid_blocks_per_cu" (persistent grid = CUs x this),
+ * "persistent" (0: one workgroup per chunk for the update kernels). */
+int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value);
+int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
+
+/* ---- tensor table ------------------------------------------------------------------
+ * One descriptor per tensor.  Which fields a kernel reads is listed at that kernel;
+ * unused pointers may be NULL.  All buffers are dense, `n` elements long.
+ * Buffers need only their natural alignment; tensors whose used pointers are all
+ * 16-byte aligned take the 128-bit path, others an element-wise path. */
+typedef struct mxopt_tensor {
+  const void* p;     /* parameter, read                                             */
+  void*       p_out; /* parameter, written; may equal p (in place)                  */
+  const void* g;     /* gradient, read                                              */
+  void*       g_out; /* transformed gradient (mxopt_grad_transform), or the
+                        accumulation buffer (mxopt_accumulate: read+written)        */
+  float*      m;     /* first moment, float32, in place (Adam/AdamW)                */
+  float*      v;     /* second moment (Adam/AdamW/RMSprop) or velocity (SGD),
+                        float32, in place                                           */
+  uint64_t    n;     /* elements; 0 is legal and skipped                            */
+  uint8_t     p_dtype, p_out_dtype, g_dtype, g_out_dtype; /* MXOPT_F32/F16/BF16     */
+  uint32_t    flags; /* MXOPT_TF_*                                                  */
+  float       bc1;   /* f32(1/(1-beta1^t)) for THIS tensor, 1.0f when bias          */
+  float       bc2;   /* correction is off (t counts update_single calls:
+                        adam.rs:73, adamw.rs:77, so it differs per tensor)          */
+} mxopt_tensor;
+
+#define MXOPT_TF_FIRST 0x1u /* SGD: no velocity stored yet -> v' = ge (sgd.rs:107-114); v is not read */
+
+int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxopt_table** out);
+/* Per-step scalars, `n` entries each; a NULL array leaves that field unchanged. */
+int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* bc2, const uint32_t* flags);
+void mxopt_table_destroy(mxopt_table* t);
+uint64_t mxopt_table_total_elems(const mxopt_table* t);
+uint64_t mxopt_table_num_chunks(const mxopt_table* t);
+uint64_t mxopt_table_num_tensors(const mxopt_table* t);
+#define MXOPT_CHUNK_ELEMS 4096 /* elements one workgroup handles per table entry */
+
+/* ---- device-resident result of the global-norm reduction ------------------------ */
+typedef struct mxopt_norm_result {
+  double   sumsq;     /* sum of squares, accumulated in float64                     */
+  double   norm;      /* sqrt(sumsq)                                                */
+  float    norm_f32;  /* (float)norm: what clip_grad_norm_with_norm returns          */
+  float    scale;     /* clip factor, see mxopt_clip_mode                           */
+  uint64_t nonfinite; /* number of NaN/Inf gradient elements seen                   */
+} mxopt_norm_result;
+
+/* How `scale` is derived from the norm. */
+enum {
+  /* GradientUtils::clip_grad_norm (optimizers/mod.rs:87-96):
+   * scale = min(f32(max) / (norm_f32 + f32(1e-6)), 1.0f), applied also when it is 1. */
+  MXOPT_CLIP_ALWAYS_MULTIPLY = 0,
+  /* clip_gradients_by_global_norm (gradients/mod.rs:255-270): norm <= max -> 1.0f
+   * exactly (gradients unchanged), else f32(max / (norm + 1e-6)) evaluated in float64. */
+  MXOPT_CLIP_IF_ABOVE = 1
+};
+
+/* ---- gradient pre-processing done in registers ----------------------------------
+ * g_eff = clamp_post( d_scale * clamp_pre( pre_mul * g ) ), each stage optional, each one
+ * float32 op per reference op.  Covers the engines' orders:
+ *  GRPO: clamp(+-v) -> clip-norm                 (grpo/engine.rs:636-653)
+ *  SFT : x(1/N) -> clip-norm -> clamp(+-v)       (sft/engine.rs:299-329)
+ * The global norm is always taken after pre_mul and clamp_pre.  NaN passes through
+ * the clamps unchanged. */
+typedef struct mxopt_grad_prep {
+  int          has_pre_mul;    float pre_mul;           /* f32(1/N) (sft/engine.rs:299-306) */
+  int          has_clamp_pre;  float pre_lo, pre_hi;    /* mlx clip, mlx.cpp:469-481        */
+  const float* d_scale;        /* device scalar (e.g. &norm_result->scale); NULL = none    */
+  int          has_clamp_post; float post_lo, post_hi;
+} mxopt_grad_prep;
+
+/* ---- hyper-parameters: float32 coefficients exactly as the reference hands them to MLX */
+typedef struct mxopt_adam_hp {
+  float lr, beta1, beta2, one_minus_beta1, one_minus_beta2, eps;
+  float decay;           /* f32(1 - lr*wd) (adamw.rs:83); used when decoupled_decay      */
+  int   decoupled_decay; /* 1 = AdamW (adamw.rs:84), 0 = Adam (adam.rs:108)              */
+} mxopt_adam_hp;
+void mxopt_adam_hp_from_f64(double lr, double beta1, double beta2, double eps, double weight_decay,
+                            int decoupled_decay, mxopt_adam_hp* out);
+/* bc = f32(1/(1-beta^t)) in float64 then cast (adamw.rs:99-104). */
+void mxopt_bias_correction(double beta1, double beta2, int64_t t, float* bc1, float* bc2);
+
+typedef struct mxopt_sgd_hp {
+  float lr, momentum, one_minus_dampening, weight_decay;
+  int   has_weight_decay; /* wd != 0 (sgd.rs:86) */
+  int   has_momentum;     /* momentum != 0 (sgd.rs:96) */
+  int   nesterov;         /* stores v'+ge as the new state (sgd.rs:117-130) */
+} mxopt_sgd_hp;
+/* Returns MXOPT_ERR_INVALID_ARG for nesterov with momentum <= 0 or dampening != 0 (sgd.rs:51-56). */
+int mxopt_sgd_hp_from_f64(double lr, double momentum, double weight_decay, double dampening, int nesterov,
+                          mxopt_sgd_hp* out);
+
+typedef struct mxopt_rmsprop_hp {
+  float lr, alpha, one_minus_alpha, eps, weight_decay;
+  int   has_weight_decay;
+} mxopt_rmsprop_hp;
+void mxopt_rmsprop_hp_from_f64(double lr, double alpha, double eps, double weight_decay, mxopt_rmsprop_hp* out);
+
+/* ---- update kernels: one launch per dtype group for the whole table -------------- */
+
+/* Adam / AdamW step.  Reads p, g, m, v; writes p_out, m, v.
+ * Replaces the 12/13-op chains of Adam::update_single (optimizers/adam.rs:77-108) and
+ * AdamW::update_single (optimizers/adamw.rs:81-116) for every tensor of the table.
+ * `prep` may be NULL. */
+int mxopt_adam(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp, const mxopt_grad_prep* prep);
+
+/* SGD with momentum / dampening / Nesterov / coupled L2.  Reads p, g, v (unless
+ * MXOPT_TF_FIRST); writes p_out, v.  Replaces SGD::update_single (optimizers/sgd.rs:84-150). */
+int mxopt_sgd(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp, const mxopt_grad_prep* prep);
+
+/* RMSprop.  Reads p, g, v; writes p_out, v.  Replaces RMSprop::update_single
+ * (optimizers/rmsprop.rs:67-112). */
+int mxopt_rmsprop(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* hp, const mxopt_grad_prep* prep);
+
+/* Plain SGD in the parameter's dtype: p_out = astype(p - astype(lr, dtype(p)) * g, dtype(p)),
+ * with the intermediate product rounded to the 16-bit dtype when p and g share it.
+ * Optional coupled decay g + f32(wd)*p first (sft/engine.rs:345-365).
+ * Replaces Qwen3Model::apply_gradients (models/qwen3/model.rs:2434-2451). */
+int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
+                    const mxopt_grad_prep* prep);
+
+/* ---- global norm ------------------------------------------------------------------ */
+
+/* Sum of squares of the gradients (after prep's pre_mul / clamp_pre) over the whole
+ * table: wavefront shuffle -> LDS -> one float64 partial per workgroup -> one
+ * single-workgroup second pass; no atomics, run-to-run deterministic.  `which` = 0 reads
+ * tensor.g, 1 reads tensor.g_out (the accumulation buffer).  If max_norm >= 0 the second
+ * pass also derives `scale` per `clip_mode`; otherwise scale = 1.  Writes *d_result
+ * (device memory).  Replaces the square/sum/add chain of GradientUtils::clip_grad_norm
+ * (optimizers/mod.rs:76-96), compute_gradient_norm (:43-55) and the per-tensor reductions
+ * of clip_gradients_by_global_norm (gradients/mod.rs:246-256). */
+int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep,
+                      double max_norm, int clip_mode, mxopt_norm_result* d_result);
+
+/* g_out = prep(g) element-wise (scale and/or clamps): the scale pass of clip_grad_norm
+ * (optimizers/mod.rs:98-102), clip_grad_value (:164-166), clip_gradients_by_value
+ * (gradients/mod.rs:299-312).  Only needed when the clipped gradients themselves must be
+ * handed back; the update kernels apply `prep` in registers instead. */
+int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep);
+
+/* ---- accumulation -------------------------------------------------------------------
+ * g_out = first ? astype(g) : g_out + g, in promote(dtype(g_out), dtype(g)) then stored as
+ * dtype(g_out).  With a float32 g_out and bf16 g this is the mixed-precision accumulation
+ * buffer; with equal dtypes it is the reference's `acc.add(&grad)`
+ * (models/qwen3/model.rs:2227, grpo/engine.rs:2643, sft/engine.rs:285).  If d_result is not
+ * NULL the sum of squares of the NEW buffer contents (after prep's pre_mul/clamp_pre) is
+ * reduced in the same pass and finished exactly like mxopt_global_norm. */
+int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep,
+                     double max_norm, int clip_mode, mxopt_norm_result* d_result);
+
+/* ---- small host<->device helpers (each synchronises the context's stream) --------- */
+int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out);
+
+const char* mxopt_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXOPT_H */

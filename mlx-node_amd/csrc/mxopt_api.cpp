@@ -1,0 +1,524 @@
+// C ABI of mxopt: contexts, tensor tables and kernel entry points (host side).
+// Declarations and the reference interfaces they replace are in include/mxopt.h.
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "mxopt.h"
+#include "mxopt_host_types.h"
+#include "mxopt_launch.h"
+
+namespace mxopt {
+
+static thread_local std::string g_thread_error;
+
+int fail(mxopt_ctx* ctx, int code, const std::string& msg) {
+  if (ctx) ctx->err = msg;
+  g_thread_error = msg;
+  return code;
+}
+
+int hip_fail(mxopt_ctx* ctx, hipError_t e, const char* what) {
+  return fail(ctx, e == hipErrorOutOfMemory ? MXOPT_ERR_OOM : MXOPT_ERR_HIP,
+              std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(ctx, call)                                   \
+  do {                                                       \
+    hipError_t e_ = (call);                                  \
+    if (e_ != hipSuccess) return hip_fail((ctx), e_, #call); \
+  } while (0)
+
+static bool float_dtype(int dt) { return dt == MXOPT_F32 || dt == MXOPT_F16 || dt == MXOPT_BF16; }
+
+float round_to_dtype(float x, int dt) {
+  if (dt == MXOPT_BF16) {
+    uint32_t u;
+    std::memcpy(&u, &x, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+      u = ((u >> 16) | 0x40u) << 16;
+    } else {
+      u = ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16;
+    }
+    std::memcpy(&x, &u, 4);
+    return x;
+  }
+  if (dt == MXOPT_F16) return (float)(_Float16)x;
+  return x;
+}
+
+static DevPrep make_prep(const mxopt_grad_prep* p) {
+  DevPrep d{};
+  d.d_scale = nullptr;
+  d.pre_mul = 1.0f;
+  d.pre_lo = d.post_lo = -INFINITY;
+  d.pre_hi = d.post_hi = INFINITY;
+  d.flags = 0;
+  if (!p) return d;
+  d.d_scale = p->d_scale;
+  if (p->has_pre_mul) { d.flags |= kPrepPreMul; d.pre_mul = p->pre_mul; }
+  // A non-finite bound means "no bound" (mlx.cpp:473-478); +-inf leaves values untouched.
+  if (p->has_clamp_pre) {
+    d.flags |= kPrepClampPre;
+    if (std::isfinite(p->pre_lo)) d.pre_lo = p->pre_lo;
+    if (std::isfinite(p->pre_hi)) d.pre_hi = p->pre_hi;
+  }
+  if (p->has_clamp_post) {
+    d.flags |= kPrepClampPost;
+    if (std::isfinite(p->post_lo)) d.post_lo = p->post_lo;
+    if (std::isfinite(p->post_hi)) d.post_hi = p->post_hi;
+  }
+  return d;
+}
+
+static bool prep_active(const mxopt_grad_prep* p) {
+  return p && (p->has_pre_mul || p->has_clamp_pre || p->d_scale || p->has_clamp_post);
+}
+
+static uint32_t persistent_grid(const mxopt_ctx* ctx, uint32_t nchunks) {
+  uint64_t cap = (uint64_t)ctx->num_cus * (uint64_t)ctx->grid_blocks_per_cu;
+  return (uint32_t)std::min<uint64_t>(nchunks, std::max<uint64_t>(cap, 1));
+}
+
+static int ensure_partials(mxopt_ctx* ctx, size_t need) {
+  if (need <= ctx->partial_cap) return MXOPT_OK;
+  size_t cap = std::max<size_t>(need, 4096);
+  double* ps = nullptr;
+  unsigned long long* pc = nullptr;
+  HIP_TRY(ctx, hipMalloc((void**)&ps, cap * sizeof(double)));
+  hipError_t e = hipMalloc((void**)&pc, cap * sizeof(unsigned long long));
+  if (e != hipSuccess) {
+    (void)hipFree(ps);
+    return hip_fail(ctx, e, "hipMalloc(partials)");
+  }
+  // Earlier launches may still be reading the old buffers.
+  if (ctx->d_partial_sum) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->d_partial_sum);
+    (void)hipFree(ctx->d_partial_cnt);
+  }
+  ctx->d_partial_sum = ps;
+  ctx->d_partial_cnt = pc;
+  ctx->partial_cap = cap;
+  return MXOPT_OK;
+}
+
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = true;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != dev) ok = hipSetDevice(dev) == hipSuccess;
+  }
+  ~DeviceGuard() {
+    int cur = -1;
+    if (prev >= 0 && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+  }
+};
+
+static int check_launch(mxopt_ctx* ctx, const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(ctx, e, what);
+  return MXOPT_OK;
+}
+
+// Which descriptor pointers an entry point dereferences.
+enum : uint32_t { kNeedP = 1, kNeedPOut = 2, kNeedG = 4, kNeedGOut = 8, kNeedM = 16, kNeedV = 32 };
+
+static int require(mxopt_ctx* ctx, const mxopt_table* t, uint32_t need, const char* op) {
+  if (!ctx || !t) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null context or table");
+  if (t->ctx != ctx) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": table belongs to another context");
+  if ((t->have_mask & need) != need) {
+    static const char* names[] = {"p", "p_out", "g", "g_out", "m", "v"};
+    std::string missing;
+    for (int b = 0; b < 6; ++b)
+      if ((need & (1u << b)) && !(t->have_mask & (1u << b))) missing += std::string(missing.empty() ? "" : ", ") + names[b];
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": table has tensors with a NULL pointer for: " + missing);
+  }
+  return MXOPT_OK;
+}
+
+static Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Group& g, bool persistent) {
+  Launch L;
+  L.tensors = t->d_tensors;
+  L.chunks = t->d_chunks + g.chunk_begin;
+  L.nchunks = g.nchunks;
+  L.grid = persistent ? persistent_grid(ctx, g.nchunks) : g.nchunks;
+  L.stream = ctx->stream;
+  L.nontemporal = ctx->nontemporal != 0;
+  return L;
+}
+
+static std::string dtype_names(const Group& g) {
+  auto nm = [](int d) { return d == MXOPT_F32 ? "f32" : d == MXOPT_BF16 ? "bf16" : d == MXOPT_F16 ? "f16" : "?"; };
+  return std::string("p=") + nm(g.pd) + " g=" + nm(g.gd) + " p_out=" + nm(g.pod) + " g_out=" + nm(g.god);
+}
+
+// Second pass shared by mxopt_global_norm and mxopt_accumulate.
+static int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode,
+                       mxopt_norm_result* d_result) {
+  const int has_max = max_norm >= 0.0;
+  launch_norm_finish(ctx->stream, ctx->d_partial_sum, ctx->d_partial_cnt, npartials, max_norm, has_max, clip_mode,
+                     d_result);
+  return check_launch(ctx, "norm_finish_kernel");
+}
+
+static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, const mxopt_grad_prep* prep,
+                     double max_norm, int clip_mode, mxopt_norm_result* d_result, const char* op) {
+  if (clip_mode != MXOPT_CLIP_ALWAYS_MULTIPLY && clip_mode != MXOPT_CLIP_IF_ABOVE)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unknown clip mode");
+  DeviceGuard guard(ctx->device);
+  const DevPrep dp = make_prep(prep);
+  size_t total_grid = 0;
+  for (const Group& g : t->groups) total_grid += persistent_grid(ctx, g.nchunks);
+  const bool want = d_result != nullptr;
+  if (want) {
+    int rc = ensure_partials(ctx, std::max<size_t>(total_grid, 1));
+    if (rc) return rc;
+  }
+  size_t offset = 0;
+  for (const Group& g : t->groups) {
+    Launch L = make_launch(ctx, t, g, true);
+    const int ad = mode == 0 ? g.gd : g.god;
+    if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr,
+                      want ? ctx->d_partial_cnt + offset : nullptr))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
+    int rc = check_launch(ctx, op);
+    if (rc) return rc;
+    offset += L.grid;
+  }
+  if (want) return finish_norm(ctx, (uint32_t)offset, max_norm, clip_mode, d_result);
+  return MXOPT_OK;
+}
+
+template <class F>
+static int run_update(mxopt_ctx* ctx, const mxopt_table* t, const char* op, F&& launch_one) {
+  DeviceGuard guard(ctx->device);
+  for (const Group& g : t->groups) {
+    Launch L = make_launch(ctx, t, g, ctx->persistent != 0);
+    if (!launch_one(g, L)) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
+    int rc = check_launch(ctx, op);
+    if (rc) return rc;
+  }
+  return MXOPT_OK;
+}
+
+}  // namespace mxopt
+
+using namespace mxopt;
+
+extern "C" {
+
+const char* mxopt_version(void) { return "mxopt 0.1 (gfx950)"; }
+
+int mxopt_create(int device, void* hip_stream, mxopt_ctx** out) {
+  if (!out) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_create: out is NULL");
+  *out = nullptr;
+  int ndev = 0;
+  HIP_TRY(nullptr, hipGetDeviceCount(&ndev));
+  if (device < 0 || device >= ndev) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_create: no such device");
+  hipDeviceProp_t prop;
+  HIP_TRY(nullptr, hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(nullptr, MXOPT_ERR_FAILURE,
+                std::string("mxopt_create: kernels are built for gfx950 only, device is ") + prop.gcnArchName);
+  mxopt_ctx* ctx = new (std::nothrow) mxopt_ctx();
+  if (!ctx) return fail(nullptr, MXOPT_ERR_OOM, "mxopt_create: out of host memory");
+  ctx->device = device;
+  ctx->stream = (hipStream_t)hip_stream;
+  ctx->num_cus = prop.multiProcessorCount;
+  *out = ctx;
+  return MXOPT_OK;
+}
+
+void mxopt_destroy(mxopt_ctx* ctx) {
+  if (!ctx) return;
+  DeviceGuard guard(ctx->device);
+  if (ctx->d_partial_sum) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->d_partial_sum);
+    (void)hipFree(ctx->d_partial_cnt);
+  }
+  delete ctx;
+}
+
+const char* mxopt_last_error(const mxopt_ctx* ctx) { return ctx ? ctx->err.c_str() : g_thread_error.c_str(); }
+
+int mxopt_synchronize(mxopt_ctx* ctx) {
+  if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_synchronize: null context");
+  DeviceGuard guard(ctx->device);
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  return MXOPT_OK;
+}
+
+int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
+  if (!ctx || !name) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: null argument");
+  std::string n(name);
+  if (n == "grid_blocks_per_cu") {
+    if (value < 1 || value > 64) return fail(ctx, MXOPT_ERR_INVALID_ARG, "grid_blocks_per_cu must be in [1, 64]");
+    ctx->grid_blocks_per_cu = (int)value;
+  } else if (n == "persistent") {
+    ctx->persistent = value != 0;
+  } else if (n == "nontemporal") {
+    ctx->nontemporal = value != 0;
+  } else {
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: unknown option " + n);
+  }
+  return MXOPT_OK;
+}
+
+int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
+  if (!ctx || !name || !value) return MXOPT_ERR_INVALID_ARG;
+  std::string n(name);
+  if (n == "grid_blocks_per_cu") *value = ctx->grid_blocks_per_cu;
+  else if (n == "persistent") *value = ctx->persistent;
+  else if (n == "nontemporal") *value = ctx->nontemporal;
+  else if (n == "num_cus") *value = ctx->num_cus;
+  else return MXOPT_ERR_INVALID_ARG;
+  return MXOPT_OK;
+}
+
+// ---- tables ---------------------------------------------------------------------------
+
+static void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d) {
+  d.p = s.p; d.p_out = s.p_out; d.g = s.g; d.g_out = s.g_out; d.m = s.m; d.v = s.v;
+  d.n = s.n; d.bc1 = s.bc1; d.bc2 = s.bc2;
+  d.flags = s.flags & ~kTfUnaligned;
+  const void* ptrs[6] = {s.p, s.p_out, s.g, s.g_out, s.m, s.v};
+  for (const void* q : ptrs)
+    if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) d.flags |= kTfUnaligned;
+  d.pad = 0;
+}
+
+int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxopt_table** out) {
+  if (!ctx || !out || (n && !tensors)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: null argument");
+  *out = nullptr;
+  if (n > 0xffffffffull) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: too many tensors");
+  DeviceGuard guard(ctx->device);
+  mxopt_table* t = new (std::nothrow) mxopt_table();
+  if (!t) return fail(ctx, MXOPT_ERR_OOM, "mxopt_table_build: out of host memory");
+  t->ctx = ctx;
+  t->host.assign(tensors, tensors + n);
+  t->dev.resize(n);
+  t->have_mask = 0x3f;
+  std::map<uint32_t, std::vector<uint32_t>> by_key;  // dtype key -> tensor indices, in table order
+  for (size_t i = 0; i < n; ++i) {
+    const mxopt_tensor& s = t->host[i];
+    auto used_ok = [&](const void* ptr, int dt) { return ptr == nullptr || float_dtype(dt); };
+    if (!used_ok(s.p, s.p_dtype) || !used_ok(s.p_out, s.p_out_dtype) || !used_ok(s.g, s.g_dtype) ||
+        !used_ok(s.g_out, s.g_out_dtype)) {
+      delete t;
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  "mxopt_table_build: tensor " + std::to_string(i) + " has a non-floating dtype code");
+    }
+    if (s.n > (uint64_t)0xffffffffu * kChunkElems) {
+      delete t;
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: tensor " + std::to_string(i) + " is too large");
+    }
+    fill_dev_tensor(s, t->dev[i]);
+    if (s.n == 0) continue;  // legal, skipped
+    uint32_t have = (s.p ? kNeedP : 0) | (s.p_out ? kNeedPOut : 0) | (s.g ? kNeedG : 0) | (s.g_out ? kNeedGOut : 0) |
+                    (s.m ? kNeedM : 0) | (s.v ? kNeedV : 0);
+    t->have_mask &= have;
+    t->total_elems += s.n;
+    // Unused streams must not split groups: their dtype byte is normalised to 0.
+    uint32_t key = ((s.p ? s.p_dtype : 0u) << 24) | ((s.g ? s.g_dtype : 0u) << 16) |
+                   ((s.p_out ? s.p_out_dtype : 0u) << 8) | (s.g_out ? s.g_out_dtype : 0u);
+    by_key[key].push_back((uint32_t)i);
+  }
+  std::vector<DevChunk> chunks;
+  for (auto& kv : by_key) {
+    Group g;
+    g.pd = (kv.first >> 24) & 0xff; g.gd = (kv.first >> 16) & 0xff; g.pod = (kv.first >> 8) & 0xff; g.god = kv.first & 0xff;
+    g.chunk_begin = (uint32_t)chunks.size();
+    for (uint32_t ti : kv.second) {
+      const uint64_t nc = (t->host[ti].n + kChunkElems - 1) / kChunkElems;
+      for (uint64_t c = 0; c < nc; ++c) chunks.push_back(DevChunk{ti, (uint32_t)c});
+    }
+    if (chunks.size() > 0xffffffffull) {
+      delete t;
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: too many chunks");
+    }
+    g.nchunks = (uint32_t)chunks.size() - g.chunk_begin;
+    t->groups.push_back(g);
+  }
+  t->num_chunks = chunks.size();
+  hipError_t e = hipSuccess;
+  if (n) e = hipMalloc((void**)&t->d_tensors, n * sizeof(DevTensor));
+  if (e == hipSuccess && !chunks.empty()) e = hipMalloc((void**)&t->d_chunks, chunks.size() * sizeof(DevChunk));
+  if (e == hipSuccess && n)
+    e = hipMemcpyAsync(t->d_tensors, t->dev.data(), n * sizeof(DevTensor), hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess && !chunks.empty())
+    e = hipMemcpyAsync(t->d_chunks, chunks.data(), chunks.size() * sizeof(DevChunk), hipMemcpyHostToDevice, ctx->stream);
+  // `chunks` is a local: the copy must have left host memory before it goes away.
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) {
+    if (t->d_tensors) (void)hipFree(t->d_tensors);
+    if (t->d_chunks) (void)hipFree(t->d_chunks);
+    delete t;
+    return hip_fail(ctx, e, "mxopt_table_build");
+  }
+  *out = t;
+  return MXOPT_OK;
+}
+
+int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* bc2, const uint32_t* flags) {
+  if (!t) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_set_step_scalars: null table");
+  mxopt_ctx* ctx = t->ctx;
+  DeviceGuard guard(ctx->device);
+  const size_t n = t->host.size();
+  for (size_t i = 0; i < n; ++i) {
+    if (bc1) t->host[i].bc1 = bc1[i];
+    if (bc2) t->host[i].bc2 = bc2[i];
+    if (flags) t->host[i].flags = flags[i];
+    fill_dev_tensor(t->host[i], t->dev[i]);
+  }
+  if (n) {
+    // t->dev is rewritten by the next call: wait until the copy has read it.
+    HIP_TRY(ctx, hipMemcpyAsync(t->d_tensors, t->dev.data(), n * sizeof(DevTensor), hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  }
+  return MXOPT_OK;
+}
+
+void mxopt_table_destroy(mxopt_table* t) {
+  if (!t) return;
+  DeviceGuard guard(t->ctx->device);
+  (void)hipStreamSynchronize(t->ctx->stream);
+  if (t->d_tensors) (void)hipFree(t->d_tensors);
+  if (t->d_chunks) (void)hipFree(t->d_chunks);
+  delete t;
+}
+
+uint64_t mxopt_table_total_elems(const mxopt_table* t) { return t ? t->total_elems : 0; }
+uint64_t mxopt_table_num_chunks(const mxopt_table* t) { return t ? t->num_chunks : 0; }
+uint64_t mxopt_table_num_tensors(const mxopt_table* t) { return t ? t->host.size() : 0; }
+
+// ---- hyper-parameter helpers: float64 on the host, then one cast (mlx.cpp:531-535) --------
+
+void mxopt_adam_hp_from_f64(double lr, double beta1, double beta2, double eps, double weight_decay,
+                            int decoupled_decay, mxopt_adam_hp* out) {
+  out->lr = (float)lr;
+  out->beta1 = (float)beta1;
+  out->beta2 = (float)beta2;
+  out->one_minus_beta1 = (float)(1.0 - beta1);
+  out->one_minus_beta2 = (float)(1.0 - beta2);
+  out->eps = (float)eps;
+  out->decay = decoupled_decay ? (float)(1.0 - lr * weight_decay) : 1.0f;
+  out->decoupled_decay = decoupled_decay ? 1 : 0;
+}
+
+void mxopt_bias_correction(double beta1, double beta2, int64_t t, float* bc1, float* bc2) {
+  const double step = (double)t;
+  if (bc1) *bc1 = (float)(1.0 / (1.0 - std::pow(beta1, step)));
+  if (bc2) *bc2 = (float)(1.0 / (1.0 - std::pow(beta2, step)));
+}
+
+int mxopt_sgd_hp_from_f64(double lr, double momentum, double weight_decay, double dampening, int nesterov,
+                          mxopt_sgd_hp* out) {
+  if (nesterov && (momentum <= 0.0 || dampening != 0.0))
+    return fail(nullptr, MXOPT_ERR_INVALID_ARG, "Nesterov momentum requires momentum > 0 and dampening = 0");
+  out->lr = (float)lr;
+  out->momentum = (float)momentum;
+  out->one_minus_dampening = (float)(1.0 - dampening);
+  out->weight_decay = (float)weight_decay;
+  out->has_weight_decay = weight_decay != 0.0;
+  out->has_momentum = momentum != 0.0;
+  out->nesterov = nesterov ? 1 : 0;
+  return MXOPT_OK;
+}
+
+void mxopt_rmsprop_hp_from_f64(double lr, double alpha, double eps, double weight_decay, mxopt_rmsprop_hp* out) {
+  out->lr = (float)lr;
+  out->alpha = (float)alpha;
+  out->one_minus_alpha = (float)(1.0 - alpha);
+  out->eps = (float)eps;
+  out->weight_decay = (float)weight_decay;
+  out->has_weight_decay = weight_decay != 0.0;
+}
+
+// ---- kernels ----------------------------------------------------------------------------
+
+int mxopt_adam(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp, const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedM | kNeedV, "mxopt_adam");
+  if (rc) return rc;
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_adam: hp is NULL");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_adam",
+                    [&](const Group& g, const Launch& L) { return launch_adam(g.pd, g.gd, g.pod, L, *hp, dp); });
+}
+
+int mxopt_sgd(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp, const mxopt_grad_prep* prep) {
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_sgd: hp is NULL");
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | (hp->has_momentum ? kNeedV : 0), "mxopt_sgd");
+  if (rc) return rc;
+  if (hp->nesterov && !hp->has_momentum)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "Nesterov momentum requires momentum > 0 and dampening = 0");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_sgd",
+                    [&](const Group& g, const Launch& L) { return launch_sgd(g.pd, g.gd, g.pod, L, *hp, dp); });
+}
+
+int mxopt_rmsprop(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* hp, const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedV, "mxopt_rmsprop");
+  if (rc) return rc;
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_rmsprop: hp is NULL");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_rmsprop",
+                    [&](const Group& g, const Launch& L) { return launch_rmsprop(g.pd, g.gd, g.pod, L, *hp, dp); });
+}
+
+int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
+                    const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG, "mxopt_sgd_plain");
+  if (rc) return rc;
+  const DevPrep dp = make_prep(prep);
+  const int has_wd = weight_decay > 0.0;  // sft/engine.rs:345
+  const bool promoted = has_wd || prep_active(prep);
+  const float lr32 = (float)learning_rate;
+  const float wd32 = (float)weight_decay;
+  return run_update(ctx, t, "mxopt_sgd_plain", [&](const Group& g, const Launch& L) {
+    // astype(lr, dtype(p)) (model.rs:2437)
+    return launch_sgd_plain(g.pd, g.gd, g.pod, L, round_to_dtype(lr32, g.pd), wd32, has_wd, promoted, dp);
+  });
+}
+
+int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_grad_transform");
+  if (rc) return rc;
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_grad_transform",
+                    [&](const Group& g, const Launch& L) { return launch_transform(g.gd, g.god, L, dp); });
+}
+
+int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep, double max_norm,
+                      int clip_mode, mxopt_norm_result* d_result) {
+  if (which != 0 && which != 1) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm: which must be 0 or 1");
+  int rc = require(ctx, t, which == 0 ? kNeedG : kNeedGOut, "mxopt_global_norm");
+  if (rc) return rc;
+  if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm: d_result is NULL");
+  return run_sumsq(ctx, t, which, 0, prep, max_norm, clip_mode, d_result, "mxopt_global_norm");
+}
+
+int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep, double max_norm,
+                     int clip_mode, mxopt_norm_result* d_result) {
+  int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_accumulate");
+  if (rc) return rc;
+  return run_sumsq(ctx, t, 2, first ? 1 : 0, prep, max_norm, clip_mode, d_result, "mxopt_accumulate");
+}
+
+int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out) {
+  if (!ctx || !d_result || !host_out) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_read_norm_result: null argument");
+  DeviceGuard guard(ctx->device);
+  HIP_TRY(ctx, hipMemcpyAsync(host_out, d_result, sizeof(*host_out), hipMemcpyDeviceToHost, ctx->stream));
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  return MXOPT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,208 @@
+// Device-side building blocks of the mxopt kernels (gfx950 only).
+//
+// Layout in HBM: every tensor is a dense buffer owned by the caller.  The table holds one
+// DevTensor per tensor and one DevChunk per kChunk-element slice of a tensor; a workgroup
+// of 256 lanes (4 wavefronts of 64) takes one chunk at a time.  Inside a chunk, lane L of
+// pass j owns the E contiguous elements starting at (j*256 + L)*E, so one wavefront-wide
+// load instruction covers 64 consecutive 16-byte pieces of a stream.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxopt.h"
+#include "mxopt_host_types.h"
+
+namespace mxopt {
+
+constexpr int kThreads = 256;
+constexpr int kChunk = kChunkElems;
+constexpr int kElemsPerLane = kChunk / kThreads;  // 16
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---- element conversions ----------------------------------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// Round-to-nearest-even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  uint32_t q = (u >> 16) | 0x40u;
+  return ((u & 0x7fffffffu) > 0x7f800000u) ? q : r;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);  // v_cvt_f16_f32: RNE
+}
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<MXOPT_F32> {
+  using T = float;
+  static constexpr int kBytes = 4;
+  static __device__ __forceinline__ float load(const void* base, uint64_t i) { return ((const float*)base)[i]; }
+  static __device__ __forceinline__ void store(void* base, uint64_t i, float x) { ((float*)base)[i] = x; }
+  static __device__ __forceinline__ float round(float x) { return x; }
+};
+template <>
+struct Elem<MXOPT_BF16> {
+  using T = uint16_t;
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float unpack(uint32_t b) { return bf16_bits_to_f32(b); }
+  static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_bf16_bits(x); }
+  static __device__ __forceinline__ float load(const void* base, uint64_t i) {
+    return unpack(((const uint16_t*)base)[i]);
+  }
+  static __device__ __forceinline__ void store(void* base, uint64_t i, float x) {
+    ((uint16_t*)base)[i] = (uint16_t)pack(x);
+  }
+  static __device__ __forceinline__ float round(float x) { return unpack(pack(x)); }
+};
+template <>
+struct Elem<MXOPT_F16> {
+  using T = uint16_t;
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ float unpack(uint32_t b) { return f16_bits_to_f32(b); }
+  static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_f16_bits(x); }
+  static __device__ __forceinline__ float load(const void* base, uint64_t i) {
+    return unpack(((const uint16_t*)base)[i]);
+  }
+  static __device__ __forceinline__ void store(void* base, uint64_t i, float x) {
+    ((uint16_t*)base)[i] = (uint16_t)pack(x);
+  }
+  static __device__ __forceinline__ float round(float x) { return unpack(pack(x)); }
+};
+
+// ---- E-element group loads / stores (E = 4 or 8), 128-bit where the type allows -----
+// `off` is an element offset whose byte offset is 16-byte aligned (8-byte for E=4 x 16-bit).
+
+template <int DT, int E, bool NT>
+__device__ __forceinline__ void load_group(const void* base, uint64_t off, float (&x)[E]) {
+  if constexpr (DT == MXOPT_F32) {
+    const f32x4* q = (const f32x4*)((const float*)base + off);
+#pragma unroll
+    for (int k = 0; k < E / 4; ++k) {
+      f32x4 t = NT ? __builtin_nontemporal_load(q + k) : q[k];
+      x[4 * k + 0] = t.x; x[4 * k + 1] = t.y; x[4 * k + 2] = t.z; x[4 * k + 3] = t.w;
+    }
+  } else if constexpr (E == 8) {
+    const u32x4* q = (const u32x4*)((const uint16_t*)base + off);
+    u32x4 t = NT ? __builtin_nontemporal_load(q) : *q;
+    uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[2 * k + 0] = Elem<DT>::unpack(w[k] & 0xffffu);
+      x[2 * k + 1] = Elem<DT>::unpack(w[k] >> 16);
+    }
+  } else {
+    const u32x2* q = (const u32x2*)((const uint16_t*)base + off);
+    u32x2 t = NT ? __builtin_nontemporal_load(q) : *q;
+    x[0] = Elem<DT>::unpack(t.x & 0xffffu); x[1] = Elem<DT>::unpack(t.x >> 16);
+    x[2] = Elem<DT>::unpack(t.y & 0xffffu); x[3] = Elem<DT>::unpack(t.y >> 16);
+  }
+}
+
+template <int DT, int E, bool NT>
+__device__ __forceinline__ void store_group(void* base, uint64_t off, const float (&x)[E]) {
+  if constexpr (DT == MXOPT_F32) {
+    f32x4* q = (f32x4*)((float*)base + off);
+#pragma unroll
+    for (int k = 0; k < E / 4; ++k) {
+      f32x4 t = {x[4 * k + 0], x[4 * k + 1], x[4 * k + 2], x[4 * k + 3]};
+      if (NT) __builtin_nontemporal_store(t, q + k); else q[k] = t;
+    }
+  } else if constexpr (E == 8) {
+    u32x4 t;
+    t.x = Elem<DT>::pack(x[0]) | (Elem<DT>::pack(x[1]) << 16);
+    t.y = Elem<DT>::pack(x[2]) | (Elem<DT>::pack(x[3]) << 16);
+    t.z = Elem<DT>::pack(x[4]) | (Elem<DT>::pack(x[5]) << 16);
+    t.w = Elem<DT>::pack(x[6]) | (Elem<DT>::pack(x[7]) << 16);
+    u32x4* q = (u32x4*)((uint16_t*)base + off);
+    if (NT) __builtin_nontemporal_store(t, q); else *q = t;
+  } else {
+    u32x2 t;
+    t.x = Elem<DT>::pack(x[0]) | (Elem<DT>::pack(x[1]) << 16);
+    t.y = Elem<DT>::pack(x[2]) | (Elem<DT>::pack(x[3]) << 16);
+    u32x2* q = (u32x2*)((uint16_t*)base + off);
+    if (NT) __builtin_nontemporal_store(t, q); else *q = t;
+  }
+}
+
+// ---- gradient pre-processing (one float32 op per reference op) ----------------------
+
+__device__ __forceinline__ float clamp_keep_nan(float g, float lo, float hi) {
+  float c = fminf(fmaxf(g, lo), hi);
+  return (g != g) ? g : c;
+}
+
+struct PrepRegs {  // block-uniform copy of DevPrep with the device scalar already loaded
+  float pre_mul, pre_lo, pre_hi, scale, post_lo, post_hi;
+  uint32_t flags;
+  bool has_scale;
+};
+
+__device__ __forceinline__ PrepRegs load_prep(const DevPrep& p) {
+  PrepRegs r;
+  r.pre_mul = p.pre_mul; r.pre_lo = p.pre_lo; r.pre_hi = p.pre_hi;
+  r.post_lo = p.post_lo; r.post_hi = p.post_hi; r.flags = p.flags;
+  r.has_scale = p.d_scale != nullptr;
+  r.scale = r.has_scale ? *p.d_scale : 1.0f;
+  return r;
+}
+
+// Stages before the norm is taken.
+__device__ __forceinline__ float prep_pre(const PrepRegs& r, float g) {
+  if (r.flags & kPrepPreMul) g = g * r.pre_mul;
+  if (r.flags & kPrepClampPre) g = clamp_keep_nan(g, r.pre_lo, r.pre_hi);
+  return g;
+}
+__device__ __forceinline__ float prep_all(const PrepRegs& r, float g) {
+  g = prep_pre(r, g);
+  if (r.has_scale) g = g * r.scale;
+  if (r.flags & kPrepClampPost) g = clamp_keep_nan(g, r.post_lo, r.post_hi);
+  return g;
+}
+
+// ---- block reduction: wavefront shuffle -> LDS -> lane 0 ---------------------------
+
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, 64);
+  return x;
+}
+__device__ __forceinline__ unsigned long long wave_sum(unsigned long long x) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, 64);
+  return x;
+}
+
+// Valid on thread 0 only.  Fixed order => deterministic.
+__device__ __forceinline__ void block_sum(double& s, unsigned long long& c) {
+  __shared__ double sh_s[kThreads / 64];
+  __shared__ unsigned long long sh_c[kThreads / 64];
+  s = wave_sum(s);
+  c = wave_sum(c);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { sh_s[wave] = s; sh_c[wave] = c; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    s = sh_s[0]; c = sh_c[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) { s += sh_s[w]; c += sh_c[w]; }
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ bool is_nonfinite(float x) {
+  return (__float_as_uint(x) & 0x7f800000u) == 0x7f800000u;
+}
+
+}  // namespace mxopt

@@ -1,0 +1,77 @@
+// Plain structs shared by the host API and the kernels: the device-side table layout and
+// the opaque handle types behind the C ABI.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "mxopt.h"
+
+namespace mxopt {
+
+constexpr int kChunkElems = MXOPT_CHUNK_ELEMS;
+constexpr uint32_t kTfFirst = MXOPT_TF_FIRST;
+constexpr uint32_t kTfUnaligned = 0x80000000u;  // set by the table builder: element-wise path
+
+// One per tensor, in device memory.
+struct DevTensor {
+  const void* p;
+  void* p_out;
+  const void* g;
+  void* g_out;
+  float* m;
+  float* v;
+  uint64_t n;
+  float bc1, bc2;
+  uint32_t flags;
+  uint32_t pad;
+};
+
+// One per kChunkElems-element slice of a tensor, in device memory.
+struct DevChunk {
+  uint32_t tensor;  // index into the DevTensor array
+  uint32_t index;   // chunk number inside that tensor; first element = index * kChunkElems
+};
+
+constexpr uint32_t kPrepPreMul = 1u, kPrepClampPre = 2u, kPrepClampPost = 4u;
+struct DevPrep {  // kernel argument
+  const float* d_scale;
+  float pre_mul, pre_lo, pre_hi, post_lo, post_hi;
+  uint32_t flags;
+};
+
+// Tensors of one dtype combination: a contiguous run of chunk entries, one launch.
+struct Group {
+  int pd, gd, pod, god;
+  uint32_t chunk_begin, nchunks;
+};
+
+}  // namespace mxopt
+
+struct mxopt_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  int num_cus = 0;
+  int grid_blocks_per_cu = 8;
+  int persistent = 1;
+  int nontemporal = 1;
+  double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
+  unsigned long long* d_partial_cnt = nullptr;
+  size_t partial_cap = 0;
+  std::string err;
+};
+
+struct mxopt_table {
+  mxopt_ctx* ctx = nullptr;
+  std::vector<mxopt_tensor> host;             // caller's descriptors (kept for per-step scalar updates)
+  std::vector<mxopt::DevTensor> dev;          // staging copy of the device descriptors
+  std::vector<mxopt::Group> groups;
+  mxopt::DevTensor* d_tensors = nullptr;
+  mxopt::DevChunk* d_chunks = nullptr;
+  uint64_t total_elems = 0;
+  uint64_t num_chunks = 0;
+  uint32_t have_mask = 0;                     // which pointers are non-NULL in every non-empty tensor
+};

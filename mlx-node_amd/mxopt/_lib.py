@@ -1,0 +1,120 @@
+"""ctypes view of include/mxopt.h.  Loading fails loudly when the HIP library has not been
+built: there is no CPU fallback in this package."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(HERE), "libmxopt.so")
+
+F32, I32, F16, BF16, U32 = 0, 1, 2, 3, 4
+OK, ERR_INVALID_ARG, ERR_FAILURE, ERR_HIP, ERR_OOM = 0, 1, 2, 3, 4
+TF_FIRST = 0x1
+CLIP_ALWAYS_MULTIPLY, CLIP_IF_ABOVE = 0, 1
+CHUNK_ELEMS = 4096
+
+
+class MxoptError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"mxopt error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class InvalidArg(MxoptError, ValueError):
+    """napi Status::InvalidArg."""
+
+
+class Tensor(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("p_out", C.c_void_p), ("g", C.c_void_p), ("g_out", C.c_void_p),
+                ("m", C.c_void_p), ("v", C.c_void_p), ("n", C.c_uint64),
+                ("p_dtype", C.c_uint8), ("p_out_dtype", C.c_uint8), ("g_dtype", C.c_uint8), ("g_out_dtype", C.c_uint8),
+                ("flags", C.c_uint32), ("bc1", C.c_float), ("bc2", C.c_float)]
+
+
+class NormResult(C.Structure):
+    _fields_ = [("sumsq", C.c_double), ("norm", C.c_double), ("norm_f32", C.c_float), ("scale", C.c_float),
+                ("nonfinite", C.c_uint64)]
+
+
+class GradPrep(C.Structure):
+    _fields_ = [("has_pre_mul", C.c_int), ("pre_mul", C.c_float),
+                ("has_clamp_pre", C.c_int), ("pre_lo", C.c_float), ("pre_hi", C.c_float),
+                ("d_scale", C.c_void_p),
+                ("has_clamp_post", C.c_int), ("post_lo", C.c_float), ("post_hi", C.c_float)]
+
+
+class AdamHp(C.Structure):
+    _fields_ = [("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("one_minus_beta1", C.c_float),
+                ("one_minus_beta2", C.c_float), ("eps", C.c_float), ("decay", C.c_float),
+                ("decoupled_decay", C.c_int)]
+
+
+class SgdHp(C.Structure):
+    _fields_ = [("lr", C.c_float), ("momentum", C.c_float), ("one_minus_dampening", C.c_float),
+                ("weight_decay", C.c_float), ("has_weight_decay", C.c_int), ("has_momentum", C.c_int),
+                ("nesterov", C.c_int)]
+
+
+class RmspropHp(C.Structure):
+    _fields_ = [("lr", C.c_float), ("alpha", C.c_float), ("one_minus_alpha", C.c_float), ("eps", C.c_float),
+                ("weight_decay", C.c_float), ("has_weight_decay", C.c_int)]
+
+
+# name -> (restype, argtypes); every symbol declared in include/mxopt.h
+SIGNATURES = {
+    "mxopt_create": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "mxopt_destroy": (None, [C.c_void_p]),
+    "mxopt_last_error": (C.c_char_p, [C.c_void_p]),
+    "mxopt_synchronize": (C.c_int, [C.c_void_p]),
+    "mxopt_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int64]),
+    "mxopt_get_option": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64)]),
+    "mxopt_table_build": (C.c_int, [C.c_void_p, C.POINTER(Tensor), C.c_size_t, C.POINTER(C.c_void_p)]),
+    "mxopt_table_set_step_scalars": (C.c_int, [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                               C.POINTER(C.c_uint32)]),
+    "mxopt_table_destroy": (None, [C.c_void_p]),
+    "mxopt_table_total_elems": (C.c_uint64, [C.c_void_p]),
+    "mxopt_table_num_chunks": (C.c_uint64, [C.c_void_p]),
+    "mxopt_table_num_tensors": (C.c_uint64, [C.c_void_p]),
+    "mxopt_adam_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int,
+                                      C.POINTER(AdamHp)]),
+    "mxopt_bias_correction": (None, [C.c_double, C.c_double, C.c_int64, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "mxopt_sgd_hp_from_f64": (C.c_int, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_int, C.POINTER(SgdHp)]),
+    "mxopt_rmsprop_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.POINTER(RmspropHp)]),
+    "mxopt_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
+    "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),
+    "mxopt_sgd_plain": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double, C.POINTER(GradPrep)]),
+    "mxopt_global_norm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                    C.c_void_p]),
+    "mxopt_grad_transform": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep)]),
+    "mxopt_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                   C.c_void_p]),
+    "mxopt_read_norm_result": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(NormResult)]),
+    "mxopt_version": (C.c_char_p, []),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: build it with `python mlx-node_amd/build.py` "
+                              "(there is no CPU fallback)")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, ctx=None) -> None:
+    if rc == OK:
+        return
+    msg = load().mxopt_last_error(ctx).decode("utf-8", "replace")
+    raise (InvalidArg if rc == ERR_INVALID_ARG else MxoptError)(rc, msg)

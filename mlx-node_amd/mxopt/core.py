@@ -1,0 +1,245 @@
+"""Thin object wrappers over the C ABI for callers that hold torch tensors.
+
+torch is used for device memory and streams only; every computation goes through
+libmxopt.so.  Tensors handed to a Table must stay alive (and keep their storage) for as
+long as the table is used: the table stores raw device pointers.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib as L
+
+_DTYPES = {torch.float32: L.F32, torch.float16: L.F16, torch.bfloat16: L.BF16}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise L.InvalidArg(L.ERR_INVALID_ARG, f"unsupported dtype {t.dtype}") from None
+
+
+def _dev_ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise L.InvalidArg(L.ERR_INVALID_ARG, "mxopt needs device tensors (no CPU path exists)")
+    if not t.is_contiguous():
+        raise L.InvalidArg(L.ERR_INVALID_ARG, "mxopt needs dense (contiguous) buffers")
+    return t.data_ptr() if t.numel() else None
+
+
+@dataclass
+class TensorSpec:
+    """One row of a table, as torch tensors (any may be None when the kernel does not use it)."""
+    p: Optional[torch.Tensor] = None
+    p_out: Optional[torch.Tensor] = None
+    g: Optional[torch.Tensor] = None
+    g_out: Optional[torch.Tensor] = None
+    m: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    bc1: float = 1.0
+    bc2: float = 1.0
+    flags: int = 0
+
+    def numel(self) -> int:
+        ns = {t.numel() for t in (self.p, self.p_out, self.g, self.g_out, self.m, self.v) if t is not None}
+        if len(ns) != 1:
+            raise L.InvalidArg(L.ERR_INVALID_ARG, f"tensors of one table row differ in size: {sorted(ns)}")
+        return ns.pop()
+
+    def to_c(self) -> L.Tensor:
+        for name in ("m", "v"):
+            t = getattr(self, name)
+            if t is not None and t.dtype != torch.float32:
+                raise L.InvalidArg(L.ERR_INVALID_ARG, f"{name} must be float32")
+        c = L.Tensor()
+        c.p, c.p_out, c.g, c.g_out = _dev_ptr(self.p), _dev_ptr(self.p_out), _dev_ptr(self.g), _dev_ptr(self.g_out)
+        c.m, c.v = _dev_ptr(self.m), _dev_ptr(self.v)
+        c.n = self.numel()
+        c.p_dtype = dtype_code(self.p) if self.p is not None else 0
+        c.p_out_dtype = dtype_code(self.p_out) if self.p_out is not None else 0
+        c.g_dtype = dtype_code(self.g) if self.g is not None else 0
+        c.g_out_dtype = dtype_code(self.g_out) if self.g_out is not None else 0
+        c.flags, c.bc1, c.bc2 = self.flags, self.bc1, self.bc2
+        return c
+
+
+def make_prep(pre_mul: Optional[float] = None, clamp_pre: Optional[Sequence[float]] = None,
+              scale: Optional["NormResultBuffer"] = None, clamp_post: Optional[Sequence[float]] = None
+              ) -> Optional[L.GradPrep]:
+    if pre_mul is None and clamp_pre is None and scale is None and clamp_post is None:
+        return None
+    p = L.GradPrep()
+    if pre_mul is not None:
+        p.has_pre_mul, p.pre_mul = 1, pre_mul
+    if clamp_pre is not None:
+        p.has_clamp_pre, p.pre_lo, p.pre_hi = 1, clamp_pre[0], clamp_pre[1]
+    if scale is not None:
+        p.d_scale = scale.scale_ptr
+    if clamp_post is not None:
+        p.has_clamp_post, p.post_lo, p.post_hi = 1, clamp_post[0], clamp_post[1]
+    return p
+
+
+class NormResultBuffer:
+    """Device memory for one mxopt_norm_result."""
+
+    def __init__(self, device):
+        self.buf = torch.zeros(C.sizeof(L.NormResult), dtype=torch.uint8, device=device)
+        self.buf[L.NormResult.scale.offset:L.NormResult.scale.offset + 4] = torch.tensor(
+            [0, 0, 0x80, 0x3F], dtype=torch.uint8, device=device)  # scale = 1.0f
+
+    @property
+    def ptr(self) -> int:
+        return self.buf.data_ptr()
+
+    @property
+    def scale_ptr(self) -> int:
+        return self.buf.data_ptr() + L.NormResult.scale.offset
+
+
+class Context:
+    def __init__(self, device: Optional[torch.device] = None, stream: Optional[torch.cuda.Stream] = None):
+        self.lib = L.load()
+        if not torch.cuda.is_available():
+            raise L.MxoptError(L.ERR_FAILURE, "no GPU visible: mxopt has no CPU path")
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self.device = torch.device("cuda", index)
+        # torch's current stream, so that mxopt kernels order with the torch ops that made the inputs
+        self.stream = torch.cuda.current_stream(self.device) if stream is None else stream
+        handle = C.c_void_p()
+        L.check(self.lib.mxopt_create(index, C.c_void_p(self.stream.cuda_stream), C.byref(handle)))
+        self.handle = handle
+
+    def close(self) -> None:
+        if getattr(self, "handle", None):
+            self.lib.mxopt_destroy(self.handle)
+            self.handle = None
+
+    __del__ = close
+
+    def set_option(self, name: str, value: int) -> None:
+        L.check(self.lib.mxopt_set_option(self.handle, name.encode(), value), self.handle)
+
+    def get_option(self, name: str) -> int:
+        v = C.c_int64()
+        L.check(self.lib.mxopt_get_option(self.handle, name.encode(), C.byref(v)), self.handle)
+        return v.value
+
+    def synchronize(self) -> None:
+        L.check(self.lib.mxopt_synchronize(self.handle), self.handle)
+
+    def table(self, rows: Sequence[TensorSpec]) -> "Table":
+        return Table(self, rows)
+
+    def norm_result(self) -> NormResultBuffer:
+        return NormResultBuffer(self.device)
+
+    def read_norm_result(self, buf: NormResultBuffer) -> L.NormResult:
+        out = L.NormResult()
+        L.check(self.lib.mxopt_read_norm_result(self.handle, C.c_void_p(buf.ptr), C.byref(out)), self.handle)
+        return out
+
+    # ---- kernels ----
+    def adam(self, table: "Table", hp: L.AdamHp, prep: Optional[L.GradPrep] = None) -> None:
+        L.check(self.lib.mxopt_adam(self.handle, table.handle, C.byref(hp), C.byref(prep) if prep else None),
+                self.handle)
+
+    def sgd(self, table: "Table", hp: L.SgdHp, prep: Optional[L.GradPrep] = None) -> None:
+        L.check(self.lib.mxopt_sgd(self.handle, table.handle, C.byref(hp), C.byref(prep) if prep else None),
+                self.handle)
+
+    def rmsprop(self, table: "Table", hp: L.RmspropHp, prep: Optional[L.GradPrep] = None) -> None:
+        L.check(self.lib.mxopt_rmsprop(self.handle, table.handle, C.byref(hp), C.byref(prep) if prep else None),
+                self.handle)
+
+    def sgd_plain(self, table: "Table", learning_rate: float, weight_decay: float = 0.0,
+                  prep: Optional[L.GradPrep] = None) -> None:
+        L.check(self.lib.mxopt_sgd_plain(self.handle, table.handle, learning_rate, weight_decay,
+                                         C.byref(prep) if prep else None), self.handle)
+
+    def global_norm(self, table: "Table", out: NormResultBuffer, which: int = 0,
+                    prep: Optional[L.GradPrep] = None, max_norm: float = -1.0,
+                    clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
+        L.check(self.lib.mxopt_global_norm(self.handle, table.handle, which, C.byref(prep) if prep else None,
+                                           max_norm, clip_mode, C.c_void_p(out.ptr)), self.handle)
+
+    def grad_transform(self, table: "Table", prep: Optional[L.GradPrep]) -> None:
+        L.check(self.lib.mxopt_grad_transform(self.handle, table.handle, C.byref(prep) if prep else None),
+                self.handle)
+
+    def accumulate(self, table: "Table", first: bool, out: Optional[NormResultBuffer] = None,
+                   prep: Optional[L.GradPrep] = None, max_norm: float = -1.0,
+                   clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
+        L.check(self.lib.mxopt_accumulate(self.handle, table.handle, int(first), C.byref(prep) if prep else None,
+                                          max_norm, clip_mode, C.c_void_p(out.ptr) if out else None), self.handle)
+
+
+class Table:
+    def __init__(self, ctx: Context, rows: Sequence[TensorSpec]):
+        self.ctx = ctx
+        self.rows: List[TensorSpec] = list(rows)   # keeps the tensors alive
+        n = len(self.rows)
+        arr = (L.Tensor * max(n, 1))()
+        for i, r in enumerate(self.rows):
+            arr[i] = r.to_c()
+        handle = C.c_void_p()
+        L.check(ctx.lib.mxopt_table_build(ctx.handle, arr, n, C.byref(handle)), ctx.handle)
+        self.handle = handle
+
+    def close(self) -> None:
+        if getattr(self, "handle", None) and getattr(self.ctx, "handle", None):
+            self.ctx.lib.mxopt_table_destroy(self.handle)
+        self.handle = None
+
+    __del__ = close
+
+    @property
+    def total_elems(self) -> int:
+        return self.ctx.lib.mxopt_table_total_elems(self.handle)
+
+    @property
+    def num_chunks(self) -> int:
+        return self.ctx.lib.mxopt_table_num_chunks(self.handle)
+
+    def set_step_scalars(self, bc1: Optional[Sequence[float]] = None, bc2: Optional[Sequence[float]] = None,
+                         flags: Optional[Sequence[int]] = None) -> None:
+        n = len(self.rows)
+        a = (C.c_float * n)(*bc1) if bc1 is not None else None
+        b = (C.c_float * n)(*bc2) if bc2 is not None else None
+        f = (C.c_uint32 * n)(*flags) if flags is not None else None
+        L.check(self.ctx.lib.mxopt_table_set_step_scalars(self.handle, a, b, f), self.ctx.handle)
+
+
+def adam_hp(lr: float, beta1: float, beta2: float, eps: float, weight_decay: Optional[float] = None) -> L.AdamHp:
+    """weight_decay None = Adam, a number = AdamW."""
+    hp = L.AdamHp()
+    L.load().mxopt_adam_hp_from_f64(lr, beta1, beta2, eps, 0.0 if weight_decay is None else weight_decay,
+                                    int(weight_decay is not None), C.byref(hp))
+    return hp
+
+
+def bias_correction(beta1: float, beta2: float, t: int):
+    a, b = C.c_float(), C.c_float()
+    L.load().mxopt_bias_correction(beta1, beta2, t, C.byref(a), C.byref(b))
+    return a.value, b.value
+
+
+def sgd_hp(lr: float, momentum: float = 0.0, weight_decay: float = 0.0, dampening: float = 0.0,
+           nesterov: bool = False) -> L.SgdHp:
+    hp = L.SgdHp()
+    L.check(L.load().mxopt_sgd_hp_from_f64(lr, momentum, weight_decay, dampening, int(nesterov), C.byref(hp)))
+    return hp
+
+
+def rmsprop_hp(lr: float, alpha: float, eps: float, weight_decay: float = 0.0) -> L.RmspropHp:
+    hp = L.RmspropHp()
+    L.load().mxopt_rmsprop_hp_from_f64(lr, alpha, eps, weight_decay, C.byref(hp))
+    return hp
