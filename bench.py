@@ -1,0 +1,363 @@
+#!/usr/bin/env python3
+"""Benchmark of the optimizer-step hot path on one MI355X.
+
+Default workload (the one the headline metric is quoted on): Qwen3-8B-shaped training step --
+4 micro-batch bf16 gradients accumulated into a float32 buffer, global-norm clip at 1.0 (sum of
+squares fused into the last accumulation pass), AdamW with bf16 parameters updated in place and
+float32 moments; everything resident in HBM (~131 GB + 3 more micro-gradient buffers).
+
+Prints ONE JSON line.  `value` = optimizer steps/s over the timed region (inputs resident
+before it starts).  `roofline` describes the dominant kernel (the AdamW update): algorithmic
+bytes per launch / its average duration measured with events on the launch stream.
+`cpu_baseline` times the CPU restatement of the reference's un-fused op chain (oracle/) on a
+bounded sample of the same workload and scales it to the full parameter list.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg5",
+                    choices=["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat", "cfg5"])
+    ap.add_argument("--cpu-sample", type=int, default=128 * 1024 * 1024,
+                    help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
+    ap.add_argument("--scale", type=float, default=1.0,
+                    help="shrink every tensor's first dimension (for quick runs; invalid as a result)")
+    ap.add_argument("--option", action="append", default=[], help="mxopt option name=value")
+    return ap.parse_args()
+
+
+# ----------------------------------------------------------------------------------------
+# workloads
+# ----------------------------------------------------------------------------------------
+
+def tensor_sizes(args):
+    from mxopt.qwen3_shapes import QWEN3, numel, param_list
+    model = {"cfg1": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B"}.get(args.workload)
+    if model:
+        sizes = []
+        for _, shape in param_list(QWEN3[model]):
+            if args.scale != 1.0 and len(shape) == 2:
+                shape = (max(1, int(shape[0] * args.scale)), shape[1])
+            sizes.append(numel(shape))
+        return sizes, f"qwen3-{model.lower()}"
+    import numpy as np
+    rng = np.random.default_rng(0x5EED0001)
+    sizes = np.floor(np.exp(rng.uniform(np.log(64), np.log(65536), 10000))).astype(np.int64).tolist()
+    if args.workload == "cfg4-flat":
+        return [int(sum(sizes))], "one-flat-tensor-of-cfg4-size"
+    return sizes, "10000-small-tensors"
+
+
+class Workload:
+    """Holds device buffers + tables and knows how to run one step and what it costs."""
+
+    def __init__(self, args, torch, mx):
+        self.args, self.torch, self.mx = args, torch, mx
+        self.ctx = mx.Context()
+        for opt in args.option:
+            k, v = opt.split("=")
+            self.ctx.set_option(k, int(v))
+        self.sizes, self.list_name = tensor_sizes(args)
+        self.n = int(sum(self.sizes))
+        self.kernel_events = {}     # kernel name -> list of (start, end) events
+        self.res = self.ctx.norm_result()
+        getattr(self, "_setup_" + args.workload.replace("-", "_"))()
+        torch.cuda.synchronize()
+
+    # -- helpers
+    def _randn(self, n, dtype, std):
+        return self.torch.empty(n, dtype=dtype, device="cuda").normal_(0.0, std)
+
+    def _zeros(self, n):
+        return self.torch.zeros(n, dtype=self.torch.float32, device="cuda")
+
+    def _timed(self, name, fn):
+        s = self.torch.cuda.Event(enable_timing=True)
+        e = self.torch.cuda.Event(enable_timing=True)
+        s.record(self.ctx.stream)
+        fn()
+        e.record(self.ctx.stream)
+        self.kernel_events.setdefault(name, []).append((s, e))
+
+    def kernel_ms(self, name):
+        ev = self.kernel_events.get(name, [])
+        return [s.elapsed_time(e) for s, e in ev]
+
+    # -- cfg5: 4x accumulate (bf16 -> f32), clip 1.0, AdamW bf16 p / f32 m,v
+    def _setup_cfg5(self):
+        t, mx = self.torch, self.mx
+        bf = t.bfloat16
+        need = self.n * (2 + 8 + 4)
+        free, _ = t.cuda.mem_get_info()
+        self.n_micro = 4
+        n_gbuf = 4 if free > need + 4 * self.n * 2 + (8 << 30) else 1
+        self.p = [self._randn(n, bf, 0.02) for n in self.sizes]
+        self.m = [self._zeros(n) for n in self.sizes]
+        self.v = [self._zeros(n) for n in self.sizes]
+        self.acc = [t.empty(n, dtype=t.float32, device="cuda") for n in self.sizes]
+        self.g = [[self._randn(n, bf, 1e-3) for n in self.sizes] for _ in range(n_gbuf)]
+        self.t_acc = [self.ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(gk, self.acc)]) for gk in self.g]
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, m=m, v=v)
+                                     for p, a, m, v in zip(self.p, self.acc, self.m, self.v)])
+        self.hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
+        self.prep = mx.make_prep(scale=self.res)
+        self.dtype = "bf16 params/grads, f32 accumulate + moments + arithmetic"
+        self.bytes_per_elem = {"accumulate_first": 6, "accumulate": 10, "accumulate_sumsq": 10, "adamw": 24}
+        self.step_bytes_per_elem = 6 + 10 * 3 + 24
+        self.dominant = "adamw"
+        self.note = f"{n_gbuf} resident micro-gradient buffer(s)"
+
+    def _step_cfg5(self):
+        c = self.ctx
+        for k in range(self.n_micro):
+            tab = self.t_acc[k % len(self.t_acc)]
+            last = k == self.n_micro - 1
+            name = "accumulate_first" if k == 0 else ("accumulate_sumsq" if last else "accumulate")
+            self._timed(name, lambda: c.accumulate(tab, first=(k == 0), out=self.res if last else None,
+                                                   max_norm=1.0))
+        self._timed("adamw", lambda: c.adam(self.t_upd, self.hp, self.prep))
+
+    # -- cfg1: fp32 AdamW
+    def _setup_cfg1(self):
+        t, mx = self.torch, self.mx
+        self.p = [self._randn(n, t.float32, 0.02) for n in self.sizes]
+        self.g = [self._randn(n, t.float32, 1e-3) for n in self.sizes]
+        self.m = [self._zeros(n) for n in self.sizes]
+        self.v = [self._zeros(n) for n in self.sizes]
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
+                                     for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
+        self.hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01)
+        self.dtype = "f32"
+        self.bytes_per_elem = {"adamw": 28}
+        self.step_bytes_per_elem = 28
+        self.dominant = "adamw"
+        self.note = ""
+
+    def _step_cfg1(self):
+        self._timed("adamw", lambda: self.ctx.adam(self.t_upd, self.hp))
+
+    # -- cfg2 / cfg4: bf16 p,g + f32 m,v AdamW with a separate norm pass
+    def _setup_cfg2(self, lr=5e-6, wd=0.01, gstd=1e-3, uniform_p=False):
+        t, mx = self.torch, self.mx
+        bf = t.bfloat16
+        if uniform_p:
+            self.p = [t.empty(n, dtype=bf, device="cuda").uniform_(0.9, 1.1) for n in self.sizes]
+        else:
+            self.p = [self._randn(n, bf, 0.02) for n in self.sizes]
+        self.g = [self._randn(n, bf, gstd) for n in self.sizes]
+        if self.args.workload == "cfg2":   # 1 % of the elements are x100 outliers
+            for g in self.g:
+                g.mul_(t.where(t.rand(g.shape, device="cuda") < 0.01, 100.0, 1.0).to(bf))
+        self.m = [self._zeros(n) for n in self.sizes]
+        self.v = [self._zeros(n) for n in self.sizes]
+        self.t_g = self.ctx.table([mx.TensorSpec(g=g) for g in self.g])
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
+                                     for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
+        self.hp = mx.adam_hp(lr, 0.9, 0.999, 1e-8, wd)
+        self.prep = mx.make_prep(scale=self.res)
+        self.dtype = "bf16 params/grads, f32 moments + arithmetic"
+        self.bytes_per_elem = {"global_norm": 2, "adamw": 22}
+        self.step_bytes_per_elem = 24
+        self.dominant = "adamw"
+        self.note = ""
+
+    def _step_cfg2(self):
+        self._timed("global_norm", lambda: self.ctx.global_norm(self.t_g, self.res, max_norm=1.0))
+        self._timed("adamw", lambda: self.ctx.adam(self.t_upd, self.hp, self.prep))
+
+    def _setup_cfg4(self):
+        self._setup_cfg2(lr=1e-3, wd=0.0, gstd=1e-2, uniform_p=True)
+
+    _step_cfg4 = _step_cfg2
+    _setup_cfg4_flat = _setup_cfg4
+    _step_cfg4_flat = _step_cfg2
+
+    # -- cfg3: fp32 SGD / RMSprop
+    def _setup_cfg3(self):
+        t, mx = self.torch, self.mx
+        self.p = [self._randn(n, t.float32, 0.02) for n in self.sizes]
+        self.g = [self._randn(n, t.float32, 1e-3) for n in self.sizes]
+        self.v = [self._zeros(n) for n in self.sizes]
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v)
+                                     for p, g, v in zip(self.p, self.g, self.v)])
+        self.dtype = "f32"
+        self.step_bytes_per_elem = 20
+        self.note = ""
+
+    def _setup_cfg3_sgd(self):
+        self._setup_cfg3()
+        self.hp = self.mx.sgd_hp(1e-4, 0.9, 1e-4, 0.0, False)
+        self.bytes_per_elem = {"sgd": 20}
+        self.dominant = "sgd"
+
+    def _step_cfg3_sgd(self):
+        self._timed("sgd", lambda: self.ctx.sgd(self.t_upd, self.hp))
+
+    def _setup_cfg3_rmsprop(self):
+        self._setup_cfg3()
+        self.hp = self.mx.rmsprop_hp(1e-4, 0.99, 1e-8, 0.0)
+        self.bytes_per_elem = {"rmsprop": 20}
+        self.dominant = "rmsprop"
+
+    def _step_cfg3_rmsprop(self):
+        self._timed("rmsprop", lambda: self.ctx.rmsprop(self.t_upd, self.hp))
+
+    def step(self):
+        getattr(self, "_step_" + self.args.workload.replace("-", "_"))()
+
+
+# ----------------------------------------------------------------------------------------
+# CPU baseline: the oracle's C twin (un-fused op chain) on a bounded sample
+# ----------------------------------------------------------------------------------------
+
+def cpu_baseline(args, n_total):
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle_c_binding as B
+    oc = B.load()
+    S = int(min(args.cpu_sample, n_total))
+    rng = np.random.default_rng(1)
+    w = args.workload
+    f32 = np.float32
+    p32 = (rng.standard_normal(S, dtype=f32) * f32(0.02))
+    g32 = (rng.standard_normal(S, dtype=f32) * f32(1e-3))
+    m, v = np.zeros(S, f32), np.zeros(S, f32)
+
+    def timeit(fn, reps=2):
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    fused_s = None
+    if w in ("cfg5", "cfg2", "cfg4", "cfg4-flat"):
+        p, g = oc.f32_to_bf16(p32), oc.f32_to_bf16(g32)
+        del p32, g32
+        acc = np.empty(S, f32)
+        lr, wd = (5e-6, 0.01) if w != "cfg4" else (1e-3, 0.0)
+
+        def step(fused):
+            src = g
+            if w == "cfg5":
+                for k in range(4):
+                    oc.accumulate_f32(acc, g, k == 0)
+                src = acc
+            sumsq = oc.sumsq(src)
+            scale = float(min(np.float32(1.0) / (np.float32(np.sqrt(sumsq)) + np.float32(1e-6)), np.float32(1.0)))
+            a = B.adam_args(lr, 0.9, 0.999, 1e-8, wd, scale=scale)
+            out = oc.adam(p, src, m, v, a, fused=fused)
+            oc.f32_to_bf16(out)     # parameters are kept in bf16
+        what = ("4x accumulate + sumsq + scale + AdamW as 13 separate float32 passes (adamw.rs:84-116) + bf16 cast"
+                if w == "cfg5" else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
+        t_unfused = timeit(lambda: step(False))
+        fused_s = timeit(lambda: step(True))
+    elif w == "cfg1":
+        a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01)
+        t_unfused = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=False))
+        fused_s = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=True))
+        what = "AdamW as 13 separate float32 passes (adamw.rs:84-116)"
+    elif w == "cfg3-sgd":
+        fl = lambda x: float(np.float32(x))
+        a = B.SgdArgs(lr=fl(1e-4), momentum=fl(0.9), one_minus_damp=1.0, wd=fl(1e-4), has_wd=1, has_momentum=1,
+                      nesterov=0, first=0)
+        t_unfused = timeit(lambda: oc.sgd(p32, g32, v, a, fused=False))
+        fused_s = timeit(lambda: oc.sgd(p32, g32, v, a, fused=True))
+        what = "SGD+momentum+L2 as 7 separate float32 passes (sgd.rs:86-140)"
+    else:
+        fl = lambda x: float(np.float32(x))
+        a = B.RmspropArgs(lr=fl(1e-4), alpha=fl(0.99), one_minus_alpha=fl(1.0 - 0.99), eps=fl(1e-8), wd=0.0, has_wd=0)
+        t_unfused = timeit(lambda: oc.rmsprop(p32, g32, v, a, fused=False))
+        fused_s = timeit(lambda: oc.rmsprop(p32, g32, v, a, fused=True))
+        what = "RMSprop as 9 separate float32 passes (rmsprop.rs:69-93)"
+
+    scale_up = n_total / S
+    return {
+        "value": 1.0 / (t_unfused * scale_up), "unit": "steps/s", "cores": oc.num_threads(), "kind": "port",
+        "sample": f"{S} of {n_total} elements, one flat tensor, best of 2; {what}; scaled per element "
+                  f"to the full list (sample step {t_unfused * 1e3:.1f} ms)",
+        "fused_single_pass_value": (1.0 / (fused_s * scale_up)) if fused_s else None,
+    }
+
+
+# ----------------------------------------------------------------------------------------
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
+    import torch
+    import mxopt
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X: mxopt has no CPU path")
+    torch.cuda.set_device(0)
+    torch.manual_seed(0x5EED0001)
+
+    wl = Workload(args, torch, mxopt)
+    for _ in range(args.warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    wl.kernel_events.clear()
+
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        wl.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    steps_per_s = args.steps / elapsed
+    n = wl.n
+    step_gbps = wl.step_bytes_per_elem * n / (elapsed / args.steps) / 1e9
+
+    kernels = {}
+    for name, bpe in wl.bytes_per_elem.items():
+        ms = wl.kernel_ms(name)
+        if not ms:
+            continue
+        avg = sum(ms) / len(ms)
+        kernels[name] = {"avg_ms": round(avg, 4), "min_ms": round(min(ms), 4), "launches": len(ms),
+                         "bytes_per_elem": bpe, "gbps": round(bpe * n / (avg * 1e-3) / 1e9, 1)}
+    dom = kernels[wl.dominant]
+    roofline = {"bound": "hbm", "achieved": dom["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(dom["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
+                "avg_launch_ms": dom["avg_ms"]}
+
+    cpu = cpu_baseline(args, n) if args.cpu_sample > 0 else None
+
+    out = {
+        "metric": "optimizer steps/s + achieved HBM GB/s (% of 8 TB/s), AdamW on Qwen3-8B shapes",
+        "value": round(steps_per_s, 4), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": wl.dtype, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
+                   "bytes_per_elem_per_step": wl.step_bytes_per_elem, "note": wl.note, "scale": args.scale},
+        "elements_per_s": round(n * steps_per_s, 1),
+        "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
+        "kernels": kernels,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
