@@ -151,7 +151,7 @@ static Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Grou
   L.nchunks = g.nchunks;
   L.grid = persistent ? persistent_grid(ctx, g.nchunks) : g.nchunks;
   L.stream = ctx->stream;
-  L.nontemporal = ctx->nontemporal != 0;
+  L.nontemporal = ctx->nontemporal & 3;
   return L;
 }
 
@@ -184,7 +184,10 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
   }
   size_t offset = 0;
   for (const Group& g : t->groups) {
-    Launch L = make_launch(ctx, t, g, true);
+    // Reductions need one partial per workgroup, so they keep a bounded grid; so does the
+    // read-modify-write accumulation, which measured faster that way.  Only the first,
+    // write-dominated accumulation pass follows the update kernels' launch policy.
+    Launch L = make_launch(ctx, t, g, want || !(mode == 2 && first) || ctx->persistent != 0);
     const int ad = mode == 0 ? g.gd : g.god;
     if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr,
                       want ? ctx->d_partial_cnt + offset : nullptr))
@@ -266,7 +269,8 @@ int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
   } else if (n == "persistent") {
     ctx->persistent = value != 0;
   } else if (n == "nontemporal") {
-    ctx->nontemporal = value != 0;
+    if (value < 0 || value > 3) return fail(ctx, MXOPT_ERR_INVALID_ARG, "nontemporal must be in [0, 3]");
+    ctx->nontemporal = (int)value;
   } else {
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: unknown option " + n);
   }

@@ -55,9 +55,9 @@ struct mxopt_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   int num_cus = 0;
-  int grid_blocks_per_cu = 8;
-  int persistent = 1;
-  int nontemporal = 1;
+  int grid_blocks_per_cu = 16;  // bounded grids (reductions, accumulation): workgroups per CU
+  int persistent = 0;           // update kernels: 0 = one workgroup per chunk, 1 = bounded grid
+  int nontemporal = 0;          // bit 0: streaming loads, bit 1: streaming stores
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
   unsigned long long* d_partial_cnt = nullptr;
   size_t partial_cap = 0;

@@ -119,7 +119,7 @@ struct PlainSgdMath {
 // Update kernel
 // ------------------------------------------------------------------------------------
 
-template <int PD, int GD, int OD, class Math, bool NT>
+template <int PD, int GD, int OD, class Math, int NT>
 __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __restrict__ T,
                                                           const DevChunk* __restrict__ C, uint32_t nchunks,
                                                           Math math, DevPrep prep) {
@@ -149,10 +149,10 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        load_group<PD, E, NT>(P, off, p[j]);
-        load_group<GD, E, NT>(G, off, g[j]);
-        if (Math::kM) load_group<MXOPT_F32, E, NT>(M, off, m[j]);
-        if (read_v) load_group<MXOPT_F32, E, NT>(V, off, v[j]);
+        load_group<PD, E, (NT & 1) != 0>(P, off, p[j]);
+        load_group<GD, E, (NT & 1) != 0>(G, off, g[j]);
+        if (Math::kM) load_group<MXOPT_F32, E, (NT & 1) != 0>(M, off, m[j]);
+        if (read_v) load_group<MXOPT_F32, E, (NT & 1) != 0>(V, off, v[j]);
       }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
@@ -162,9 +162,9 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        store_group<OD, E, NT>(PO, off, p[j]);
-        if (Math::kM) store_group<MXOPT_F32, E, NT>(M, off, m[j]);
-        if (use_v) store_group<MXOPT_F32, E, NT>(V, off, v[j]);
+        store_group<OD, E, (NT & 2) != 0>(PO, off, p[j]);
+        if (Math::kM) store_group<MXOPT_F32, E, (NT & 2) != 0>(M, off, m[j]);
+        if (use_v) store_group<MXOPT_F32, E, (NT & 2) != 0>(V, off, v[j]);
       }
     } else {
       // Last chunk of a tensor, or a tensor whose buffers are not 16-byte aligned.
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 // Gradient transform: g_out = prep(g)
 // ------------------------------------------------------------------------------------
 
-template <int GD, int OD, bool NT>
+template <int GD, int OD, int NT>
 __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __restrict__ T,
                                                              const DevChunk* __restrict__ C, uint32_t nchunks,
                                                              DevPrep prep) {
@@ -221,12 +221,12 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
     if (!(flags & kTfUnaligned) && len == (uint32_t)kChunk) {
       float g[U][E];
 #pragma unroll
-      for (int j = 0; j < U; ++j) load_group<GD, E, NT>(G, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+      for (int j = 0; j < U; ++j) load_group<GD, E, (NT & 1) != 0>(G, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
 #pragma unroll
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int e = 0; e < E; ++e) g[j][e] = prep_all(pr, g[j][e]);
-        store_group<OD, E, NT>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+        store_group<OD, E, (NT & 2) != 0>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
       }
     } else {
       const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
@@ -257,7 +257,7 @@ __device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
   return Elem<AD>::round(s);
 }
 
-template <int MODE, int AD, int GD, bool NT>
+template <int MODE, int AD, int GD, int NT>
 __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __restrict__ T,
                                                          const DevChunk* __restrict__ C, uint32_t nchunks,
                                                          DevPrep prep, int first, double* __restrict__ partial_sum,
@@ -287,12 +287,12 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        if (MODE != 2 || !first) load_group<AD, E, NT>(X, off, x[j]);
+        if (MODE != 2 || !first) load_group<AD, E, (NT & 1) != 0>(X, off, x[j]);
         else {
 #pragma unroll
           for (int e = 0; e < E; ++e) x[j][e] = 0.0f;
         }
-        if (MODE == 2) load_group<GD, E, NT>(G, off, g[j]);
+        if (MODE == 2) load_group<GD, E, (NT & 1) != 0>(G, off, g[j]);
       }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
           acc_cnt += is_nonfinite(y);
           s32 = s32 + y * y;
         }
-        if (MODE == 2) store_group<AD, E, NT>(A, start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+        if (MODE == 2) store_group<AD, E, (NT & 2) != 0>(A, start + (uint64_t)(j * kThreads + tid) * E, x[j]);
       }
     } else {
       const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
@@ -394,10 +394,12 @@ __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __r
 
 template <int PD, int GD, int OD, class Math>
 static void launch_update_t(const Launch& L, const Math& math, const DevPrep& prep) {
-  if (L.nontemporal)
-    MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, true>), L, math, prep);
-  else
-    MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, false>), L, math, prep);
+  switch (L.nontemporal & 3) {
+    case 0: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 0>), L, math, prep); break;
+    case 1: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 1>), L, math, prep); break;
+    case 2: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 2>), L, math, prep); break;
+    case 3: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 3>), L, math, prep); break;
+  }
 }
 
 template <int PD, int GD, class Math>
@@ -464,13 +466,13 @@ bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float
 template <int GD>
 static bool transform_for_gd(int od, const Launch& L, const DevPrep& prep) {
   if (od == MXOPT_F32) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, true>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, false>), L, prep);
+    if (L.nontemporal & 2) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, 2>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, 0>), L, prep);
     return true;
   }
   if (od == GD) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, GD, true>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, GD, false>), L, prep);
+    if (L.nontemporal & 2) MXOPT_LAUNCH((transform_kernel<GD, GD, 2>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, GD, 0>), L, prep);
     return true;
   }
   return false;
@@ -487,8 +489,12 @@ bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep) {
 
 template <int MODE, int AD, int GD>
 static void launch_sumsq_t(const Launch& L, const DevPrep& prep, int first, double* ps, unsigned long long* pc) {
-  if (L.nontemporal) MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, true>), L, prep, first, ps, pc);
-  else MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, false>), L, prep, first, ps, pc);
+  switch (L.nontemporal & 3) {
+    case 0: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 0>), L, prep, first, ps, pc); break;
+    case 1: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 1>), L, prep, first, ps, pc); break;
+    case 2: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 2>), L, prep, first, ps, pc); break;
+    case 3: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 3>), L, prep, first, ps, pc); break;
+  }
 }
 
 template <int MODE, int AD>

@@ -19,7 +19,7 @@ struct Launch {
   uint32_t nchunks;
   uint32_t grid;           // workgroups (<= nchunks)
   hipStream_t stream;
-  bool nontemporal;
+  int nontemporal;         // bit 0: streaming loads, bit 1: streaming stores
 };
 
 // Each returns false when the dtype combination has no kernel.
