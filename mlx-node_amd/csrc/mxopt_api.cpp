@@ -12,6 +12,7 @@
 
 #include "mxopt.h"
 #include "mxopt_host_types.h"
+#include "mxopt_internal.h"
 #include "mxopt_launch.h"
 
 namespace mxopt {
@@ -29,13 +30,8 @@ int hip_fail(mxopt_ctx* ctx, hipError_t e, const char* what) {
               std::string(what) + ": " + hipGetErrorString(e));
 }
 
-#define HIP_TRY(ctx, call)                                   \
-  do {                                                       \
-    hipError_t e_ = (call);                                  \
-    if (e_ != hipSuccess) return hip_fail((ctx), e_, #call); \
-  } while (0)
 
-static bool float_dtype(int dt) { return dt == MXOPT_F32 || dt == MXOPT_F16 || dt == MXOPT_BF16; }
+bool float_dtype(int dt) { return dt == MXOPT_F32 || dt == MXOPT_F16 || dt == MXOPT_BF16; }
 
 float round_to_dtype(float x, int dt) {
   if (dt == MXOPT_BF16) {
@@ -53,7 +49,7 @@ float round_to_dtype(float x, int dt) {
   return x;
 }
 
-static DevPrep make_prep(const mxopt_grad_prep* p) {
+DevPrep make_prep(const mxopt_grad_prep* p) {
   DevPrep d{};
   d.d_scale = nullptr;
   d.pre_mul = 1.0f;
@@ -77,16 +73,16 @@ static DevPrep make_prep(const mxopt_grad_prep* p) {
   return d;
 }
 
-static bool prep_active(const mxopt_grad_prep* p) {
+bool prep_active(const mxopt_grad_prep* p) {
   return p && (p->has_pre_mul || p->has_clamp_pre || p->d_scale || p->has_clamp_post);
 }
 
-static uint32_t persistent_grid(const mxopt_ctx* ctx, uint32_t nchunks) {
+uint32_t persistent_grid(const mxopt_ctx* ctx, uint32_t nchunks) {
   uint64_t cap = (uint64_t)ctx->num_cus * (uint64_t)ctx->grid_blocks_per_cu;
   return (uint32_t)std::min<uint64_t>(nchunks, std::max<uint64_t>(cap, 1));
 }
 
-static int ensure_partials(mxopt_ctx* ctx, size_t need) {
+int ensure_partials(mxopt_ctx* ctx, size_t need) {
   if (need <= ctx->partial_cap) return MXOPT_OK;
   size_t cap = std::max<size_t>(need, 4096);
   double* ps = nullptr;
@@ -109,20 +105,8 @@ static int ensure_partials(mxopt_ctx* ctx, size_t need) {
   return MXOPT_OK;
 }
 
-struct DeviceGuard {
-  int prev = -1;
-  bool ok = true;
-  explicit DeviceGuard(int dev) {
-    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
-    if (prev != dev) ok = hipSetDevice(dev) == hipSuccess;
-  }
-  ~DeviceGuard() {
-    int cur = -1;
-    if (prev >= 0 && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
-  }
-};
 
-static int check_launch(mxopt_ctx* ctx, const char* what) {
+int check_launch(mxopt_ctx* ctx, const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return hip_fail(ctx, e, what);
   return MXOPT_OK;
@@ -144,7 +128,7 @@ static int require(mxopt_ctx* ctx, const mxopt_table* t, uint32_t need, const ch
   return MXOPT_OK;
 }
 
-static Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Group& g, bool persistent) {
+Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Group& g, bool persistent) {
   Launch L;
   L.tensors = t->d_tensors;
   L.chunks = t->d_chunks + g.chunk_begin;
@@ -155,13 +139,13 @@ static Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Grou
   return L;
 }
 
-static std::string dtype_names(const Group& g) {
+std::string dtype_names(const Group& g) {
   auto nm = [](int d) { return d == MXOPT_F32 ? "f32" : d == MXOPT_BF16 ? "bf16" : d == MXOPT_F16 ? "f16" : "?"; };
   return std::string("p=") + nm(g.pd) + " g=" + nm(g.gd) + " p_out=" + nm(g.pod) + " g_out=" + nm(g.god);
 }
 
 // Second pass shared by mxopt_global_norm and mxopt_accumulate.
-static int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode,
+int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode,
                        mxopt_norm_result* d_result) {
   const int has_max = max_norm >= 0.0;
   launch_norm_finish(ctx->stream, ctx->d_partial_sum, ctx->d_partial_cnt, npartials, max_norm, has_max, clip_mode,
@@ -212,6 +196,26 @@ static int run_update(mxopt_ctx* ctx, const mxopt_table* t, const char* op, F&& 
   return MXOPT_OK;
 }
 
+void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d) {
+  d.p = s.p; d.p_out = s.p_out; d.g = s.g; d.g_out = s.g_out; d.m = s.m; d.v = s.v;
+  d.n = s.n; d.bc1 = s.bc1; d.bc2 = s.bc2;
+  d.flags = s.flags & ~kTfUnaligned;
+  const void* ptrs[6] = {s.p, s.p_out, s.g, s.g_out, s.m, s.v};
+  for (const void* q : ptrs)
+    if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) d.flags |= kTfUnaligned;
+  d.pad = 0;
+}
+
+Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool persistent) {
+  Launch L;
+  fill_dev_tensor(t, L.one);
+  L.nchunks = (uint32_t)((t.n + kChunkElems - 1) / kChunkElems);
+  L.grid = persistent ? persistent_grid(ctx, L.nchunks) : L.nchunks;
+  L.stream = ctx->stream;
+  L.nontemporal = ctx->nontemporal & 3;
+  return L;
+}
+
 }  // namespace mxopt
 
 using namespace mxopt;
@@ -243,6 +247,12 @@ int mxopt_create(int device, void* hip_stream, mxopt_ctx** out) {
 void mxopt_destroy(mxopt_ctx* ctx) {
   if (!ctx) return;
   DeviceGuard guard(ctx->device);
+  for (auto& entry : ctx->table_cache) mxopt_table_destroy(entry.table);
+  ctx->table_cache.clear();
+  if (ctx->d_norm_scratch) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->d_norm_scratch);
+  }
   if (ctx->d_partial_sum) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->d_partial_sum);
@@ -289,16 +299,6 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
 }
 
 // ---- tables ---------------------------------------------------------------------------
-
-static void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d) {
-  d.p = s.p; d.p_out = s.p_out; d.g = s.g; d.g_out = s.g_out; d.m = s.m; d.v = s.v;
-  d.n = s.n; d.bc1 = s.bc1; d.bc2 = s.bc2;
-  d.flags = s.flags & ~kTfUnaligned;
-  const void* ptrs[6] = {s.p, s.p_out, s.g, s.g_out, s.m, s.v};
-  for (const void* q : ptrs)
-    if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) d.flags |= kTfUnaligned;
-  d.pad = 0;
-}
 
 int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxopt_table** out) {
   if (!ctx || !out || (n && !tensors)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: null argument");
@@ -384,9 +384,19 @@ int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* 
     fill_dev_tensor(t->host[i], t->dev[i]);
   }
   if (n) {
-    // t->dev is rewritten by the next call: wait until the copy has read it.
-    HIP_TRY(ctx, hipMemcpyAsync(t->d_tensors, t->dev.data(), n * sizeof(DevTensor), hipMemcpyHostToDevice, ctx->stream));
-    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    // Stage through one of two pinned buffers so that the call returns without waiting for the
+    // copy; a buffer is reused only after the copy issued from it two calls ago has finished.
+    const size_t bytes = n * sizeof(DevTensor);
+    const int k = t->turn ^= 1;
+    if (!t->pinned[k]) {
+      HIP_TRY(ctx, hipHostMalloc((void**)&t->pinned[k], bytes, hipHostMallocDefault));
+      HIP_TRY(ctx, hipEventCreateWithFlags(&t->copied[k], hipEventDisableTiming));
+    } else {
+      HIP_TRY(ctx, hipEventSynchronize(t->copied[k]));
+    }
+    std::memcpy(t->pinned[k], t->dev.data(), bytes);
+    HIP_TRY(ctx, hipMemcpyAsync(t->d_tensors, t->pinned[k], bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, hipEventRecord(t->copied[k], ctx->stream));
   }
   return MXOPT_OK;
 }
@@ -397,6 +407,12 @@ void mxopt_table_destroy(mxopt_table* t) {
   (void)hipStreamSynchronize(t->ctx->stream);
   if (t->d_tensors) (void)hipFree(t->d_tensors);
   if (t->d_chunks) (void)hipFree(t->d_chunks);
+  for (int k = 0; k < 2; ++k) {
+    if (t->pinned[k]) {
+      (void)hipHostFree(t->pinned[k]);
+      (void)hipEventDestroy(t->copied[k]);
+    }
+  }
   delete t;
 }
 

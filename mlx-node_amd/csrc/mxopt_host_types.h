@@ -51,6 +51,8 @@ struct Group {
 
 }  // namespace mxopt
 
+struct mxopt_table;
+
 struct mxopt_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
@@ -61,6 +63,12 @@ struct mxopt_ctx {
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
   unsigned long long* d_partial_cnt = nullptr;
   size_t partial_cap = 0;
+  mxopt_norm_result* d_norm_scratch = nullptr;  // result slot of the gradient utilities
+  struct CachedTable {                          // tables built by the host layer, most recent last
+    std::vector<mxopt_tensor> key;
+    mxopt_table* table;
+  };
+  std::vector<CachedTable> table_cache;
   std::string err;
 };
 
@@ -74,4 +82,7 @@ struct mxopt_table {
   uint64_t total_elems = 0;
   uint64_t num_chunks = 0;
   uint32_t have_mask = 0;                     // which pointers are non-NULL in every non-empty tensor
+  mxopt::DevTensor* pinned[2] = {nullptr, nullptr};  // staging for per-step scalar updates
+  hipEvent_t copied[2] = {nullptr, nullptr};
+  int turn = 0;
 };

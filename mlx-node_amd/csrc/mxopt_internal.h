@@ -1,0 +1,48 @@
+// Helpers shared by the two host translation units (mxopt_api.cpp, mxopt_optimizers.cpp).
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <string>
+
+#include "mxopt.h"
+#include "mxopt_host_types.h"
+#include "mxopt_launch.h"
+
+namespace mxopt {
+
+int fail(mxopt_ctx* ctx, int code, const std::string& msg);
+int hip_fail(mxopt_ctx* ctx, hipError_t e, const char* what);
+
+#define HIP_TRY(ctx, call)                                            \
+  do {                                                                \
+    hipError_t e_ = (call);                                           \
+    if (e_ != hipSuccess) return ::mxopt::hip_fail((ctx), e_, #call); \
+  } while (0)
+
+// Makes `dev` current for the calling thread and restores the previous device on exit.
+struct DeviceGuard {
+  int prev = -1;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != dev) (void)hipSetDevice(dev);
+  }
+  ~DeviceGuard() {
+    int cur = -1;
+    if (prev >= 0 && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+  }
+};
+
+bool float_dtype(int dt);
+float round_to_dtype(float x, int dt);
+DevPrep make_prep(const mxopt_grad_prep* p);
+bool prep_active(const mxopt_grad_prep* p);
+uint32_t persistent_grid(const mxopt_ctx* ctx, uint32_t nchunks);
+int ensure_partials(mxopt_ctx* ctx, size_t need);
+int check_launch(mxopt_ctx* ctx, const char* what);
+int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode, mxopt_norm_result* d_result);
+void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d);
+// A launch over the single tensor `t` (descriptor passed in the kernel arguments).
+Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool persistent);
+
+}  // namespace mxopt

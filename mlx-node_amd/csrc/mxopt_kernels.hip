@@ -121,7 +121,7 @@ struct PlainSgdMath {
 
 template <int PD, int GD, int OD, class Math, int NT>
 __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __restrict__ T,
-                                                          const DevChunk* __restrict__ C, uint32_t nchunks,
+                                                          const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
                                                           Math math, DevPrep prep) {
   constexpr int E = (PD != MXOPT_F32 || GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
@@ -129,9 +129,18 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
   const uint32_t tid = threadIdx.x;
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    const DevChunk ch = C[c];
-    const DevTensor* t = T + ch.tensor;
-    const uint64_t start = (uint64_t)ch.index * kChunk;
+    DevTensor tv;
+    uint32_t index;
+    if (C != nullptr) {  // table walk
+      const DevChunk ch = C[c];
+      tv = T[ch.tensor];
+      index = ch.index;
+    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
+      tv = one;
+      index = c;
+    }
+    const DevTensor* t = &tv;
+    const uint64_t start = (uint64_t)index * kChunk;
     const uint64_t left = t->n - start;
     const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
     const uint32_t flags = t->flags;
@@ -203,16 +212,25 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 
 template <int GD, int OD, int NT>
 __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __restrict__ T,
-                                                             const DevChunk* __restrict__ C, uint32_t nchunks,
+                                                             const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
                                                              DevPrep prep) {
   constexpr int E = (GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    const DevChunk ch = C[c];
-    const DevTensor* t = T + ch.tensor;
-    const uint64_t start = (uint64_t)ch.index * kChunk;
+    DevTensor tv;
+    uint32_t index;
+    if (C != nullptr) {  // table walk
+      const DevChunk ch = C[c];
+      tv = T[ch.tensor];
+      index = ch.index;
+    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
+      tv = one;
+      index = c;
+    }
+    const DevTensor* t = &tv;
+    const uint64_t start = (uint64_t)index * kChunk;
     const uint64_t left = t->n - start;
     const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
     const uint32_t flags = t->flags;
@@ -259,7 +277,7 @@ __device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
 
 template <int MODE, int AD, int GD, int NT>
 __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __restrict__ T,
-                                                         const DevChunk* __restrict__ C, uint32_t nchunks,
+                                                         const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
                                                          DevPrep prep, int first, double* __restrict__ partial_sum,
                                                          unsigned long long* __restrict__ partial_cnt) {
   // AD: dtype of the stream that is squared (g for MODE 0, g_out for MODE 1/2); GD: dtype of g (MODE 2).
@@ -271,15 +289,26 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
   unsigned long long acc_cnt = 0;
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    const DevChunk ch = C[c];
-    const DevTensor* t = T + ch.tensor;
-    const uint64_t start = (uint64_t)ch.index * kChunk;
+    DevTensor tv;
+    uint32_t index;
+    if (C != nullptr) {  // table walk
+      const DevChunk ch = C[c];
+      tv = T[ch.tensor];
+      index = ch.index;
+    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
+      tv = one;
+      index = c;
+    }
+    const DevTensor* t = &tv;
+    const uint64_t start = (uint64_t)index * kChunk;
     const uint64_t left = t->n - start;
     const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
     const uint32_t flags = t->flags;
     const void* G = t->g;
     void* A = t->g_out;
-    const void* X = (MODE == 0) ? G : (const void*)A;
+    // MODE 2 reads the running sum from tensor.p when that is set (out-of-place accumulate:
+    // g_out = p + g) and from g_out itself otherwise (in place).
+    const void* X = (MODE == 0) ? G : ((MODE == 2 && t->p != nullptr) ? t->p : (const void*)A);
     float s32 = 0.0f;  // float32 partial of this lane's <=16 squares, widened once per chunk
 
     if (!(flags & kTfUnaligned) && len == (uint32_t)kChunk) {
@@ -390,7 +419,7 @@ __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __r
 // ------------------------------------------------------------------------------------
 
 #define MXOPT_LAUNCH(kernel, L, ...) \
-  hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).nchunks, __VA_ARGS__)
+  hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).one, (L).nchunks, __VA_ARGS__)
 
 template <int PD, int GD, int OD, class Math>
 static void launch_update_t(const Launch& L, const Math& math, const DevPrep& prep) {

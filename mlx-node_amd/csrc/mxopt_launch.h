@@ -5,21 +5,21 @@
 #include <stdint.h>
 
 #include "mxopt.h"
+#include "mxopt_host_types.h"
 
 namespace mxopt {
 
-struct DevTensor;
-struct DevChunk;
-struct DevPrep;
-
-// One launch = one dtype group of a table: a contiguous run of chunk entries.
+// One launch = one dtype group of a table (a contiguous run of chunk entries), or -- when
+// `chunks` is NULL -- the single tensor `one`, whose descriptor travels in the kernel
+// arguments so that nothing has to be staged in device memory.
 struct Launch {
-  const DevTensor* tensors;
-  const DevChunk* chunks;  // first chunk of the group
-  uint32_t nchunks;
-  uint32_t grid;           // workgroups (<= nchunks)
-  hipStream_t stream;
-  int nontemporal;         // bit 0: streaming loads, bit 1: streaming stores
+  const DevTensor* tensors = nullptr;
+  const DevChunk* chunks = nullptr;  // first chunk of the group
+  DevTensor one{};
+  uint32_t nchunks = 0;
+  uint32_t grid = 0;                 // workgroups (<= nchunks)
+  hipStream_t stream = nullptr;
+  int nontemporal = 0;               // bit 0: streaming loads, bit 1: streaming stores
 };
 
 // Each returns false when the dtype combination has no kernel.

@@ -95,6 +95,47 @@ SIGNATURES = {
     "mxopt_version": (C.c_char_p, []),
 }
 
+
+class Array(C.Structure):
+    """mxopt_array (include/mxopt_optimizers.h)."""
+    _fields_ = [("data", C.c_void_p), ("n", C.c_uint64), ("dtype", C.c_int32)]
+
+
+_PD = C.POINTER(C.c_double)
+_PI = C.POINTER(C.c_int)
+_PA = C.POINTER(Array)
+
+# every symbol declared in include/mxopt_optimizers.h
+SIGNATURES.update({
+    "mxopt_adam_new": (C.c_int, [C.c_void_p, _PD, _PD, _PD, _PD, _PI, C.POINTER(C.c_void_p)]),
+    "mxopt_adamw_new": (C.c_int, [C.c_void_p, _PD, _PD, _PD, _PD, _PD, _PI, C.POINTER(C.c_void_p)]),
+    "mxopt_sgd_new": (C.c_int, [C.c_void_p, C.c_double, _PD, _PD, _PD, _PI, C.POINTER(C.c_void_p)]),
+    "mxopt_rmsprop_new": (C.c_int, [C.c_void_p, _PD, _PD, _PD, _PD, C.POINTER(C.c_void_p)]),
+    "mxopt_optimizer_free": (None, [C.c_void_p]),
+    "mxopt_optimizer_update_single": (C.c_int, [C.c_void_p, C.c_char_p, _PA, _PA, _PA]),
+    "mxopt_optimizer_update_many": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA, _PA, _PA,
+                                              C.POINTER(GradPrep)]),
+    "mxopt_optimizer_reset": (C.c_int, [C.c_void_p]),
+    "mxopt_optimizer_step_count": (C.c_int64, [C.c_void_p]),
+    "mxopt_optimizer_state": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                        C.POINTER(C.c_uint64), _PI]),
+    "mxopt_optimizer_save_state": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p]),
+    "mxopt_optimizer_load_state": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64,
+                                             C.c_int64]),
+    "mxopt_compute_gradient_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, _PD]),
+    "mxopt_clip_grad_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, _PA, _PD]),
+    "mxopt_clip_grad_value": (C.c_int, [C.c_void_p, _PA, C.c_double, C.c_double, _PA]),
+    "mxopt_clip_grad_value_and_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, _PD, _PA]),
+    "mxopt_clip_gradients_by_global_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, _PA]),
+    "mxopt_clip_gradients_by_value": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, C.c_double, _PA]),
+    "mxopt_accumulate_gradients": (C.c_int, [C.c_void_p, C.c_size_t, _PA, _PA, _PA]),
+    "mxopt_apply_gradients": (C.c_int, [C.c_void_p, C.c_size_t, _PA, _PA, C.c_double, _PA]),
+    "mxopt_lr_linear_decay": (C.c_double, [C.c_double, C.c_double, C.c_int64, C.c_int64]),
+    "mxopt_lr_exponential_decay": (C.c_double, [C.c_double, C.c_double, C.c_int64, C.c_int64]),
+    "mxopt_lr_cosine_annealing": (C.c_double, [C.c_double, C.c_double, C.c_int64, C.c_int64]),
+    "mxopt_lr_step_decay": (C.c_double, [C.c_double, C.c_double, C.c_int64, C.c_int64]),
+})
+
 _lib = None
 
 
