@@ -32,7 +32,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
-                    choices=["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat", "cfg5"])
+                    choices=["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat", "cfg5", "copy"])
     ap.add_argument("--cpu-sample", type=int, default=128 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -55,6 +55,8 @@ def tensor_sizes(args):
                 shape = (max(1, int(shape[0] * args.scale)), shape[1])
             sizes.append(numel(shape))
         return sizes, f"qwen3-{model.lower()}"
+    if args.workload == "copy":
+        return [int((1 << 30) * args.scale)], "one-flat-f32-tensor"
     import numpy as np
     rng = np.random.default_rng(0x5EED0001)
     sizes = np.floor(np.exp(rng.uniform(np.log(64), np.log(65536), 10000))).astype(np.int64).tolist()
@@ -217,6 +219,21 @@ class Workload:
     def _step_cfg3_rmsprop(self):
         self._timed("rmsprop", lambda: self.ctx.rmsprop(self.t_upd, self.hp))
 
+    # -- copy: g_out = g (float32, no pre-processing): the plain copy that calibrates HBM counters
+    def _setup_copy(self):
+        t, mx = self.torch, self.mx
+        self.g = [self._randn(n, t.float32, 1.0) for n in self.sizes]
+        self.o = [t.empty_like(g) for g in self.g]
+        self.t_copy = self.ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(self.g, self.o)])
+        self.dtype = "f32"
+        self.bytes_per_elem = {"copy": 8}
+        self.step_bytes_per_elem = 8
+        self.dominant = "copy"
+        self.note = "mxopt_grad_transform with no stage enabled"
+
+    def _step_copy(self):
+        self._timed("copy", lambda: self.ctx.grad_transform(self.t_copy, None))
+
     def step(self):
         getattr(self, "_step_" + self.args.workload.replace("-", "_"))()
 
@@ -341,7 +358,7 @@ def main():
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
-    cpu = cpu_baseline(args, n) if args.cpu_sample > 0 else None
+    cpu = cpu_baseline(args, n) if args.cpu_sample > 0 and args.workload != "copy" else None
 
     out = {
         "metric": "optimizer steps/s + achieved HBM GB/s (% of 8 TB/s), AdamW on Qwen3-8B shapes",
