@@ -38,6 +38,9 @@ def parse_args():
     ap.add_argument("--scale", type=float, default=1.0,
                     help="shrink every tensor's first dimension (for quick runs; invalid as a result)")
     ap.add_argument("--option", action="append", default=[], help="mxopt option name=value")
+    ap.add_argument("--fold-last", type=int, default=1,
+                    help="cfg5: 1 = the last micro-batch is measured (norm) but folded into the update instead of "
+                         "being written to the accumulation buffer; 0 = four plain accumulation passes")
     return ap.parse_args()
 
 
@@ -119,20 +122,36 @@ class Workload:
         self.hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
         self.prep = mx.make_prep(scale=self.res)
         self.dtype = "bf16 params/grads, f32 accumulate + moments + arithmetic"
-        self.bytes_per_elem = {"accumulate_first": 6, "accumulate": 10, "accumulate_sumsq": 10, "adamw": 24}
-        self.step_bytes_per_elem = 6 + 10 * 3 + 24
+        self.fold_last = bool(self.args.fold_last)
+        if self.fold_last:
+            # the update reads the accumulation buffer AND the last micro-batch (24 + 2 B/elem); the last
+            # accumulation pass only measures the norm (6 B/elem): 6 + 10 + 10 + 6 + 26 = 58 B/elem/step
+            last = self.g[(self.n_micro - 1) % n_gbuf]
+            self.t_upd_pending = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=gl, m=m, v=v)
+                                                 for p, a, gl, m, v in zip(self.p, self.acc, last, self.m, self.v)])
+            self.bytes_per_elem = {"accumulate_first": 6, "accumulate": 10, "accumulate_norm_only": 6, "adamw": 26}
+            self.step_bytes_per_elem = 6 + 10 * 2 + 6 + 26
+        else:
+            self.bytes_per_elem = {"accumulate_first": 6, "accumulate": 10, "accumulate_sumsq": 10, "adamw": 24}
+            self.step_bytes_per_elem = 6 + 10 * 3 + 24
         self.dominant = "adamw"
-        self.note = f"{n_gbuf} resident micro-gradient buffer(s)"
+        self.note = f"{n_gbuf} resident micro-gradient buffer(s); fold_last={int(self.fold_last)}"
 
     def _step_cfg5(self):
         c = self.ctx
         for k in range(self.n_micro):
             tab = self.t_acc[k % len(self.t_acc)]
             last = k == self.n_micro - 1
+            if last and self.fold_last:
+                self._timed("accumulate_norm_only", lambda: c.accumulate_norm_only(tab, self.res, max_norm=1.0))
+                continue
             name = "accumulate_first" if k == 0 else ("accumulate_sumsq" if last else "accumulate")
             self._timed(name, lambda: c.accumulate(tab, first=(k == 0), out=self.res if last else None,
                                                    max_norm=1.0))
-        self._timed("adamw", lambda: c.adam(self.t_upd, self.hp, self.prep))
+        if self.fold_last:
+            self._timed("adamw", lambda: c.adam_with_pending(self.t_upd_pending, self.hp, self.prep))
+        else:
+            self._timed("adamw", lambda: c.adam(self.t_upd, self.hp, self.prep))
 
     # -- cfg1: fp32 AdamW
     def _setup_cfg1(self):

@@ -61,7 +61,8 @@ const char* mxopt_last_error(const mxopt_ctx* ctx);
  * crates/mlx-sys/src/mlx.cpp:189-209). */
 int mxopt_synchronize(mxopt_ctx* ctx);
 /* Tuning knobs, by name: "grid_blocks_per_cu" (persistent grid = CUs x this),
- * "persistent" (0: one workgroup per chunk for the update kernels). */
+ * "persistent" (0: one workgroup per chunk for the update kernels), "nontemporal" /
+ * "nontemporal_reduce" (streaming-hint memory instructions in the read-write / read-only kernels). */
 int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value);
 int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
 
@@ -104,7 +105,9 @@ typedef struct mxopt_norm_result {
   double   norm;      /* sqrt(sumsq)                                                */
   float    norm_f32;  /* (float)norm: what clip_grad_norm_with_norm returns          */
   float    scale;     /* clip factor, see mxopt_clip_mode                           */
-  uint64_t nonfinite; /* number of NaN/Inf gradient elements seen                   */
+  uint64_t nonfinite; /* 1 when the sum of squares is not finite (a NaN/Inf element, or
+                         squares beyond float32 range), else 0: the reference's sum-based
+                         validity check (grpo/engine.rs:1692-1698)                   */
 } mxopt_norm_result;
 
 /* How `scale` is derived from the norm. */
@@ -129,6 +132,10 @@ typedef struct mxopt_grad_prep {
   int          has_clamp_pre;  float pre_lo, pre_hi;    /* mlx clip, mlx.cpp:469-481        */
   const float* d_scale;        /* device scalar (e.g. &norm_result->scale); NULL = none    */
   int          has_clamp_post; float post_lo, post_hi;
+  /* Device counter (e.g. &norm_result->nonfinite); when it is non-zero the update / transform
+   * kernel changes nothing: the engines' "any NaN/Inf gradient => skip the whole step" policy
+   * (grpo/engine.rs:561-607, sft/engine.rs:221-258) without a host round trip.  NULL = never skip. */
+  const uint64_t* d_skip_if_nonzero;
 } mxopt_grad_prep;
 
 /* ---- hyper-parameters: float32 coefficients exactly as the reference hands them to MLX */
@@ -166,6 +173,15 @@ void mxopt_rmsprop_hp_from_f64(double lr, double alpha, double eps, double weigh
  * `prep` may be NULL. */
 int mxopt_adam(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp, const mxopt_grad_prep* prep);
 
+/* mxopt_adam with the last micro-batch still pending: the gradient is tensor.g (the float32
+ * accumulation buffer) + tensor.g_out (the micro-batch that mxopt_accumulate_norm_only measured
+ * but did not store), one float32 add, i.e. exactly the value mxopt_accumulate would have
+ * written.  Saves the accumulation buffer's last write (4 B/elem) at the price of re-reading the
+ * micro-batch (2 B/elem for bf16).  The accumulation buffer is left WITHOUT the last micro-batch.
+ * No counterpart in the reference (it has no fused accumulate/update at all). */
+int mxopt_adam_with_pending(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp,
+                            const mxopt_grad_prep* prep);
+
 /* SGD with momentum / dampening / Nesterov / coupled L2.  Reads p, g, v (unless
  * MXOPT_TF_FIRST); writes p_out, v.  Replaces SGD::update_single (optimizers/sgd.rs:84-150). */
 int mxopt_sgd(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp, const mxopt_grad_prep* prep);
@@ -185,7 +201,7 @@ int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, 
 
 /* Sum of squares of the gradients (after prep's pre_mul / clamp_pre) over the whole
  * table: wavefront shuffle -> LDS -> one float64 partial per workgroup -> one
- * single-workgroup second pass; no atomics, run-to-run deterministic.  `which` = 0 reads
+ * single-workgroup second pass; no atomics, run-to-run deterministic; the same pass yields the gradient-validity flag.  `which` = 0 reads
  * tensor.g, 1 reads tensor.g_out (the accumulation buffer).  If max_norm >= 0 the second
  * pass also derives `scale` per `clip_mode`; otherwise scale = 1.  Writes *d_result
  * (device memory).  Replaces the square/sum/add chain of GradientUtils::clip_grad_norm
@@ -209,6 +225,12 @@ int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_
  * reduced in the same pass and finished exactly like mxopt_global_norm. */
 int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep,
                      double max_norm, int clip_mode, mxopt_norm_result* d_result);
+
+/* The global norm the accumulation buffer would have after adding g, without writing it:
+ * *d_result describes g_out + g (read only, 6 B/elem for a float32 buffer and bf16 gradients).
+ * Pair with mxopt_adam_with_pending. */
+int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep, double max_norm,
+                               int clip_mode, mxopt_norm_result* d_result);
 
 /* ---- small host<->device helpers (each synchronises the context's stream) --------- */
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out);

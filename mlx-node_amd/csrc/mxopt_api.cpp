@@ -52,12 +52,14 @@ float round_to_dtype(float x, int dt) {
 DevPrep make_prep(const mxopt_grad_prep* p) {
   DevPrep d{};
   d.d_scale = nullptr;
+  d.d_skip_if_nonzero = nullptr;
   d.pre_mul = 1.0f;
   d.pre_lo = d.post_lo = -INFINITY;
   d.pre_hi = d.post_hi = INFINITY;
   d.flags = 0;
   if (!p) return d;
   d.d_scale = p->d_scale;
+  d.d_skip_if_nonzero = (const unsigned long long*)p->d_skip_if_nonzero;
   if (p->has_pre_mul) { d.flags |= kPrepPreMul; d.pre_mul = p->pre_mul; }
   // A non-finite bound means "no bound" (mlx.cpp:473-478); +-inf leaves values untouched.
   if (p->has_clamp_pre) {
@@ -86,21 +88,13 @@ int ensure_partials(mxopt_ctx* ctx, size_t need) {
   if (need <= ctx->partial_cap) return MXOPT_OK;
   size_t cap = std::max<size_t>(need, 4096);
   double* ps = nullptr;
-  unsigned long long* pc = nullptr;
   HIP_TRY(ctx, hipMalloc((void**)&ps, cap * sizeof(double)));
-  hipError_t e = hipMalloc((void**)&pc, cap * sizeof(unsigned long long));
-  if (e != hipSuccess) {
-    (void)hipFree(ps);
-    return hip_fail(ctx, e, "hipMalloc(partials)");
-  }
-  // Earlier launches may still be reading the old buffers.
+  // Earlier launches may still be reading the old buffer.
   if (ctx->d_partial_sum) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->d_partial_sum);
-    (void)hipFree(ctx->d_partial_cnt);
   }
   ctx->d_partial_sum = ps;
-  ctx->d_partial_cnt = pc;
   ctx->partial_cap = cap;
   return MXOPT_OK;
 }
@@ -135,7 +129,7 @@ Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Group& g, b
   L.nchunks = g.nchunks;
   L.grid = persistent ? persistent_grid(ctx, g.nchunks) : g.nchunks;
   L.stream = ctx->stream;
-  L.nontemporal = ctx->nontemporal & 3;
+  L.nontemporal = ctx->nontemporal;
   return L;
 }
 
@@ -148,7 +142,7 @@ std::string dtype_names(const Group& g) {
 int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode,
                        mxopt_norm_result* d_result) {
   const int has_max = max_norm >= 0.0;
-  launch_norm_finish(ctx->stream, ctx->d_partial_sum, ctx->d_partial_cnt, npartials, max_norm, has_max, clip_mode,
+  launch_norm_finish(ctx->stream, ctx->d_partial_sum, npartials, max_norm, has_max, clip_mode,
                      d_result);
   return check_launch(ctx, "norm_finish_kernel");
 }
@@ -172,9 +166,9 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
     // read-modify-write accumulation, which measured faster that way.  Only the first,
     // write-dominated accumulation pass follows the update kernels' launch policy.
     Launch L = make_launch(ctx, t, g, want || !(mode == 2 && first) || ctx->persistent != 0);
+    if (mode != 2) L.nontemporal = ctx->nontemporal_reduce;
     const int ad = mode == 0 ? g.gd : g.god;
-    if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr,
-                      want ? ctx->d_partial_cnt + offset : nullptr))
+    if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr))
       return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
     int rc = check_launch(ctx, op);
     if (rc) return rc;
@@ -212,7 +206,7 @@ Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool pers
   L.nchunks = (uint32_t)((t.n + kChunkElems - 1) / kChunkElems);
   L.grid = persistent ? persistent_grid(ctx, L.nchunks) : L.nchunks;
   L.stream = ctx->stream;
-  L.nontemporal = ctx->nontemporal & 3;
+  L.nontemporal = ctx->nontemporal;
   return L;
 }
 
@@ -256,7 +250,6 @@ void mxopt_destroy(mxopt_ctx* ctx) {
   if (ctx->d_partial_sum) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->d_partial_sum);
-    (void)hipFree(ctx->d_partial_cnt);
   }
   delete ctx;
 }
@@ -279,8 +272,9 @@ int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
   } else if (n == "persistent") {
     ctx->persistent = value != 0;
   } else if (n == "nontemporal") {
-    if (value < 0 || value > 3) return fail(ctx, MXOPT_ERR_INVALID_ARG, "nontemporal must be in [0, 3]");
-    ctx->nontemporal = (int)value;
+    ctx->nontemporal = value != 0;
+  } else if (n == "nontemporal_reduce") {
+    ctx->nontemporal_reduce = value != 0;
   } else {
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: unknown option " + n);
   }
@@ -293,6 +287,7 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
   if (n == "grid_blocks_per_cu") *value = ctx->grid_blocks_per_cu;
   else if (n == "persistent") *value = ctx->persistent;
   else if (n == "nontemporal") *value = ctx->nontemporal;
+  else if (n == "nontemporal_reduce") *value = ctx->nontemporal_reduce;
   else if (n == "num_cus") *value = ctx->num_cus;
   else return MXOPT_ERR_INVALID_ARG;
   return MXOPT_OK;
@@ -471,7 +466,18 @@ int mxopt_adam(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp, co
   if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_adam: hp is NULL");
   const DevPrep dp = make_prep(prep);
   return run_update(ctx, t, "mxopt_adam",
-                    [&](const Group& g, const Launch& L) { return launch_adam(g.pd, g.gd, g.pod, L, *hp, dp); });
+                    [&](const Group& g, const Launch& L) { return launch_adam(g.pd, g.gd, g.pod, -1, L, *hp, dp); });
+}
+
+int mxopt_adam_with_pending(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp,
+                            const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedGOut | kNeedM | kNeedV, "mxopt_adam_with_pending");
+  if (rc) return rc;
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_adam_with_pending: hp is NULL");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_adam_with_pending", [&](const Group& g, const Launch& L) {
+    return launch_adam(g.pd, g.gd, g.pod, g.god, L, *hp, dp);
+  });
 }
 
 int mxopt_sgd(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp, const mxopt_grad_prep* prep) {
@@ -531,6 +537,14 @@ int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxop
   int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_accumulate");
   if (rc) return rc;
   return run_sumsq(ctx, t, 2, first ? 1 : 0, prep, max_norm, clip_mode, d_result, "mxopt_accumulate");
+}
+
+int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep, double max_norm,
+                               int clip_mode, mxopt_norm_result* d_result) {
+  int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_accumulate_norm_only");
+  if (rc) return rc;
+  if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_accumulate_norm_only: d_result is NULL");
+  return run_sumsq(ctx, t, 3, 0, prep, max_norm, clip_mode, d_result, "mxopt_accumulate_norm_only");
 }
 
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out) {

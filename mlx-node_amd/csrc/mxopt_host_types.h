@@ -39,6 +39,7 @@ struct DevChunk {
 constexpr uint32_t kPrepPreMul = 1u, kPrepClampPre = 2u, kPrepClampPost = 4u;
 struct DevPrep {  // kernel argument
   const float* d_scale;
+  const unsigned long long* d_skip_if_nonzero;
   float pre_mul, pre_lo, pre_hi, post_lo, post_hi;
   uint32_t flags;
 };
@@ -59,9 +60,9 @@ struct mxopt_ctx {
   int num_cus = 0;
   int grid_blocks_per_cu = 16;  // bounded grids (reductions, accumulation): workgroups per CU
   int persistent = 0;           // update kernels: 0 = one workgroup per chunk, 1 = bounded grid
-  int nontemporal = 0;          // bit 0: streaming loads, bit 1: streaming stores
+  int nontemporal = 0;          // streaming-hint loads/stores in update, transform, accumulate kernels
+  int nontemporal_reduce = 1;   // streaming-hint loads in the read-only reduction kernels
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
-  unsigned long long* d_partial_cnt = nullptr;
   size_t partial_cap = 0;
   mxopt_norm_result* d_norm_scratch = nullptr;  // result slot of the gradient utilities
   struct CachedTable {                          // tables built by the host layer, most recent last

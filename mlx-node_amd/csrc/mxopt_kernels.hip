@@ -116,77 +116,118 @@ struct PlainSgdMath {
 };
 
 // ------------------------------------------------------------------------------------
-// Update kernel
+// Chunk lookup shared by all kernels
 // ------------------------------------------------------------------------------------
 
-template <int PD, int GD, int OD, class Math, int NT>
+struct ChunkView {
+  DevTensor t;
+  uint64_t start;  // first element of the chunk inside the tensor
+  uint32_t len;    // elements in this chunk (kChunk except for the last one)
+  bool fast;       // full chunk of a 16-byte aligned tensor: 128-bit path, fully unrolled
+};
+
+__device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, const DevChunk* __restrict__ C,
+                                            const DevTensor& one, uint32_t c) {
+  ChunkView cv;
+  uint32_t index;
+  if (C != nullptr) {  // table walk
+    const DevChunk ch = C[c];
+    cv.t = T[ch.tensor];
+    index = ch.index;
+  } else {             // a single tensor described in the kernel arguments: chunk c of `one`
+    cv.t = one;
+    index = c;
+  }
+  cv.start = (uint64_t)index * kChunk;
+  const uint64_t left = cv.t.n - cv.start;
+  cv.len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
+  cv.fast = !(cv.t.flags & kTfUnaligned) && cv.len == (uint32_t)kChunk;
+  return cv;
+}
+
+// The engines skip the whole step when any gradient element is NaN/Inf (grpo/engine.rs:561-607):
+// with a counter from the norm pass the update kernels honour that without a host round trip.
+__device__ __forceinline__ bool skip_requested(const DevPrep& prep) {
+  return prep.d_skip_if_nonzero != nullptr && *prep.d_skip_if_nonzero != 0ull;
+}
+
+// ------------------------------------------------------------------------------------
+// Update kernel.  G2 >= 0: a second gradient stream of that dtype in tensor.g_out is added to g
+// first (one float32 add: the last micro-batch folded into the update instead of being written
+// back to the accumulation buffer).
+// ------------------------------------------------------------------------------------
+
+template <int PD, int GD, int OD, int G2, class Math, bool NT>
 __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __restrict__ T,
-                                                          const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
-                                                          Math math, DevPrep prep) {
-  constexpr int E = (PD != MXOPT_F32 || GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
+                                                          const DevChunk* __restrict__ C, DevTensor one,
+                                                          uint32_t nchunks, Math math, DevPrep prep) {
+  constexpr bool kHasG2 = G2 >= 0;
+  constexpr int G2D = kHasG2 ? G2 : MXOPT_F32;
+  constexpr int E =
+      (PD != MXOPT_F32 || GD != MXOPT_F32 || OD != MXOPT_F32 || (kHasG2 && G2D != MXOPT_F32)) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
+  if (skip_requested(prep)) return;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    DevTensor tv;
-    uint32_t index;
-    if (C != nullptr) {  // table walk
-      const DevChunk ch = C[c];
-      tv = T[ch.tensor];
-      index = ch.index;
-    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
-      tv = one;
-      index = c;
-    }
-    const DevTensor* t = &tv;
-    const uint64_t start = (uint64_t)index * kChunk;
-    const uint64_t left = t->n - start;
-    const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
-    const uint32_t flags = t->flags;
-    const float bc1 = t->bc1, bc2 = t->bc2;
-    const void* P = t->p;
-    void* PO = t->p_out;
-    const void* G = t->g;
-    float* M = t->m;
-    float* V = t->v;
+    const ChunkView cv = locate(T, C, one, c);
+    const uint64_t start = cv.start;
+    const uint32_t len = cv.len, flags = cv.t.flags;
+    const float bc1 = cv.t.bc1, bc2 = cv.t.bc2;
+    const void* P = cv.t.p;
+    void* PO = cv.t.p_out;
+    const void* G = cv.t.g;
+    const void* G2P = cv.t.g_out;
+    float* M = cv.t.m;
+    float* V = cv.t.v;
     const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
 
-    if (!(flags & kTfUnaligned) && len == (uint32_t)kChunk) {
+    if (cv.fast) {
       // Full chunk: issue every load of the chunk before the first use.
-      float p[U][E], g[U][E], m[U][E], v[U][E];
+      float p[U][E], g[U][E], g2[U][E], m[U][E], v[U][E];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        load_group<PD, E, (NT & 1) != 0>(P, off, p[j]);
-        load_group<GD, E, (NT & 1) != 0>(G, off, g[j]);
-        if (Math::kM) load_group<MXOPT_F32, E, (NT & 1) != 0>(M, off, m[j]);
-        if (read_v) load_group<MXOPT_F32, E, (NT & 1) != 0>(V, off, v[j]);
+        load_group<PD, E, NT>(P, off, p[j]);
+        load_group<GD, E, NT>(G, off, g[j]);
+        if (kHasG2) load_group<G2D, E, NT>(G2P, off, g2[j]);
+        if (Math::kM) load_group<MXOPT_F32, E, NT>(M, off, m[j]);
+        if (read_v) load_group<MXOPT_F32, E, NT>(V, off, v[j]);
       }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) math(p[j][e], prep_all(pr, g[j][e]), m[j][e], v[j][e], bc1, bc2, flags);
+        for (int e = 0; e < E; ++e) {
+          float ge = g[j][e];
+          if (kHasG2) ge = ge + g2[j][e];
+          math(p[j][e], prep_all(pr, ge), m[j][e], v[j][e], bc1, bc2, flags);
+        }
       }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        store_group<OD, E, (NT & 2) != 0>(PO, off, p[j]);
-        if (Math::kM) store_group<MXOPT_F32, E, (NT & 2) != 0>(M, off, m[j]);
-        if (use_v) store_group<MXOPT_F32, E, (NT & 2) != 0>(V, off, v[j]);
+        store_group<OD, E, NT>(PO, off, p[j]);
+        if (Math::kM) store_group<MXOPT_F32, E, NT>(M, off, m[j]);
+        if (use_v) store_group<MXOPT_F32, E, NT>(V, off, v[j]);
       }
     } else {
       // Last chunk of a tensor, or a tensor whose buffers are not 16-byte aligned.
       const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
       for (uint32_t q = tid; q < ngroups; q += kThreads) {
         const uint64_t off = start + (uint64_t)q * E;
-        float p[E], g[E], m[E], v[E];
+        float p[E], g[E], g2[E], m[E], v[E];
         load_group<PD, E, false>(P, off, p);
         load_group<GD, E, false>(G, off, g);
+        if (kHasG2) load_group<G2D, E, false>(G2P, off, g2);
         if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m);
         if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
 #pragma unroll
-        for (int e = 0; e < E; ++e) math(p[e], prep_all(pr, g[e]), m[e], v[e], bc1, bc2, flags);
+        for (int e = 0; e < E; ++e) {
+          float ge = g[e];
+          if (kHasG2) ge = ge + g2[e];
+          math(p[e], prep_all(pr, ge), m[e], v[e], bc1, bc2, flags);
+        }
         store_group<OD, E, false>(PO, off, p);
         if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
         if (use_v) store_group<MXOPT_F32, E, false>(V, off, v);
@@ -194,10 +235,11 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
       for (uint32_t i = ngroups * E + tid; i < len; i += kThreads) {
         const uint64_t off = start + i;
         float p = Elem<PD>::load(P, off);
-        float g = prep_all(pr, Elem<GD>::load(G, off));
+        float ge = Elem<GD>::load(G, off);
+        if (kHasG2) ge = ge + Elem<G2D>::load(G2P, off);
         float m = Math::kM ? M[off] : 0.0f;
         float v = read_v ? V[off] : 0.0f;
-        math(p, g, m, v, bc1, bc2, flags);
+        math(p, prep_all(pr, ge), m, v, bc1, bc2, flags);
         Elem<OD>::store(PO, off, p);
         if (Math::kM) M[off] = m;
         if (use_v) V[off] = v;
@@ -210,44 +252,32 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 // Gradient transform: g_out = prep(g)
 // ------------------------------------------------------------------------------------
 
-template <int GD, int OD, int NT>
+template <int GD, int OD, bool NT>
 __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __restrict__ T,
-                                                             const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
-                                                             DevPrep prep) {
+                                                             const DevChunk* __restrict__ C, DevTensor one,
+                                                             uint32_t nchunks, DevPrep prep) {
   constexpr int E = (GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
+  if (skip_requested(prep)) return;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    DevTensor tv;
-    uint32_t index;
-    if (C != nullptr) {  // table walk
-      const DevChunk ch = C[c];
-      tv = T[ch.tensor];
-      index = ch.index;
-    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
-      tv = one;
-      index = c;
-    }
-    const DevTensor* t = &tv;
-    const uint64_t start = (uint64_t)index * kChunk;
-    const uint64_t left = t->n - start;
-    const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
-    const uint32_t flags = t->flags;
-    const void* G = t->g;
-    void* GO = t->g_out;
-    if (!(flags & kTfUnaligned) && len == (uint32_t)kChunk) {
+    const ChunkView cv = locate(T, C, one, c);
+    const uint64_t start = cv.start;
+    const void* G = cv.t.g;
+    void* GO = cv.t.g_out;
+    if (cv.fast) {
       float g[U][E];
 #pragma unroll
-      for (int j = 0; j < U; ++j) load_group<GD, E, (NT & 1) != 0>(G, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+      for (int j = 0; j < U; ++j) load_group<GD, E, NT>(G, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
 #pragma unroll
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int e = 0; e < E; ++e) g[j][e] = prep_all(pr, g[j][e]);
-        store_group<OD, E, (NT & 2) != 0>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+        store_group<OD, E, NT>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
       }
     } else {
-      const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
+      const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
       for (uint32_t q = tid; q < ngroups; q += kThreads) {
         float g[E];
         load_group<GD, E, false>(G, start + (uint64_t)q * E, g);
@@ -255,7 +285,7 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
         for (int e = 0; e < E; ++e) g[e] = prep_all(pr, g[e]);
         store_group<OD, E, false>(GO, start + (uint64_t)q * E, g);
       }
-      for (uint32_t i = ngroups * E + tid; i < len; i += kThreads)
+      for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads)
         Elem<OD>::store(GO, start + i, prep_all(pr, Elem<GD>::load(G, start + i)));
     }
   }
@@ -264,8 +294,11 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
 // ------------------------------------------------------------------------------------
 // Sum of squares, pass 1 (one float64 partial per workgroup), optionally fused with the
 // accumulation  acc = first ? g : acc + g.
-//   MODE 0: read tensor.g          MODE 1: read tensor.g_out
-//   MODE 2: accumulate into g_out and square the new contents (partials optional)
+//   MODE 0: square tensor.g                 MODE 1: square tensor.g_out
+//   MODE 2: g_out = first ? g : acc + g, square the new contents (partials optional); acc is
+//           tensor.p when set (out of place), else g_out itself
+//   MODE 3: square (g_out + g) without storing it (the update kernel adds g again itself)
+// AD: dtype of the stream that is squared / accumulated into; GD: dtype of g (MODE 2, 3).
 // ------------------------------------------------------------------------------------
 
 template <int AD, int GD>
@@ -275,121 +308,135 @@ __device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
   return Elem<AD>::round(s);
 }
 
-template <int MODE, int AD, int GD, int NT>
+template <int MODE, int AD, int GD, bool NT>
+struct SumsqChunk {
+  static constexpr bool kTwoStreams = MODE >= 2;
+  static constexpr int E = (AD != MXOPT_F32 || (kTwoStreams && GD != MXOPT_F32)) ? 8 : 4;
+  static constexpr int U = kElemsPerLane / E;
+  float x[U][E], g[U][E];
+
+  static __device__ __forceinline__ const void* squared_stream(const ChunkView& cv) {
+    if (MODE == 0) return cv.t.g;
+    if (MODE == 2 && cv.t.p != nullptr) return cv.t.p;
+    return cv.t.g_out;
+  }
+
+  __device__ __forceinline__ void load(const ChunkView& cv, uint32_t tid, bool first) {
+    const void* X = squared_stream(cv);
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
+      if (MODE != 2 || !first) {
+        load_group<AD, E, NT>(X, off, x[j]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[j][e] = 0.0f;
+      }
+      if (kTwoStreams) load_group<GD, E, NT>(cv.t.g, off, g[j]);
+    }
+  }
+
+  // Returns this lane's float32 sum of squares over the chunk; stores the new sum in MODE 2.
+  __device__ __forceinline__ float finish(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
+    float s32 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
+        if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
+        const float y = prep_pre(pr, x[j][e]);
+        s32 = fmaf(y, y, s32);
+      }
+      if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+    }
+    return s32;
+  }
+
+  // Partial or unaligned chunk.
+  static __device__ __forceinline__ float slow(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
+    const void* X = squared_stream(cv);
+    const void* G = cv.t.g;
+    void* A = cv.t.g_out;
+    float s32 = 0.0f;
+    const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
+    for (uint32_t q = tid; q < ngroups; q += kThreads) {
+      const uint64_t off = cv.start + (uint64_t)q * E;
+      float x[E], g[E];
+      if (MODE != 2 || !first) {
+        load_group<AD, E, false>(X, off, x);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[e] = 0.0f;
+      }
+      if (kTwoStreams) load_group<GD, E, false>(G, off, g);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
+        if (MODE == 3) x[e] = accumulate_op<AD, GD>(x[e], g[e], false);
+        const float y = prep_pre(pr, x[e]);
+        s32 = fmaf(y, y, s32);
+      }
+      if (MODE == 2) store_group<AD, E, false>(A, off, x);
+    }
+    for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) {
+      const uint64_t off = cv.start + i;
+      float x = (MODE != 2 || !first) ? Elem<AD>::load(X, off) : 0.0f;
+      if (MODE == 2) {
+        x = accumulate_op<AD, GD>(x, Elem<GD>::load(G, off), first);
+        Elem<AD>::store(A, off, x);
+      }
+      if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(G, off), false);
+      const float y = prep_pre(pr, x);
+      s32 = fmaf(y, y, s32);
+    }
+    return s32;
+  }
+};
+
+template <int MODE, int AD, int GD, bool NT>
 __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __restrict__ T,
-                                                         const DevChunk* __restrict__ C, DevTensor one, uint32_t nchunks,
-                                                         DevPrep prep, int first, double* __restrict__ partial_sum,
-                                                         unsigned long long* __restrict__ partial_cnt) {
-  // AD: dtype of the stream that is squared (g for MODE 0, g_out for MODE 1/2); GD: dtype of g (MODE 2).
-  constexpr int E = (AD != MXOPT_F32 || (MODE == 2 && GD != MXOPT_F32)) ? 8 : 4;
-  constexpr int U = kElemsPerLane / E;
+                                                         const DevChunk* __restrict__ C, DevTensor one,
+                                                         uint32_t nchunks, DevPrep prep, int first_i,
+                                                         double* __restrict__ partial_sum) {
+  using Chunk = SumsqChunk<MODE, AD, GD, NT>;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
+  const bool first = first_i != 0;
   double acc_sum = 0.0;
-  unsigned long long acc_cnt = 0;
 
-  for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
-    DevTensor tv;
-    uint32_t index;
-    if (C != nullptr) {  // table walk
-      const DevChunk ch = C[c];
-      tv = T[ch.tensor];
-      index = ch.index;
-    } else {             // a single tensor described in the kernel arguments: chunk c of `one`
-      tv = one;
-      index = c;
-    }
-    const DevTensor* t = &tv;
-    const uint64_t start = (uint64_t)index * kChunk;
-    const uint64_t left = t->n - start;
-    const uint32_t len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
-    const uint32_t flags = t->flags;
-    const void* G = t->g;
-    void* A = t->g_out;
-    // MODE 2 reads the running sum from tensor.p when that is set (out-of-place accumulate:
-    // g_out = p + g) and from g_out itself otherwise (in place).
-    const void* X = (MODE == 0) ? G : ((MODE == 2 && t->p != nullptr) ? t->p : (const void*)A);
-    float s32 = 0.0f;  // float32 partial of this lane's <=16 squares, widened once per chunk
-
-    if (!(flags & kTfUnaligned) && len == (uint32_t)kChunk) {
-      float x[U][E], g[U][E];
-#pragma unroll
-      for (int j = 0; j < U; ++j) {
-        const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        if (MODE != 2 || !first) load_group<AD, E, (NT & 1) != 0>(X, off, x[j]);
-        else {
-#pragma unroll
-          for (int e = 0; e < E; ++e) x[j][e] = 0.0f;
-        }
-        if (MODE == 2) load_group<GD, E, (NT & 1) != 0>(G, off, g[j]);
-      }
-#pragma unroll
-      for (int j = 0; j < U; ++j) {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
-          float y = prep_pre(pr, x[j][e]);
-          acc_cnt += is_nonfinite(y);
-          s32 = s32 + y * y;
-        }
-        if (MODE == 2) store_group<AD, E, (NT & 2) != 0>(A, start + (uint64_t)(j * kThreads + tid) * E, x[j]);
-      }
+  uint32_t c = blockIdx.x;
+  for (; c < nchunks; c += gridDim.x) {
+    const ChunkView cv = locate(T, C, one, c);
+    float s;
+    if (cv.fast) {
+      Chunk k;
+      k.load(cv, tid, first);
+      s = k.finish(cv, pr, tid, first);
     } else {
-      const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
-      for (uint32_t q = tid; q < ngroups; q += kThreads) {
-        const uint64_t off = start + (uint64_t)q * E;
-        float x[E], g[E];
-        if (MODE != 2 || !first) load_group<AD, E, false>(X, off, x);
-        else {
-#pragma unroll
-          for (int e = 0; e < E; ++e) x[e] = 0.0f;
-        }
-        if (MODE == 2) load_group<GD, E, false>(G, off, g);
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
-          float y = prep_pre(pr, x[e]);
-          acc_cnt += is_nonfinite(y);
-          s32 = s32 + y * y;
-        }
-        if (MODE == 2) store_group<AD, E, false>(A, off, x);
-      }
-      for (uint32_t i = ngroups * E + tid; i < len; i += kThreads) {
-        const uint64_t off = start + i;
-        float x = (MODE != 2 || !first) ? Elem<AD>::load(X, off) : 0.0f;
-        if (MODE == 2) {
-          x = accumulate_op<AD, GD>(x, Elem<GD>::load(G, off), first);
-          Elem<AD>::store(A, off, x);
-        }
-        float y = prep_pre(pr, x);
-        acc_cnt += is_nonfinite(y);
-        s32 = s32 + y * y;
-      }
+      s = Chunk::slow(cv, pr, tid, first);
     }
-    acc_sum += (double)s32;
+    // A lane's float32 partial covers <= 16 squares of one chunk; chunks are combined in float64.
+    // A NaN/Inf element (or squares that overflow float32) makes the partial, and so the total,
+    // non-finite: that is the validity check (the reference's sum-based one, grpo/engine.rs:1692-1698).
+    acc_sum += (double)s;
   }
 
   if (partial_sum != nullptr) {
-    block_sum(acc_sum, acc_cnt);
-    if (tid == 0) {
-      partial_sum[blockIdx.x] = acc_sum;
-      partial_cnt[blockIdx.x] = acc_cnt;
-    }
+    unsigned long long unused = 0;
+    block_sum(acc_sum, unused);
+    if (tid == 0) partial_sum[blockIdx.x] = acc_sum;
   }
 }
 
 // Pass 2: one workgroup folds the partials in a fixed order and derives norm and scale.
 __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __restrict__ partial_sum,
-                                                               const unsigned long long* __restrict__ partial_cnt,
                                                                uint32_t npartials, double max_norm, int has_max,
                                                                int clip_mode, mxopt_norm_result* __restrict__ out) {
   double s = 0.0;
-  unsigned long long c = 0;
-  for (uint32_t i = threadIdx.x; i < npartials; i += kThreads) {
-    s += partial_sum[i];
-    c += partial_cnt[i];
-  }
-  block_sum(s, c);
+  unsigned long long unused = 0;
+  for (uint32_t i = threadIdx.x; i < npartials; i += kThreads) s += partial_sum[i];
+  block_sum(s, unused);
   if (threadIdx.x == 0) {
     const double sumsq = s;
     const double norm = sqrt(sumsq);
@@ -410,7 +457,7 @@ __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __r
     out->norm = norm;
     out->norm_f32 = norm32;
     out->scale = scale;
-    out->nonfinite = c;
+    out->nonfinite = (sumsq - sumsq == 0.0) ? 0ull : 1ull;  // x - x is 0 exactly for finite x only
   }
 }
 
@@ -418,24 +465,23 @@ __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __r
 // Launchers (dtype dispatch)
 // ------------------------------------------------------------------------------------
 
-#define MXOPT_LAUNCH(kernel, L, ...) \
-  hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).one, (L).nchunks, __VA_ARGS__)
+#define MXOPT_LAUNCH(kernel, L, ...)                                                                          \
+  hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).one, \
+                     (L).nchunks, __VA_ARGS__)
 
-template <int PD, int GD, int OD, class Math>
+template <int PD, int GD, int OD, int G2, class Math>
 static void launch_update_t(const Launch& L, const Math& math, const DevPrep& prep) {
-  switch (L.nontemporal & 3) {
-    case 0: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 0>), L, math, prep); break;
-    case 1: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 1>), L, math, prep); break;
-    case 2: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 2>), L, math, prep); break;
-    case 3: MXOPT_LAUNCH((update_kernel<PD, GD, OD, Math, 3>), L, math, prep); break;
-  }
+  if (L.nontemporal)
+    MXOPT_LAUNCH((update_kernel<PD, GD, OD, G2, Math, true>), L, math, prep);
+  else
+    MXOPT_LAUNCH((update_kernel<PD, GD, OD, G2, Math, false>), L, math, prep);
 }
 
 template <int PD, int GD, class Math>
 static bool dispatch_od(int od, const Launch& L, const Math& math, const DevPrep& prep) {
   // The output is either float32 (what the reference returns) or the parameter's own dtype.
-  if (od == MXOPT_F32) { launch_update_t<PD, GD, MXOPT_F32>(L, math, prep); return true; }
-  if (od == PD) { launch_update_t<PD, GD, PD>(L, math, prep); return true; }
+  if (od == MXOPT_F32) { launch_update_t<PD, GD, MXOPT_F32, -1>(L, math, prep); return true; }
+  if (od == PD) { launch_update_t<PD, GD, PD, -1>(L, math, prep); return true; }
   return false;
 }
 
@@ -459,8 +505,37 @@ static bool dispatch_update(int pd, int gd, int od, const Launch& L, const Math&
   return false;
 }
 
-bool launch_adam(int pd, int gd, int od, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
-  return dispatch_update(pd, gd, od, L, AdamMath{hp}, prep);
+// Adam with the last micro-batch folded in: g is the float32 accumulation buffer, g2 any dtype.
+template <int PD>
+static bool adam_g2_for_pd(int od, int g2d, const Launch& L, const AdamMath& math, const DevPrep& prep) {
+  if (od != PD && od != MXOPT_F32) return false;
+  const bool same = od == PD;
+  switch (g2d) {
+    case MXOPT_F32:
+      if (same) launch_update_t<PD, MXOPT_F32, PD, MXOPT_F32>(L, math, prep);
+      else launch_update_t<PD, MXOPT_F32, MXOPT_F32, MXOPT_F32>(L, math, prep);
+      return true;
+    case MXOPT_BF16:
+      if (same) launch_update_t<PD, MXOPT_F32, PD, MXOPT_BF16>(L, math, prep);
+      else launch_update_t<PD, MXOPT_F32, MXOPT_F32, MXOPT_BF16>(L, math, prep);
+      return true;
+    case MXOPT_F16:
+      if (same) launch_update_t<PD, MXOPT_F32, PD, MXOPT_F16>(L, math, prep);
+      else launch_update_t<PD, MXOPT_F32, MXOPT_F32, MXOPT_F16>(L, math, prep);
+      return true;
+  }
+  return false;
+}
+
+bool launch_adam(int pd, int gd, int od, int g2d, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
+  if (g2d < 0) return dispatch_update(pd, gd, od, L, AdamMath{hp}, prep);
+  if (gd != MXOPT_F32) return false;
+  switch (pd) {
+    case MXOPT_F32: return adam_g2_for_pd<MXOPT_F32>(od, g2d, L, AdamMath{hp}, prep);
+    case MXOPT_BF16: return adam_g2_for_pd<MXOPT_BF16>(od, g2d, L, AdamMath{hp}, prep);
+    case MXOPT_F16: return adam_g2_for_pd<MXOPT_F16>(od, g2d, L, AdamMath{hp}, prep);
+  }
+  return false;
 }
 bool launch_sgd(int pd, int gd, int od, const Launch& L, const mxopt_sgd_hp& hp, const DevPrep& prep) {
   return dispatch_update(pd, gd, od, L, SgdMath{hp}, prep);
@@ -495,13 +570,13 @@ bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float
 template <int GD>
 static bool transform_for_gd(int od, const Launch& L, const DevPrep& prep) {
   if (od == MXOPT_F32) {
-    if (L.nontemporal & 2) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, 2>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, 0>), L, prep);
+    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, true>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, false>), L, prep);
     return true;
   }
   if (od == GD) {
-    if (L.nontemporal & 2) MXOPT_LAUNCH((transform_kernel<GD, GD, 2>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, GD, 0>), L, prep);
+    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, GD, true>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, GD, false>), L, prep);
     return true;
   }
   return false;
@@ -517,52 +592,46 @@ bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep) {
 }
 
 template <int MODE, int AD, int GD>
-static void launch_sumsq_t(const Launch& L, const DevPrep& prep, int first, double* ps, unsigned long long* pc) {
-  switch (L.nontemporal & 3) {
-    case 0: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 0>), L, prep, first, ps, pc); break;
-    case 1: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 1>), L, prep, first, ps, pc); break;
-    case 2: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 2>), L, prep, first, ps, pc); break;
-    case 3: MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, 3>), L, prep, first, ps, pc); break;
-  }
+static void launch_sumsq_t(const Launch& L, const DevPrep& prep, int first, double* ps) {
+  if (L.nontemporal) MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, true>), L, prep, first, ps);
+  else MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, false>), L, prep, first, ps);
 }
 
 template <int MODE, int AD>
-static bool sumsq_for_ad(int gd, const Launch& L, const DevPrep& prep, int first, double* ps, unsigned long long* pc) {
-  if (MODE != 2) { launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps, pc); return true; }
+static bool sumsq_for_ad(int gd, const Launch& L, const DevPrep& prep, int first, double* ps) {
+  if (MODE < 2) { launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps); return true; }
   switch (gd) {
-    case MXOPT_F32: launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps, pc); return true;
-    case MXOPT_BF16: launch_sumsq_t<MODE, AD, MXOPT_BF16>(L, prep, first, ps, pc); return true;
-    case MXOPT_F16: launch_sumsq_t<MODE, AD, MXOPT_F16>(L, prep, first, ps, pc); return true;
+    case MXOPT_F32: launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps); return true;
+    case MXOPT_BF16: launch_sumsq_t<MODE, AD, MXOPT_BF16>(L, prep, first, ps); return true;
+    case MXOPT_F16: launch_sumsq_t<MODE, AD, MXOPT_F16>(L, prep, first, ps); return true;
   }
   return false;
 }
 
 template <int MODE>
-static bool sumsq_for_mode(int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* ps,
-                           unsigned long long* pc) {
+static bool sumsq_for_mode(int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* ps) {
   switch (ad) {
-    case MXOPT_F32: return sumsq_for_ad<MODE, MXOPT_F32>(gd, L, prep, first, ps, pc);
-    case MXOPT_BF16: return sumsq_for_ad<MODE, MXOPT_BF16>(gd, L, prep, first, ps, pc);
-    case MXOPT_F16: return sumsq_for_ad<MODE, MXOPT_F16>(gd, L, prep, first, ps, pc);
+    case MXOPT_F32: return sumsq_for_ad<MODE, MXOPT_F32>(gd, L, prep, first, ps);
+    case MXOPT_BF16: return sumsq_for_ad<MODE, MXOPT_BF16>(gd, L, prep, first, ps);
+    case MXOPT_F16: return sumsq_for_ad<MODE, MXOPT_F16>(gd, L, prep, first, ps);
   }
   return false;
 }
 
-bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum,
-                  unsigned long long* partial_cnt) {
+bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum) {
   switch (mode) {
-    case 0: return sumsq_for_mode<0>(ad, gd, L, prep, first, partial_sum, partial_cnt);
-    case 1: return sumsq_for_mode<1>(ad, gd, L, prep, first, partial_sum, partial_cnt);
-    case 2: return sumsq_for_mode<2>(ad, gd, L, prep, first, partial_sum, partial_cnt);
+    case 0: return sumsq_for_mode<0>(ad, gd, L, prep, first, partial_sum);
+    case 1: return sumsq_for_mode<1>(ad, gd, L, prep, first, partial_sum);
+    case 2: return sumsq_for_mode<2>(ad, gd, L, prep, first, partial_sum);
+    case 3: return sumsq_for_mode<3>(ad, gd, L, prep, first, partial_sum);
   }
   return false;
 }
 
-void launch_norm_finish(hipStream_t stream, const double* partial_sum, const unsigned long long* partial_cnt,
-                        uint32_t npartials, double max_norm, int has_max, int clip_mode,
-                        mxopt_norm_result* d_out) {
-  hipLaunchKernelGGL(norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, partial_sum, partial_cnt, npartials,
-                     max_norm, has_max, clip_mode, d_out);
+void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,
+                        int has_max, int clip_mode, mxopt_norm_result* d_out) {
+  hipLaunchKernelGGL(norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, partial_sum, npartials, max_norm,
+                     has_max, clip_mode, d_out);
 }
 
 }  // namespace mxopt

@@ -19,22 +19,23 @@ struct Launch {
   uint32_t nchunks = 0;
   uint32_t grid = 0;                 // workgroups (<= nchunks)
   hipStream_t stream = nullptr;
-  int nontemporal = 0;               // bit 0: streaming loads, bit 1: streaming stores
+  int nontemporal = 0;               // non-zero: streaming-hint loads and stores
 };
 
 // Each returns false when the dtype combination has no kernel.
-bool launch_adam(int pd, int gd, int od, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep);
+// g2d >= 0: tensor.g_out holds a second gradient of that dtype which is added to g (float32) first.
+bool launch_adam(int pd, int gd, int od, int g2d, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep);
 bool launch_sgd(int pd, int gd, int od, const Launch& L, const mxopt_sgd_hp& hp, const DevPrep& prep);
 bool launch_rmsprop(int pd, int gd, int od, const Launch& L, const mxopt_rmsprop_hp& hp, const DevPrep& prep);
 // g_promoted: the gradient reaches the multiply as float32 (decay or a prep stage ran first).
 bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float wd, int has_wd, bool g_promoted,
                       const DevPrep& prep);
 bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep);
-// mode 0: square g; 1: square g_out; 2: g_out = first ? g : g_out + g, square the result.
-// partial_sum/partial_cnt (one entry per workgroup) may be NULL in mode 2.
-bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum,
-                  unsigned long long* partial_cnt);
-void launch_norm_finish(hipStream_t stream, const double* partial_sum, const unsigned long long* partial_cnt,
-                        uint32_t npartials, double max_norm, int has_max, int clip_mode, mxopt_norm_result* d_out);
+// mode 0: square g; 1: square g_out; 2: g_out = first ? g : g_out + g, square the result;
+// 3: square g_out + g without storing it.
+// partial_sum (one entry per workgroup) may be NULL in mode 2.
+bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum);
+void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,
+                        int has_max, int clip_mode, mxopt_norm_result* d_out);
 
 }  // namespace mxopt

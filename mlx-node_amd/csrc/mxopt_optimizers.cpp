@@ -309,7 +309,7 @@ int mxopt_optimizer_update_single(mxopt_optimizer* opt, const char* param_name, 
   bool ok = false;
   switch (opt->kind) {
     case Kind::Adam:
-    case Kind::AdamW: ok = launch_adam(row.p_dtype, row.g_dtype, row.p_out_dtype, L, hp.adam, prep); break;
+    case Kind::AdamW: ok = launch_adam(row.p_dtype, row.g_dtype, row.p_out_dtype, -1, L, hp.adam, prep); break;
     case Kind::Sgd: ok = launch_sgd(row.p_dtype, row.g_dtype, row.p_out_dtype, L, hp.sgd, prep); break;
     case Kind::Rmsprop: ok = launch_rmsprop(row.p_dtype, row.g_dtype, row.p_out_dtype, L, hp.rms, prep); break;
   }

@@ -42,7 +42,8 @@ class GradPrep(C.Structure):
     _fields_ = [("has_pre_mul", C.c_int), ("pre_mul", C.c_float),
                 ("has_clamp_pre", C.c_int), ("pre_lo", C.c_float), ("pre_hi", C.c_float),
                 ("d_scale", C.c_void_p),
-                ("has_clamp_post", C.c_int), ("post_lo", C.c_float), ("post_hi", C.c_float)]
+                ("has_clamp_post", C.c_int), ("post_lo", C.c_float), ("post_hi", C.c_float),
+                ("d_skip_if_nonzero", C.c_void_p)]
 
 
 class AdamHp(C.Structure):
@@ -83,6 +84,7 @@ SIGNATURES = {
     "mxopt_sgd_hp_from_f64": (C.c_int, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_int, C.POINTER(SgdHp)]),
     "mxopt_rmsprop_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.POINTER(RmspropHp)]),
     "mxopt_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_adam_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
     "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),
     "mxopt_sgd_plain": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double, C.POINTER(GradPrep)]),
@@ -91,6 +93,8 @@ SIGNATURES = {
     "mxopt_grad_transform": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep)]),
     "mxopt_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
                                    C.c_void_p]),
+    "mxopt_accumulate_norm_only": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                             C.c_void_p]),
     "mxopt_read_norm_result": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(NormResult)]),
     "mxopt_version": (C.c_char_p, []),
 }

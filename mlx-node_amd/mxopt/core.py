@@ -71,9 +71,9 @@ class TensorSpec:
 
 
 def make_prep(pre_mul: Optional[float] = None, clamp_pre: Optional[Sequence[float]] = None,
-              scale: Optional["NormResultBuffer"] = None, clamp_post: Optional[Sequence[float]] = None
-              ) -> Optional[L.GradPrep]:
-    if pre_mul is None and clamp_pre is None and scale is None and clamp_post is None:
+              scale: Optional["NormResultBuffer"] = None, clamp_post: Optional[Sequence[float]] = None,
+              skip_if_nonfinite: Optional["NormResultBuffer"] = None) -> Optional[L.GradPrep]:
+    if pre_mul is None and clamp_pre is None and scale is None and clamp_post is None and skip_if_nonfinite is None:
         return None
     p = L.GradPrep()
     if pre_mul is not None:
@@ -84,6 +84,8 @@ def make_prep(pre_mul: Optional[float] = None, clamp_pre: Optional[Sequence[floa
         p.d_scale = scale.scale_ptr
     if clamp_post is not None:
         p.has_clamp_post, p.post_lo, p.post_hi = 1, clamp_post[0], clamp_post[1]
+    if skip_if_nonfinite is not None:
+        p.d_skip_if_nonzero = skip_if_nonfinite.nonfinite_ptr
     return p
 
 
@@ -102,6 +104,10 @@ class NormResultBuffer:
     @property
     def scale_ptr(self) -> int:
         return self.buf.data_ptr() + L.NormResult.scale.offset
+
+    @property
+    def nonfinite_ptr(self) -> int:
+        return self.buf.data_ptr() + L.NormResult.nonfinite.offset
 
 
 class Context:
@@ -152,6 +158,10 @@ class Context:
         L.check(self.lib.mxopt_adam(self.handle, table.handle, C.byref(hp), C.byref(prep) if prep else None),
                 self.handle)
 
+    def adam_with_pending(self, table: "Table", hp: L.AdamHp, prep: Optional[L.GradPrep] = None) -> None:
+        L.check(self.lib.mxopt_adam_with_pending(self.handle, table.handle, C.byref(hp),
+                                                 C.byref(prep) if prep else None), self.handle)
+
     def sgd(self, table: "Table", hp: L.SgdHp, prep: Optional[L.GradPrep] = None) -> None:
         L.check(self.lib.mxopt_sgd(self.handle, table.handle, C.byref(hp), C.byref(prep) if prep else None),
                 self.handle)
@@ -180,6 +190,15 @@ class Context:
                    clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
         L.check(self.lib.mxopt_accumulate(self.handle, table.handle, int(first), C.byref(prep) if prep else None,
                                           max_norm, clip_mode, C.c_void_p(out.ptr) if out else None), self.handle)
+
+
+def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Optional[L.GradPrep] = None,
+                          max_norm: float = -1.0, clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
+    L.check(self.lib.mxopt_accumulate_norm_only(self.handle, table.handle, C.byref(prep) if prep else None,
+                                                max_norm, clip_mode, C.c_void_p(out.ptr)), self.handle)
+
+
+Context.accumulate_norm_only = _accumulate_norm_only
 
 
 class Table:

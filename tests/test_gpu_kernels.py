@@ -268,7 +268,7 @@ def test_global_norm_and_scales(mx, ctx, bf16, offset):
     assert ctx.read_norm_result(res).scale == 1.0
 
 
-def test_global_norm_is_deterministic_and_counts_nonfinite(mx, ctx):
+def test_global_norm_is_deterministic_and_flags_nonfinite(mx, ctx):
     _, gs = make_lists(52, sizes=[4096 * 50 + 1, 77])
     gs[0][5] = np.inf
     gs[0][4096 * 3] = np.nan
@@ -278,7 +278,7 @@ def test_global_norm_is_deterministic_and_counts_nonfinite(mx, ctx):
     res = ctx.norm_result()
     ctx.global_norm(table, res, max_norm=1.0)
     r = ctx.read_norm_result(res)
-    assert r.nonfinite == 3 and math.isnan(r.sumsq) and math.isnan(r.scale)
+    assert r.nonfinite == 1 and math.isnan(r.sumsq) and math.isnan(r.scale)   # a flag, not a count
     gs[0][5] = gs[0][4096 * 3] = 0
     gs[1][76] = 0
     dg = [to_dev(g) for g in gs]
@@ -430,3 +430,88 @@ def test_errors(mx, ctx):
     other.close()
     empty = ctx.table([])
     ctx.global_norm(empty, ctx.norm_result(), max_norm=1.0)   # legal: norm 0, scale 1
+
+
+# ---------------------------------------------------------------------------------
+# Last micro-batch folded into the update; skip-on-non-finite policy
+# ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("g_bf16", [True, False])
+def test_pending_micro_batch_equals_accumulate_then_adam(mx, ctx, g_bf16):
+    """accumulate_norm_only + adam_with_pending give the numbers of accumulate(+norm) + adam,
+    without writing the accumulation buffer a last time."""
+    import torch
+    ps, _ = make_lists(80, bf16=True)
+    micro = [make_lists(81 + k, bf16=g_bf16)[1] for k in range(3)]
+    n_t = len(ps)
+    hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
+    results = []
+    for fused in (False, True):
+        dp = [to_dev(p) for p in ps]
+        dg = [to_dev(g) for g in micro[0]]
+        acc = [torch.empty(len(p), dtype=torch.float32, device="cuda") for p in ps]
+        dm = [torch.zeros(len(p), dtype=torch.float32, device="cuda") for p in ps]
+        dv = [torch.zeros(len(p), dtype=torch.float32, device="cuda") for p in ps]
+        t_acc = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(dg, acc)])
+        res = ctx.norm_result()
+        for k in range(3):
+            for i in range(n_t):
+                dg[i].copy_(to_dev(micro[k][i]))
+            last = k == 2
+            if last and fused:
+                ctx.accumulate_norm_only(t_acc, res, max_norm=1e-3)
+            else:
+                ctx.accumulate(t_acc, first=(k == 0), out=res if last else None, max_norm=1e-3)
+        prep = mx.make_prep(scale=res)
+        if fused:
+            t = ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=g, m=m, v=v)
+                           for p, a, g, m, v in zip(dp, acc, dg, dm, dv)])
+            ctx.adam_with_pending(t, hp, prep)
+        else:
+            t = ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, m=m, v=v) for p, a, m, v in zip(dp, acc, dm, dv)])
+            ctx.adam(t, hp, prep)
+        r = ctx.read_norm_result(res)
+        results.append((r.sumsq, r.scale, [to_host(x) for x in dp], [to_host(x) for x in dm], [to_host(x) for x in dv]))
+    a, b = results
+    assert a[0] == b[0] and a[1] == b[1]
+    for i in range(n_t):
+        assert_bit_equal(b[2][i], a[2][i], f"p{i}")
+        assert_bit_equal(b[3][i], a[3][i], f"m{i}")
+        assert_bit_equal(b[4][i], a[4][i], f"v{i}")
+    # and the un-fused side is the oracle's
+    acc_ref = [None] * n_t
+    for k in range(3):
+        for i in range(n_t):
+            acc_ref[i] = O.accumulate_fp32(acc_ref[i], micro[k][i])
+    ref = O.AdamW(5e-6, 0.9, 0.999, 1e-8, 0.01)
+    for i in range(n_t):
+        want = O.f32_to_bf16(ref.update_single(str(i), ps[i], acc_ref[i] * F(a[1])))
+        assert_bit_equal(a[2][i], want, f"oracle p{i}")
+
+
+def test_skip_step_when_a_gradient_is_not_finite(mx, ctx):
+    """grpo/engine.rs:561-607: any NaN/Inf gradient => nothing is modified.  The counter comes from
+    the norm pass; no host round trip."""
+    import torch
+    ps, gs = make_lists(90, sizes=[4096 * 3 + 5, 100, 4096])
+    for poison in (True, False):
+        g2 = [g.copy() for g in gs]
+        if poison:
+            g2[0][4096 + 17] = np.nan
+        dp, dg = [to_dev(p) for p in ps], [to_dev(g) for g in g2]
+        dm = [torch.zeros_like(p) for p in dp]
+        dv = [torch.zeros_like(p) for p in dp]
+        out = [torch.full_like(g, 7.0) for g in dg]
+        t_g = ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(dg, out)])
+        t_u = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
+        res = ctx.norm_result()
+        ctx.global_norm(t_g, res, max_norm=1.0)
+        prep = mx.make_prep(scale=res, skip_if_nonfinite=res)
+        ctx.adam(t_u, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01), prep)
+        ctx.grad_transform(t_g, prep)
+        assert ctx.read_norm_result(res).nonfinite == (1 if poison else 0)
+        for i in range(len(ps)):
+            changed = not np.array_equal(to_host(dp[i]), ps[i])
+            assert changed != poison, f"tensor {i}"
+            assert (to_host(dm[i]) == 0).all() == poison
+            assert (to_host(out[i]) == 7.0).all() == poison
