@@ -38,6 +38,9 @@ def parse_args():
     ap.add_argument("--scale", type=float, default=1.0,
                     help="shrink every tensor's first dimension (for quick runs; invalid as a result)")
     ap.add_argument("--option", action="append", default=[], help="mxopt option name=value")
+    ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab"],
+                    help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
+                         "tensors are 512-byte aligned views into it")
     ap.add_argument("--fold-last", type=int, default=1,
                     help="cfg5: 1 = the last micro-batch is measured (norm) but folded into the update instead of "
                          "being written to the accumulation buffer; 0 = four plain accumulation passes")
@@ -91,6 +94,39 @@ class Workload:
     def _zeros(self, n):
         return self.torch.zeros(n, dtype=self.torch.float32, device="cuda")
 
+    # one list of tensors per stream, either separately allocated or carved out of one slab
+    def _carve(self, dtype):
+        t = self.torch
+        if getattr(self.args, "alloc", "tensor") != "slab":
+            return None, [t.empty(n, dtype=dtype, device="cuda") for n in self.sizes]
+        offs, total = [], 0
+        for n in self.sizes:
+            offs.append(total)
+            total += (n + 255) // 256 * 256          # 512 B (bf16) / 1 KiB (f32) alignment
+        slab = t.empty(max(total, 1), dtype=dtype, device="cuda")
+        return slab, [slab[o:o + n] for o, n in zip(offs, self.sizes)]
+
+    def _randn_list(self, dtype, std):
+        slab, views = self._carve(dtype)
+        if slab is not None:
+            slab.normal_(0.0, std)
+        else:
+            for v in views:
+                v.normal_(0.0, std)
+        return views
+
+    def _zeros_list(self):
+        slab, views = self._carve(self.torch.float32)
+        if slab is not None:
+            slab.zero_()
+        else:
+            for v in views:
+                v.zero_()
+        return views
+
+    def _empty_list(self, dtype):
+        return self._carve(dtype)[1]
+
     def _timed(self, name, fn):
         s = self.torch.cuda.Event(enable_timing=True)
         e = self.torch.cuda.Event(enable_timing=True)
@@ -111,11 +147,11 @@ class Workload:
         free, _ = t.cuda.mem_get_info()
         self.n_micro = 4
         n_gbuf = 4 if free > need + 4 * self.n * 2 + (8 << 30) else 1
-        self.p = [self._randn(n, bf, 0.02) for n in self.sizes]
-        self.m = [self._zeros(n) for n in self.sizes]
-        self.v = [self._zeros(n) for n in self.sizes]
-        self.acc = [t.empty(n, dtype=t.float32, device="cuda") for n in self.sizes]
-        self.g = [[self._randn(n, bf, 1e-3) for n in self.sizes] for _ in range(n_gbuf)]
+        self.p = self._randn_list(bf, 0.02)
+        self.m = self._zeros_list()
+        self.v = self._zeros_list()
+        self.acc = self._empty_list(t.float32)
+        self.g = [self._randn_list(bf, 1e-3) for _ in range(n_gbuf)]
         self.t_acc = [self.ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(gk, self.acc)]) for gk in self.g]
         self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, m=m, v=v)
                                      for p, a, m, v in zip(self.p, self.acc, self.m, self.v)])
@@ -156,10 +192,10 @@ class Workload:
     # -- cfg1: fp32 AdamW
     def _setup_cfg1(self):
         t, mx = self.torch, self.mx
-        self.p = [self._randn(n, t.float32, 0.02) for n in self.sizes]
-        self.g = [self._randn(n, t.float32, 1e-3) for n in self.sizes]
-        self.m = [self._zeros(n) for n in self.sizes]
-        self.v = [self._zeros(n) for n in self.sizes]
+        self.p = self._randn_list(t.float32, 0.02)
+        self.g = self._randn_list(t.float32, 1e-3)
+        self.m = self._zeros_list()
+        self.v = self._zeros_list()
         self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
                                      for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
         self.hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01)
@@ -179,13 +215,13 @@ class Workload:
         if uniform_p:
             self.p = [t.empty(n, dtype=bf, device="cuda").uniform_(0.9, 1.1) for n in self.sizes]
         else:
-            self.p = [self._randn(n, bf, 0.02) for n in self.sizes]
-        self.g = [self._randn(n, bf, gstd) for n in self.sizes]
+            self.p = self._randn_list(bf, 0.02)
+        self.g = self._randn_list(bf, gstd)
         if self.args.workload == "cfg2":   # 1 % of the elements are x100 outliers
             for g in self.g:
                 g.mul_(t.where(t.rand(g.shape, device="cuda") < 0.01, 100.0, 1.0).to(bf))
-        self.m = [self._zeros(n) for n in self.sizes]
-        self.v = [self._zeros(n) for n in self.sizes]
+        self.m = self._zeros_list()
+        self.v = self._zeros_list()
         self.t_g = self.ctx.table([mx.TensorSpec(g=g) for g in self.g])
         self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
                                      for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
@@ -211,9 +247,9 @@ class Workload:
     # -- cfg3: fp32 SGD / RMSprop
     def _setup_cfg3(self):
         t, mx = self.torch, self.mx
-        self.p = [self._randn(n, t.float32, 0.02) for n in self.sizes]
-        self.g = [self._randn(n, t.float32, 1e-3) for n in self.sizes]
-        self.v = [self._zeros(n) for n in self.sizes]
+        self.p = self._randn_list(t.float32, 0.02)
+        self.g = self._randn_list(t.float32, 1e-3)
+        self.v = self._zeros_list()
         self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v)
                                      for p, g, v in zip(self.p, self.g, self.v)])
         self.dtype = "f32"
@@ -241,7 +277,7 @@ class Workload:
     # -- copy: g_out = g (float32, no pre-processing): the plain copy that calibrates HBM counters
     def _setup_copy(self):
         t, mx = self.torch, self.mx
-        self.g = [self._randn(n, t.float32, 1.0) for n in self.sizes]
+        self.g = self._randn_list(t.float32, 1.0)
         self.o = [t.empty_like(g) for g in self.g]
         self.t_copy = self.ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(self.g, self.o)])
         self.dtype = "f32"
@@ -385,7 +421,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
-                   "bytes_per_elem_per_step": wl.step_bytes_per_elem, "note": wl.note, "scale": args.scale},
+                   "bytes_per_elem_per_step": wl.step_bytes_per_elem, "note": wl.note, "scale": args.scale,
+                   "alloc": args.alloc},
         "elements_per_s": round(n * steps_per_s, 1),
         "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "kernels": kernels,
