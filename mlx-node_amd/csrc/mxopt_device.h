@@ -27,13 +27,15 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
-// Round-to-nearest-even; NaN stays a quiet NaN.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  uint32_t q = (u >> 16) | 0x40u;
-  return ((u & 0x7fffffffu) > 0x7f800000u) ? q : r;
+// float32 -> bf16, round-to-nearest-even, NaN stays a quiet NaN: gfx950's v_cvt_pk_bf16_f32
+// (two elements per instruction), reached through the compiler's native bf16 vector type.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return f32x2_to_bf16x2_bits(f, 0.0f) & 0xffffu; }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
@@ -58,6 +60,7 @@ struct Elem<MXOPT_BF16> {
   static constexpr int kBytes = 2;
   static __device__ __forceinline__ float unpack(uint32_t b) { return bf16_bits_to_f32(b); }
   static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_bf16_bits(x); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
   static __device__ __forceinline__ float load(const void* base, uint64_t i) {
     return unpack(((const uint16_t*)base)[i]);
   }
@@ -72,6 +75,7 @@ struct Elem<MXOPT_F16> {
   static constexpr int kBytes = 2;
   static __device__ __forceinline__ float unpack(uint32_t b) { return f16_bits_to_f32(b); }
   static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_f16_bits(x); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack(lo) | (pack(hi) << 16); }
   static __device__ __forceinline__ float load(const void* base, uint64_t i) {
     return unpack(((const uint16_t*)base)[i]);
   }
@@ -121,16 +125,16 @@ __device__ __forceinline__ void store_group(void* base, uint64_t off, const floa
     }
   } else if constexpr (E == 8) {
     u32x4 t;
-    t.x = Elem<DT>::pack(x[0]) | (Elem<DT>::pack(x[1]) << 16);
-    t.y = Elem<DT>::pack(x[2]) | (Elem<DT>::pack(x[3]) << 16);
-    t.z = Elem<DT>::pack(x[4]) | (Elem<DT>::pack(x[5]) << 16);
-    t.w = Elem<DT>::pack(x[6]) | (Elem<DT>::pack(x[7]) << 16);
+    t.x = Elem<DT>::pack2(x[0], x[1]);
+    t.y = Elem<DT>::pack2(x[2], x[3]);
+    t.z = Elem<DT>::pack2(x[4], x[5]);
+    t.w = Elem<DT>::pack2(x[6], x[7]);
     u32x4* q = (u32x4*)((uint16_t*)base + off);
     if (NT) __builtin_nontemporal_store(t, q); else *q = t;
   } else {
     u32x2 t;
-    t.x = Elem<DT>::pack(x[0]) | (Elem<DT>::pack(x[1]) << 16);
-    t.y = Elem<DT>::pack(x[2]) | (Elem<DT>::pack(x[3]) << 16);
+    t.x = Elem<DT>::pack2(x[0], x[1]);
+    t.y = Elem<DT>::pack2(x[2], x[3]);
     u32x2* q = (u32x2*)((uint16_t*)base + off);
     if (NT) __builtin_nontemporal_store(t, q); else *q = t;
   }
