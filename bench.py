@@ -2,9 +2,11 @@
 """Benchmark of the optimizer-step hot path on one MI355X.
 
 Default workload (the one the headline metric is quoted on): Qwen3-8B-shaped training step --
-4 micro-batch bf16 gradients accumulated into a float32 buffer, global-norm clip at 1.0 (sum of
-squares fused into the last accumulation pass), AdamW with bf16 parameters updated in place and
-float32 moments; everything resident in HBM (~131 GB + 3 more micro-gradient buffers).
+4 micro-batch bf16 gradients accumulated into a float32 buffer, global-norm clip at 1.0, AdamW
+with bf16 parameters updated in place and float32 moments; everything resident in HBM (~131 GB
++ 3 more micro-gradient buffers).  By default the 4th micro-batch is only measured (its norm
+contribution) and then folded into the update kernel, which saves the accumulation buffer's
+last write: 6 + 10 + 10 + 6 + 26 = 58 B/elem/step instead of 6 + 3*10 + 24 = 60 (--fold-last 0).
 
 Prints ONE JSON line.  `value` = optimizer steps/s over the timed region (inputs resident
 before it starts).  `roofline` describes the dominant kernel (the AdamW update): algorithmic
@@ -24,6 +26,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
 
 HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per element per launch of the dominant kernel, measured with rocprofv3 FETCH_SIZE and
+# WRITE_SIZE (each scaled by what the same counter reads for this library's plain copy kernel:
+# 1.98445 and 1.00000); the runs and raw values are in profiles/hbm_traffic_pmc_cfg5_and_copy.txt.
+# (workload, fold_last) -> bytes per element
+MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.97, ("cfg5", 0): 23.93}
 
 
 def parse_args():
@@ -409,7 +417,9 @@ def main():
                          "bytes_per_elem": bpe, "gbps": round(bpe * n / (avg * 1e-3) / 1e9, 1)}
     dom = kernels[wl.dominant]
     roofline = {"bound": "hbm", "achieved": dom["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(dom["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                "frac": round(dom["gbps"] / HBM_PEAK_GBPS, 4),
+                "traffic": (round(MEASURED_TRAFFIC_B_PER_ELEM[(args.workload, int(args.fold_last))] * n)
+                            if (args.workload, int(args.fold_last)) in MEASURED_TRAFFIC_B_PER_ELEM else None),
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
