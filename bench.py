@@ -40,13 +40,14 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
-                    choices=["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat", "cfg5", "copy"])
+                    choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
+                             "cfg4", "cfg4-flat", "cfg5", "copy"])
     ap.add_argument("--cpu-sample", type=int, default=128 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
                     help="shrink every tensor's first dimension (for quick runs; invalid as a result)")
     ap.add_argument("--option", action="append", default=[], help="mxopt option name=value")
-    ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab"],
+    ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab", "packed"],
                     help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
                          "tensors are 512-byte aligned views into it")
     ap.add_argument("--fold-last", type=int, default=1,
@@ -61,7 +62,7 @@ def parse_args():
 
 def tensor_sizes(args):
     from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    model = {"cfg1": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B"}.get(args.workload)
+    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B"}.get(args.workload)
     if model:
         sizes = []
         for _, shape in param_list(QWEN3[model]):
@@ -105,12 +106,14 @@ class Workload:
     # one list of tensors per stream, either separately allocated or carved out of one slab
     def _carve(self, dtype):
         t = self.torch
-        if getattr(self.args, "alloc", "tensor") != "slab":
+        mode = getattr(self.args, "alloc", "tensor")
+        if mode == "tensor":
             return None, [t.empty(n, dtype=dtype, device="cuda") for n in self.sizes]
         offs, total = [], 0
         for n in self.sizes:
             offs.append(total)
-            total += (n + 255) // 256 * 256          # 512 B (bf16) / 1 KiB (f32) alignment
+            # slab: 512 B (bf16) / 1 KiB (f32) alignment; packed: back to back, natural alignment only
+            total += (n + 255) // 256 * 256 if mode == "slab" else n
         slab = t.empty(max(total, 1), dtype=dtype, device="cuda")
         return slab, [slab[o:o + n] for o, n in zip(offs, self.sizes)]
 
@@ -215,6 +218,27 @@ class Workload:
 
     def _step_cfg1(self):
         self._timed("adamw", lambda: self.ctx.adam(self.t_upd, self.hp))
+
+    # -- cfg1 through the optimizer object, as the reference's callers use it: one updateSingle per tensor
+    #    returning a new array (310 launches per step), or the same loop as one update_many call in place
+    def _setup_cfg1_update_single(self):
+        from mxopt.qwen3_shapes import QWEN3, param_list
+        self._setup_cfg1()
+        self.names = [name for name, _ in param_list(QWEN3["0.6B"])]
+        self.opt = self.mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, ctx=self.ctx)
+        self.bytes_per_elem = {"adamw_object": 28}
+        self.dominant = "adamw_object"
+        self.note = "AdamW object through ctypes: " + self.args.workload.split("-", 1)[1]
+
+    _setup_cfg1_update_many = _setup_cfg1_update_single
+
+    def _step_cfg1_update_single(self):
+        def loop():
+            self.p = [self.opt.update_single(nm, p, g) for nm, p, g in zip(self.names, self.p, self.g)]
+        self._timed("adamw_object", loop)
+
+    def _step_cfg1_update_many(self):
+        self._timed("adamw_object", lambda: self.opt.update_many(self.names, self.p, self.g, outs=self.p))
 
     # -- cfg2 / cfg4: bf16 p,g + f32 m,v AdamW with a separate norm pass
     def _setup_cfg2(self, lr=5e-6, wd=0.01, gstd=1e-3, uniform_p=False):
@@ -348,7 +372,7 @@ def cpu_baseline(args, n_total):
                 if w == "cfg5" else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
         t_unfused = timeit(lambda: step(False))
         fused_s = timeit(lambda: step(True))
-    elif w == "cfg1":
+    elif w.startswith("cfg1"):
         a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01)
         t_unfused = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=False))
         fused_s = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=True))
@@ -396,11 +420,15 @@ def main():
     torch.cuda.synchronize()
     wl.kernel_events.clear()
 
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        marks[i].record(wl.ctx.stream)
         wl.step()
+    marks[-1].record(wl.ctx.stream)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    step_ms = sorted(a.elapsed_time(b) for a, b in zip(marks[:-1], marks[1:]))
 
     ms_per_step = elapsed * 1e3 / args.steps
     steps_per_s = args.steps / elapsed
@@ -428,7 +456,8 @@ def main():
     out = {
         "metric": "optimizer steps/s + achieved HBM GB/s (% of 8 TB/s), AdamW on Qwen3-8B shapes",
         "value": round(steps_per_s, 4), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(step_ms[len(step_ms) // 2], 4),
+        "ms_per_step_min": round(step_ms[0], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
                    "bytes_per_elem_per_step": wl.step_bytes_per_elem, "note": wl.note, "scale": args.scale,

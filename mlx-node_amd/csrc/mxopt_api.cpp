@@ -32,6 +32,7 @@ int hip_fail(mxopt_ctx* ctx, hipError_t e, const char* what) {
 
 
 bool float_dtype(int dt) { return dt == MXOPT_F32 || dt == MXOPT_F16 || dt == MXOPT_BF16; }
+static int dtype_size(int dt) { return dt == MXOPT_F32 ? 4 : 2; }
 
 float round_to_dtype(float x, int dt) {
   if (dt == MXOPT_BF16) {
@@ -194,16 +195,35 @@ void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d) {
   d.p = s.p; d.p_out = s.p_out; d.g = s.g; d.g_out = s.g_out; d.m = s.m; d.v = s.v;
   d.n = s.n; d.bc1 = s.bc1; d.bc2 = s.bc2;
   d.flags = s.flags & ~kTfUnaligned;
+  // Smallest number of leading elements after which every stream is 16-byte aligned.
   const void* ptrs[6] = {s.p, s.p_out, s.g, s.g_out, s.m, s.v};
-  for (const void* q : ptrs)
-    if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) d.flags |= kTfUnaligned;
-  d.pad = 0;
+  const int sizes[6] = {dtype_size(s.p_dtype), dtype_size(s.p_out_dtype), dtype_size(s.g_dtype),
+                        dtype_size(s.g_out_dtype), 4, 4};
+  uint32_t head = 0;
+  for (; head <= kMaxHead; ++head) {
+    bool ok = true;
+    for (int k = 0; k < 6; ++k)
+      if (ptrs[k] && ((reinterpret_cast<uintptr_t>(ptrs[k]) + (uintptr_t)head * sizes[k]) & 15u)) ok = false;
+    if (ok) break;
+  }
+  if (head > kMaxHead) {  // the streams disagree: per-element path for the whole tensor
+    d.flags |= kTfUnaligned;
+    head = 0;
+  }
+  d.head = head;
+}
+
+uint64_t chunks_of(const DevTensor& d) {
+  if (d.n == 0) return 0;
+  const uint64_t body = d.n > d.head ? d.n - d.head : 0;
+  const uint64_t nc = (body + kChunkElems - 1) / kChunkElems;
+  return nc ? nc : 1;  // a tensor that is all head still needs the workgroup of chunk 0
 }
 
 Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool persistent) {
   Launch L;
   fill_dev_tensor(t, L.one);
-  L.nchunks = (uint32_t)((t.n + kChunkElems - 1) / kChunkElems);
+  L.nchunks = (uint32_t)chunks_of(L.one);
   L.grid = persistent ? persistent_grid(ctx, L.nchunks) : L.nchunks;
   L.stream = ctx->stream;
   L.nontemporal = ctx->nontemporal;
@@ -316,7 +336,7 @@ int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxo
       return fail(ctx, MXOPT_ERR_INVALID_ARG,
                   "mxopt_table_build: tensor " + std::to_string(i) + " has a non-floating dtype code");
     }
-    if (s.n > (uint64_t)0xffffffffu * kChunkElems) {
+    if (s.n > (uint64_t)0xfffffff0u * kChunkElems) {
       delete t;
       return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_build: tensor " + std::to_string(i) + " is too large");
     }
@@ -337,7 +357,7 @@ int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxo
     g.pd = (kv.first >> 24) & 0xff; g.gd = (kv.first >> 16) & 0xff; g.pod = (kv.first >> 8) & 0xff; g.god = kv.first & 0xff;
     g.chunk_begin = (uint32_t)chunks.size();
     for (uint32_t ti : kv.second) {
-      const uint64_t nc = (t->host[ti].n + kChunkElems - 1) / kChunkElems;
+      const uint64_t nc = chunks_of(t->dev[ti]);
       for (uint64_t c = 0; c < nc; ++c) chunks.push_back(DevChunk{ti, (uint32_t)c});
     }
     if (chunks.size() > 0xffffffffull) {

@@ -15,6 +15,7 @@ namespace mxopt {
 constexpr int kChunkElems = MXOPT_CHUNK_ELEMS;
 constexpr uint32_t kTfFirst = MXOPT_TF_FIRST;
 constexpr uint32_t kTfUnaligned = 0x80000000u;  // set by the table builder: element-wise path
+constexpr uint32_t kMaxHead = 7;                // a shifted tensor peels at most this many elements
 
 // One per tensor, in device memory.
 struct DevTensor {
@@ -27,13 +28,17 @@ struct DevTensor {
   uint64_t n;
   float bc1, bc2;
   uint32_t flags;
-  uint32_t pad;
+  // Elements in front of the first chunk.  When every stream of the tensor becomes 16-byte aligned
+  // after the same small number of elements (views into packed slabs), chunk c covers
+  // [head + c*kChunkElems, ...) on the 128-bit path and the workgroup of chunk 0 also handles
+  // elements [0, head) one by one.
+  uint32_t head;
 };
 
 // One per kChunkElems-element slice of a tensor, in device memory.
 struct DevChunk {
   uint32_t tensor;  // index into the DevTensor array
-  uint32_t index;   // chunk number inside that tensor; first element = index * kChunkElems
+  uint32_t index;   // chunk number inside that tensor; first element = head + index * kChunkElems
 };
 
 constexpr uint32_t kPrepPreMul = 1u, kPrepClampPre = 2u, kPrepClampPost = 4u;

@@ -123,7 +123,8 @@ struct ChunkView {
   DevTensor t;
   uint64_t start;  // first element of the chunk inside the tensor
   uint32_t len;    // elements in this chunk (kChunk except for the last one)
-  bool fast;       // full chunk of a 16-byte aligned tensor: 128-bit path, fully unrolled
+  uint32_t head;   // chunk 0 of a shifted tensor: elements [0, head) are this workgroup's too
+  bool fast;       // full chunk of a 16-byte aligned (after the head) tensor: 128-bit path, fully unrolled
 };
 
 __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, const DevChunk* __restrict__ C,
@@ -138,9 +139,10 @@ __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, con
     cv.t = one;
     index = c;
   }
-  cv.start = (uint64_t)index * kChunk;
-  const uint64_t left = cv.t.n - cv.start;
+  cv.start = (uint64_t)cv.t.head + (uint64_t)index * kChunk;
+  const uint64_t left = cv.t.n > cv.start ? cv.t.n - cv.start : 0;
   cv.len = left < (uint64_t)kChunk ? (uint32_t)left : (uint32_t)kChunk;
+  cv.head = index == 0 ? (cv.t.n < (uint64_t)cv.t.head ? (uint32_t)cv.t.n : cv.t.head) : 0u;
   cv.fast = !(cv.t.flags & kTfUnaligned) && cv.len == (uint32_t)kChunk;
   return cv;
 }
@@ -182,6 +184,17 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
     float* M = cv.t.m;
     float* V = cv.t.v;
     const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
+    auto one_element = [&](uint64_t off) {
+      float p = Elem<PD>::load(P, off);
+      float ge = Elem<GD>::load(G, off);
+      if (kHasG2) ge = ge + Elem<G2D>::load(G2P, off);
+      float m = Math::kM ? M[off] : 0.0f;
+      float v = read_v ? V[off] : 0.0f;
+      math(p, prep_all(pr, ge), m, v, bc1, bc2, flags);
+      Elem<OD>::store(PO, off, p);
+      if (Math::kM) M[off] = m;
+      if (use_v) V[off] = v;
+    };
 
     if (cv.fast) {
       // Full chunk: issue every load of the chunk before the first use.
@@ -232,19 +245,9 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
         if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
         if (use_v) store_group<MXOPT_F32, E, false>(V, off, v);
       }
-      for (uint32_t i = ngroups * E + tid; i < len; i += kThreads) {
-        const uint64_t off = start + i;
-        float p = Elem<PD>::load(P, off);
-        float ge = Elem<GD>::load(G, off);
-        if (kHasG2) ge = ge + Elem<G2D>::load(G2P, off);
-        float m = Math::kM ? M[off] : 0.0f;
-        float v = read_v ? V[off] : 0.0f;
-        math(p, prep_all(pr, ge), m, v, bc1, bc2, flags);
-        Elem<OD>::store(PO, off, p);
-        if (Math::kM) M[off] = m;
-        if (use_v) V[off] = v;
-      }
+      for (uint32_t i = ngroups * E + tid; i < len; i += kThreads) one_element(start + i);
     }
+    if (tid < cv.head) one_element(tid);  // elements in front of the first aligned group
   }
 }
 
@@ -288,6 +291,7 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
       for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads)
         Elem<OD>::store(GO, start + i, prep_all(pr, Elem<GD>::load(G, start + i)));
     }
+    if (tid < cv.head) Elem<OD>::store(GO, tid, prep_all(pr, Elem<GD>::load(G, tid)));
   }
 }
 
@@ -379,18 +383,22 @@ struct SumsqChunk {
       }
       if (MODE == 2) store_group<AD, E, false>(A, off, x);
     }
-    for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) {
-      const uint64_t off = cv.start + i;
-      float x = (MODE != 2 || !first) ? Elem<AD>::load(X, off) : 0.0f;
-      if (MODE == 2) {
-        x = accumulate_op<AD, GD>(x, Elem<GD>::load(G, off), first);
-        Elem<AD>::store(A, off, x);
-      }
-      if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(G, off), false);
-      const float y = prep_pre(pr, x);
-      s32 = fmaf(y, y, s32);
-    }
+    for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) s32 = one_element(cv, pr, cv.start + i, first, s32);
     return s32;
+  }
+
+  // Element `off` of the tensor on its own: s32 + its square.
+  static __device__ __forceinline__ float one_element(const ChunkView& cv, const PrepRegs& pr, uint64_t off,
+                                                      bool first, float s32) {
+    const void* X = squared_stream(cv);
+    float x = (MODE != 2 || !first) ? Elem<AD>::load(X, off) : 0.0f;
+    if (MODE == 2) {
+      x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), first);
+      Elem<AD>::store(cv.t.g_out, off, x);
+    }
+    if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), false);
+    const float y = prep_pre(pr, x);
+    return fmaf(y, y, s32);
   }
 };
 
@@ -416,6 +424,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
     } else {
       s = Chunk::slow(cv, pr, tid, first);
     }
+    if (tid < cv.head) s = Chunk::one_element(cv, pr, tid, first, s);
     // A lane's float32 partial covers <= 16 squares of one chunk; chunks are combined in float64.
     // A NaN/Inf element (or squares that overflow float32) makes the partial, and so the total,
     // non-finite: that is the validity check (the reference's sum-based one, grpo/engine.rs:1692-1698).

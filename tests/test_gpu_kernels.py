@@ -515,3 +515,49 @@ def test_skip_step_when_a_gradient_is_not_finite(mx, ctx):
             assert changed != poison, f"tensor {i}"
             assert (to_host(dm[i]) == 0).all() == poison
             assert (to_host(out[i]) == 7.0).all() == poison
+
+
+# ---------------------------------------------------------------------------------
+# Tensors whose streams all start the same number of elements off a 16-byte boundary (views into
+# packed slabs): a few head elements are peeled and the rest takes the 128-bit path.
+# ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shift", [1, 2, 3, 5, 7])
+def test_common_shift_of_all_streams(mx, ctx, shift):
+    import torch
+    sizes = [1, 2, shift, shift + 1, 7, 8, 9, 15, 4096, 4096 + shift, 4097 + shift, 2 * 4096 + shift - 1, 50001]
+    ps, gs = make_lists(70 + shift, sizes=sizes, bf16=True)
+    zeros = [np.zeros(n, F) for n in sizes]
+    dp, dg = [to_dev(p, shift) for p in ps], [to_dev(g, shift) for g in gs]
+    dm, dv, da = ([to_dev(z, shift) for z in zeros] for _ in range(3))
+    for a in da:
+        a.fill_(float("nan"))
+    res = ctx.norm_result()
+    t_acc = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(dg, da)])
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=g, m=m, v=v)
+                       for p, a, g, m, v in zip(dp, da, dg, dm, dv)])
+    ctx.accumulate(t_acc, first=True)
+    ctx.accumulate(t_acc, first=False)
+    ctx.accumulate_norm_only(t_acc, res, max_norm=1e-3)
+    acc2 = [O.accumulate_fp32(O.accumulate_fp32(None, g), g) for g in gs]
+    acc3 = [O.accumulate_fp32(a, g) for a, g in zip(acc2, gs)]
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(da[i]), acc2[i], f"acc {i}")
+    scale = device_scale(ctx, res, acc3, 1e-3)
+    ctx.adam_with_pending(t_upd, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01), mx.make_prep(scale=res))
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    for i in range(len(sizes)):
+        want = O.f32_to_bf16(ref.update_single(str(i), ps[i], acc3[i] * scale))
+        assert_bit_equal(to_host(dp[i]), want, f"p {i} (n={sizes[i]})")
+        assert_bit_equal(to_host(dm[i]), ref.state[str(i)][0], f"m {i}")
+        assert_bit_equal(to_host(dv[i]), ref.state[str(i)][1], f"v {i}")
+    # gradient transform and a separate norm pass over the same views
+    out = [to_dev(z, shift) for z in zeros]
+    t_g = ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(dg, out)])
+    ctx.global_norm(t_g, res, max_norm=1e-3)
+    s2 = device_scale(ctx, res, gs, 1e-3)
+    ctx.grad_transform(t_g, mx.make_prep(scale=res))
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(out[i]), O.bf16_to_f32(gs[i]) * s2, f"scaled g {i}")
+    for t in (t_acc, t_upd, t_g):
+        t.close()

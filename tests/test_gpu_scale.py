@@ -1,12 +1,20 @@
 """Parity at the full sizes of the benchmark configurations.
 
 * Qwen3-0.6B list, float32 AdamW (config 1): EVERY element of parameters and moments, two steps,
-  bit for bit against the C twin of the oracle.
+  bit for bit against the C twin of the oracle -- once with the reference's default (no bias
+  correction) through the kernel-level table, once bias-corrected through the optimizer object, where
+  tensor i of step s must see t = s*N + i + 1 (the reference counts update_single calls).
+* Qwen3-1.7B list, bf16 parameters and gradients with 1 % x100 outliers, clip 1.0 (config 2) and the
+  Qwen3-4B list, float32 SGD with momentum / RMSprop (config 3): every tensor of at most 1 Mi elements in
+  full plus seeded windows (head, tail, interior) of every larger one, two steps, bit for bit; the
+  global norm of every step against a float64 reduction done by torch on the device (a library routine
+  that is not the reference) at rel 1e-5.
+* 10,000 small bf16 tensors (config 4): EVERY element, three steps, packed back to back so that most
+  tensors start at an address that is only 2-byte aligned, and separately allocated.
 * Qwen3-8B list, bf16 parameters / float32 moments, 4 micro-batches into a float32 buffer, clip 1.0,
   last micro-batch folded into the update (config 5, ~131 GB resident): seeded windows of every stream
   are read back before and after the step and pushed through the NumPy oracle (bit-exact given the
-  device's clip factor); the global norm is checked against a float64 reduction done by torch on the
-  device (a library routine that is not the reference) at rel 1e-5.
+  device's clip factor); norm as above.
 """
 import math
 
@@ -22,6 +30,10 @@ from gpu_util import to_host
 F = np.float32
 
 
+def f32(x):
+    return float(np.float32(x))
+
+
 def carve(torch, sizes, dtype, align=256):
     offs, total = [], 0
     for n in sizes:
@@ -31,11 +43,57 @@ def carve(torch, sizes, dtype, align=256):
     return slab, offs, [slab[o:o + n] for o, n in zip(offs, sizes)]
 
 
+def qwen_sizes(model):
+    from mxopt.qwen3_shapes import QWEN3, numel, param_list
+    plist = param_list(QWEN3[model])
+    return [name for name, _ in plist], [numel(s) for _, s in plist]
+
+
+def window_index(torch, sizes, offs, seed, small=1 << 20, W=16384, interior=3):
+    """Flat slab indices: all of every tensor <= `small` elements; head, tail and `interior` seeded
+    windows (odd starts, so not group aligned) of every larger one."""
+    rng = np.random.default_rng(seed)
+    pieces = []
+    for o, n in zip(offs, sizes):
+        if n <= small:
+            pieces.append(np.arange(o, o + n))
+            continue
+        pieces.append(np.arange(o, o + W))
+        pieces.append(np.arange(o + n - W, o + n))
+        for s in rng.integers(0, n - W, interior):
+            s = int(s) // 8 * 8 + 3
+            pieces.append(np.arange(o + s, min(o + s + W, o + n)))
+    return torch.from_numpy(np.concatenate(pieces)).cuda()
+
+
+def device_sumsq_f64(torch, tensors):
+    return sum(float(t.double().square().sum()) for t in tensors)
+
+
+def check_norm(r, ref_sumsq, max_norm=1.0):
+    """rel 1e-5 on the norm; the clip factor is the reference's scalar chain applied to the device's sum."""
+    assert abs(r.norm - math.sqrt(ref_sumsq)) <= 1e-5 * math.sqrt(ref_sumsq)
+    n32, scale = O.norm_scale_c1(r.sumsq, max_norm)
+    assert F(r.scale) == scale and F(r.norm_f32) == n32 and r.nonfinite == 0
+    return float(scale)
+
+
+def same_bits(got, want, what):
+    got, want = np.ascontiguousarray(got), np.ascontiguousarray(want)
+    assert got.dtype == want.dtype and got.shape == want.shape, what
+    v = np.uint32 if got.dtype == np.float32 else np.uint16
+    bad = got.view(v) != want.view(v)
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.size} differ, first at {int(np.flatnonzero(bad)[0])}"
+
+
+# ---------------------------------------------------------------------------------------
+# config 1
+# ---------------------------------------------------------------------------------------
+
 def test_config1_full_list_every_element(oracle_c):
     import torch
     import mxopt as mx
-    from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    sizes = [numel(s) for _, s in param_list(QWEN3["0.6B"])]
+    _, sizes = qwen_sizes("0.6B")
     n = sum(sizes)
     assert n == 596_049_920 and len(sizes) == 310
     gen = torch.Generator().manual_seed(0x5EED0001)
@@ -64,11 +122,206 @@ def test_config1_full_list_every_element(oracle_c):
     ctx.close()
 
 
+def test_config1_bias_corrected_per_call_step_count(oracle_c):
+    import torch
+    import mxopt as mx
+    names, sizes = qwen_sizes("0.6B")
+    n, nt = sum(sizes), len(sizes)
+    gen = torch.Generator().manual_seed(0x5EED0011)
+    p_ref = torch.empty(n).normal_(0, 0.02, generator=gen).numpy()
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    dp = [torch.from_numpy(p_ref[offs[i]:offs[i + 1]]).cuda() for i in range(nt)]
+    dg = [torch.empty(s, device="cuda") for s in sizes]
+    ctx = mx.Context()
+    opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True, ctx=ctx)
+    m_ref, v_ref = np.zeros(n, F), np.zeros(n, F)
+    for step in range(2):
+        g_h = torch.empty(n).normal_(0, 1e-3, generator=gen)
+        for i, g in enumerate(dg):
+            g.copy_(g_h[offs[i]:offs[i + 1]])
+        opt.update_many(names, dp, dg, outs=dp)                      # in place, one launch
+        g_np = g_h.numpy()
+        new_p = np.empty(n, F)
+        for i in range(nt):
+            t = float(step * nt + i + 1)                             # adam.rs:73: one count per call
+            a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01, bc1=1.0 / (1.0 - math.pow(0.9, t)),
+                            bc2=1.0 / (1.0 - math.pow(0.999, t)), bias_correction=True)
+            s = slice(offs[i], offs[i + 1])
+            new_p[s] = oracle_c.adam(p_ref[s], g_np[s], m_ref[s], v_ref[s], a, fused=True)
+        p_ref = new_p
+        assert opt.step == (step + 1) * nt
+        same_bits(torch.cat(dp).cpu().numpy(), p_ref, f"p step {step}")
+    for i in (0, 1, 5, nt // 2, nt - 1):                              # moments live inside the object
+        m, v = opt.state(names[i])
+        same_bits(m.cpu().numpy(), m_ref[offs[i]:offs[i + 1]], f"m {names[i]}")
+        same_bits(v.cpu().numpy(), v_ref[offs[i]:offs[i + 1]], f"v {names[i]}")
+    del opt
+    ctx.close()
+
+
+# ---------------------------------------------------------------------------------------
+# config 2
+# ---------------------------------------------------------------------------------------
+
+def test_config2_full_size_outliers_clip_windows(oracle_c):
+    import torch
+    import mxopt as mx
+    _, sizes = qwen_sizes("1.7B")
+    n = sum(sizes)
+    assert n == 1_720_574_976 and len(sizes) == 310
+    torch.manual_seed(0x5EED0002)
+    bf = torch.bfloat16
+    p_slab, offs, dp = carve(torch, sizes, bf)
+    g_slab, _, dg = carve(torch, sizes, bf)
+    m_slab, _, dm = carve(torch, sizes, torch.float32)
+    v_slab, _, dv = carve(torch, sizes, torch.float32)
+    p_slab.normal_(0, 0.02)
+    m_slab.zero_()
+    v_slab.zero_()
+    idx = window_index(torch, sizes, offs, seed=2)
+    win = lambda slab: to_host(slab[idx])
+    ctx = mx.Context()
+    t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
+    hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
+    res = ctx.norm_result()
+    p_ref, m_ref, v_ref = win(p_slab), win(m_slab), win(v_slab)
+    for step in range(2):
+        g_slab.normal_(0, 1e-3)
+        for lo in range(0, g_slab.numel(), 1 << 28):                # 1 % of the elements x100, in pieces
+            piece = g_slab[lo:lo + (1 << 28)]
+            piece.mul_(torch.where(torch.rand(piece.shape, device="cuda") < 0.01, 100.0, 1.0).to(bf))
+        ctx.global_norm(t_g, res, max_norm=1.0)
+        ctx.adam(t_upd, hp, mx.make_prep(scale=res))
+        r = ctx.read_norm_result(res)
+        scale = check_norm(r, device_sumsq_f64(torch, dg))
+        expected = 1e-3 * math.sqrt(n * (0.99 + 0.01 * 1e4))         # ~417: the clip is active
+        assert abs(r.norm - expected) < 0.02 * expected and scale < 0.01
+        args = B.adam_args(5e-6, 0.9, 0.999, 1e-8, 0.01, scale=scale)
+        p_ref = oracle_c.f32_to_bf16(oracle_c.adam(p_ref, win(g_slab), m_ref, v_ref, args, fused=True))
+        same_bits(win(p_slab), p_ref, f"p step {step}")
+        same_bits(win(m_slab), m_ref, f"m step {step}")
+        same_bits(win(v_slab), v_ref, f"v step {step}")
+    t_g.close()
+    t_upd.close()
+    ctx.close()
+
+
+# ---------------------------------------------------------------------------------------
+# config 3
+# ---------------------------------------------------------------------------------------
+
+def test_config3_full_size_sgd_and_rmsprop_windows(oracle_c):
+    import torch
+    import mxopt as mx
+    _, sizes = qwen_sizes("4B")
+    n = sum(sizes)
+    assert n == 4_022_468_096 and len(sizes) == 398
+    torch.manual_seed(0x5EED0003)
+    p_slab, offs, dp = carve(torch, sizes, torch.float32)
+    g_slab, _, dg = carve(torch, sizes, torch.float32)
+    v_slab, _, dv = carve(torch, sizes, torch.float32)
+    p_slab.normal_(0, 0.02)
+    idx = window_index(torch, sizes, offs, seed=3)
+    win = lambda slab: to_host(slab[idx])
+    ctx = mx.Context()
+
+    # SGD, momentum 0.9, dampening 0, weight decay 1e-4: step 1 takes the velocity-less branch
+    v_slab.fill_(float("nan"))                                        # must not be read on the first step
+    table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v, flags=mx.TF_FIRST) for p, g, v in zip(dp, dg, dv)])
+    hp = mx.sgd_hp(1e-4, 0.9, 1e-4, 0.0, False)
+    p_ref, v_ref = win(p_slab), np.zeros(idx.numel(), F)
+    for step in range(3):
+        g_slab.normal_(0, 1e-3)
+        if step == 1:
+            table.set_step_scalars(flags=[0] * len(sizes))
+        ctx.sgd(table, hp)
+        args = B.SgdArgs(lr=f32(1e-4), momentum=f32(0.9), one_minus_damp=f32(1.0), wd=f32(1e-4), has_wd=1,
+                         has_momentum=1, nesterov=0, first=int(step == 0))
+        p_ref = oracle_c.sgd(p_ref, win(g_slab), v_ref, args, fused=True)
+        same_bits(win(p_slab), p_ref, f"sgd p step {step}")
+        same_bits(win(v_slab), v_ref, f"sgd v step {step}")
+    table.close()
+
+    # RMSprop, alpha 0.99, eps 1e-8, lr 1e-4
+    v_slab.zero_()
+    table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v) for p, g, v in zip(dp, dg, dv)])
+    hp = mx.rmsprop_hp(1e-4, 0.99, 1e-8, 0.0)
+    p_ref, v_ref = win(p_slab), np.zeros(idx.numel(), F)
+    for step in range(2):
+        g_slab.normal_(0, 1e-3)
+        ctx.rmsprop(table, hp)
+        args = B.RmspropArgs(lr=f32(1e-4), alpha=f32(0.99), one_minus_alpha=f32(1.0 - 0.99), eps=f32(1e-8),
+                             wd=0.0, has_wd=0)
+        p_ref = oracle_c.rmsprop(p_ref, win(g_slab), v_ref, args, fused=True)
+        same_bits(win(p_slab), p_ref, f"rmsprop p step {step}")
+        same_bits(win(v_slab), v_ref, f"rmsprop v step {step}")
+    table.close()
+    ctx.close()
+
+
+# ---------------------------------------------------------------------------------------
+# config 4
+# ---------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("alloc", ["packed", "separate"])
+def test_config4_ten_thousand_small_tensors_every_element(oracle_c, alloc):
+    import torch
+    import mxopt as mx
+    rng = np.random.default_rng(0x5EED0001)
+    sizes = np.floor(np.exp(rng.uniform(np.log(64), np.log(65536), 10000))).astype(np.int64).tolist()
+    n = int(sum(sizes))
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    bf = torch.bfloat16
+    torch.manual_seed(0x5EED0004)
+
+    def make(dtype):
+        if alloc == "packed":        # back to back: tensor i starts offs[i] elements into the slab
+            slab = torch.empty(n, dtype=dtype, device="cuda")
+            return [slab[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+        return [torch.empty(s, dtype=dtype, device="cuda") for s in sizes]
+
+    dp, dg, dm, dv = make(bf), make(bf), make(torch.float32), make(torch.float32)
+    if alloc == "packed":
+        assert sum(1 for p in dp if p.data_ptr() % 16) > 8000         # most heads are not 16-byte aligned
+    for p, m, v in zip(dp, dm, dv):
+        p.uniform_(0.9, 1.1)
+        m.zero_()
+        v.zero_()
+    flat = lambda ts: to_host(torch.cat(ts))
+    ctx = mx.Context()
+    t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
+    hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.0)
+    res = ctx.norm_result()
+    p_ref, m_ref, v_ref = flat(dp), np.zeros(n, F), np.zeros(n, F)
+    for step in range(3):
+        for g in dg:
+            g.normal_(0, 1e-2)
+        ctx.global_norm(t_g, res, max_norm=1.0)
+        ctx.adam(t_upd, hp, mx.make_prep(scale=res))
+        r = ctx.read_norm_result(res)
+        g_h = flat(dg)
+        scale = check_norm(r, oracle_c.sumsq(g_h))                    # exact float64 sum on the host
+        assert scale < 0.02                                           # norm ~ 1e-2 * sqrt(n) ~ 97: clip active
+        args = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.0, scale=scale)
+        p_ref = oracle_c.f32_to_bf16(oracle_c.adam(p_ref, g_h, m_ref, v_ref, args, fused=True))
+        same_bits(flat(dp), p_ref, f"p step {step}")
+        same_bits(flat(dm), m_ref, f"m step {step}")
+        same_bits(flat(dv), v_ref, f"v step {step}")
+    t_g.close()
+    t_upd.close()
+    ctx.close()
+
+
+# ---------------------------------------------------------------------------------------
+# config 5
+# ---------------------------------------------------------------------------------------
+
 def test_config5_full_size_windows_and_norm():
     import torch
     import mxopt as mx
-    from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    sizes = [numel(s) for _, s in param_list(QWEN3["8B"])]
+    _, sizes = qwen_sizes("8B")
     n = sum(sizes)
     assert n == 8_190_735_360 and len(sizes) == 399
     free, _ = torch.cuda.mem_get_info()
