@@ -69,8 +69,9 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
 /* ---- tensor table ------------------------------------------------------------------
  * One descriptor per tensor.  Which fields a kernel reads is listed at that kernel;
  * unused pointers may be NULL.  All buffers are dense, `n` elements long.
- * Buffers need only their natural alignment; tensors whose used pointers are all
- * 16-byte aligned take the 128-bit path, others an element-wise path. */
+ * Buffers need only their natural alignment.  A tensor whose used pointers all become
+ * 16-byte aligned after the same number (0..7) of leading elements takes the 128-bit
+ * path (those leading elements are handled one by one); others an element-wise path. */
 typedef struct mxopt_tensor {
   const void* p;     /* parameter, read                                             */
   void*       p_out; /* parameter, written; may equal p (in place)                  */
@@ -97,6 +98,11 @@ void mxopt_table_destroy(mxopt_table* t);
 uint64_t mxopt_table_total_elems(const mxopt_table* t);
 uint64_t mxopt_table_num_chunks(const mxopt_table* t);
 uint64_t mxopt_table_num_tensors(const mxopt_table* t);
+/* Host-only query (no device needed, pointers are not dereferenced): how the table builder
+ * lays out one tensor.  *head = leading elements handled one by one (0..7), *vector_path = 1
+ * when the rest takes the 128-bit path, *num_chunks = table entries (workgroups of work).
+ * Any out pointer may be NULL.  No counterpart in the reference (MLX picks its own kernels). */
+int mxopt_tensor_layout(const mxopt_tensor* t, uint32_t* head, int* vector_path, uint64_t* num_chunks);
 #define MXOPT_CHUNK_ELEMS 4096 /* elements one workgroup handles per table entry */
 
 /* ---- device-resident result of the global-norm reduction ------------------------ */

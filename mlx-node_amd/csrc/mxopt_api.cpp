@@ -431,6 +431,16 @@ void mxopt_table_destroy(mxopt_table* t) {
   delete t;
 }
 
+int mxopt_tensor_layout(const mxopt_tensor* t, uint32_t* head, int* vector_path, uint64_t* num_chunks) {
+  if (!t) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_tensor_layout: null tensor");
+  DevTensor d;
+  fill_dev_tensor(*t, d);
+  if (head) *head = d.head;
+  if (vector_path) *vector_path = (d.flags & kTfUnaligned) ? 0 : 1;
+  if (num_chunks) *num_chunks = chunks_of(d);
+  return MXOPT_OK;
+}
+
 uint64_t mxopt_table_total_elems(const mxopt_table* t) { return t ? t->total_elems : 0; }
 uint64_t mxopt_table_num_chunks(const mxopt_table* t) { return t ? t->num_chunks : 0; }
 uint64_t mxopt_table_num_tensors(const mxopt_table* t) { return t ? t->host.size() : 0; }

@@ -123,3 +123,36 @@ def test_product_does_not_import_the_oracle():
             if fn.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, fn), errors="replace").read()
                 assert "oracle" not in text.lower(), f"{fn} mentions the oracle"
+
+
+def test_tensor_layout_head_and_chunk_count(L):
+    """Host logic of the table builder: the common head that aligns every stream, the chunk count,
+    and the per-element fallback when the streams disagree (pointers are never dereferenced)."""
+    lib = L.load()
+    BASE = 0x7f0000000000
+
+    def layout(n, p=None, g=None, m=None, v=None, p_dt=L.BF16, g_dt=L.BF16):
+        t = L.Tensor(p=p, p_out=p, g=g, g_out=None, m=m, v=v, n=n, p_dtype=p_dt, p_out_dtype=p_dt, g_dtype=g_dt,
+                     g_out_dtype=0, flags=0, bc1=1.0, bc2=1.0)
+        head, vec, nc = C.c_uint32(), C.c_int(), C.c_uint64()
+        assert lib.mxopt_tensor_layout(C.byref(t), C.byref(head), C.byref(vec), C.byref(nc)) == 0
+        return head.value, vec.value, nc.value
+
+    assert layout(4096, p=BASE, g=BASE + 4096 * 2, m=BASE + 65536, v=BASE + 131072) == (0, 1, 1)
+    assert layout(4097, p=BASE, g=BASE) == (0, 1, 2)
+    assert layout(0, p=BASE + 2, g=BASE + 2) == (7, 1, 0)
+    # the same element offset k into packed bf16 and float32 slabs: head = (8 - k) % 8
+    for k in range(1, 16):
+        h = (8 - k) % 8
+        got = layout(10000, p=BASE + 2 * k, g=BASE + (1 << 20) + 2 * k, m=BASE + (2 << 20) + 4 * k,
+                     v=BASE + (3 << 20) + 4 * k)
+        assert got == (h, 1, (10000 - h + 4095) // 4096), (k, got)
+    # float32 only: the smallest head is k-dependent modulo 4
+    assert layout(100, p=BASE + 4, g=BASE + 20, p_dt=L.F32, g_dt=L.F32) == (3, 1, 1)
+    # fewer elements than the head: one entry, all of it head
+    assert layout(3, p=BASE + 2, g=BASE + 2) == (7, 1, 1)
+    assert layout(7 + 4096, p=BASE + 2, g=BASE + 2) == (7, 1, 1)
+    assert layout(7 + 4097, p=BASE + 2, g=BASE + 2) == (7, 1, 2)
+    # streams that disagree: bf16 p one element in, float32 m on a boundary
+    assert layout(5000, p=BASE + 2, g=BASE + 2, m=BASE + 65536, v=BASE + 131072) == (0, 0, 2)
+    assert lib.mxopt_tensor_layout(None, None, None, None) == 1
