@@ -22,6 +22,12 @@
  * Threading: calls on one context are serialised by the caller; different contexts
  * may be used from different threads.  Kernels are enqueued on the context's stream;
  * no call synchronises with the host except mxopt_synchronize / mxopt_read_*.
+ *
+ * HIP graphs: the kernel entry points (mxopt_adam ... mxopt_accumulate_norm_only) only launch
+ * kernels -- no allocation, copy or memset -- once the first reduction call on a context has
+ * allocated its per-workgroup partials buffer, so a step may be recorded into a graph after
+ * one eager warm-up call.  mxopt_table_build and mxopt_table_set_step_scalars copy from host
+ * memory and stay outside a capture.
  */
 #ifndef MXOPT_H
 #define MXOPT_H
