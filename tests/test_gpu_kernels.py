@@ -561,3 +561,43 @@ def test_common_shift_of_all_streams(mx, ctx, shift):
         assert_bit_equal(to_host(out[i]), O.bf16_to_f32(gs[i]) * s2, f"scaled g {i}")
     for t in (t_acc, t_upd, t_g):
         t.close()
+
+
+# ---------------------------------------------------------------------------------
+# One table, several dtype combinations: one launch per group, one norm over all of them
+# ---------------------------------------------------------------------------------
+
+def test_mixed_dtype_table(mx, ctx):
+    import torch
+    rng = np.random.default_rng(404)
+    sizes = [100003, 4096, 7, 0, 12289, 4097, 64, 9000]
+    kinds = ["f32/f32", "bf16/bf16", "bf16/f32", "f32/bf16", "bf16/bf16", "f32/f32", "bf16/f32", "f32/bf16"]
+    ps, gs = [], []
+    for n, k in zip(sizes, kinds):
+        p = rng.normal(0, 0.02, n).astype(F)
+        g = rng.normal(0, 1e-3, n).astype(F)
+        pk, gk = k.split("/")
+        ps.append(O.f32_to_bf16(p) if pk == "bf16" else p)
+        gs.append(O.f32_to_bf16(g) if gk == "bf16" else g)
+    dp, dg = [to_dev(p) for p in ps], [to_dev(g) for g in gs]
+    dm = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in sizes]
+    dv = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in sizes]
+    res = ctx.norm_result()
+    t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
+    assert t_upd.total_elems == sum(sizes)
+    hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    cur = list(ps)
+    for it in range(2):
+        ctx.global_norm(t_g, res, max_norm=1e-2)
+        scale = device_scale(ctx, res, gs, 1e-2)
+        ctx.adam(t_upd, hp, mx.make_prep(scale=res))
+        for i in range(len(sizes)):
+            r = ref.update_single(str(i), cur[i], O.as_f32(gs[i]) * scale)
+            cur[i] = O.f32_to_bf16(r) if cur[i].dtype == np.uint16 else r
+            assert_bit_equal(to_host(dp[i]), cur[i], f"p{i} ({kinds[i]}) it {it}")
+            assert_bit_equal(to_host(dm[i]), ref.state[str(i)][0], f"m{i} it {it}")
+            assert_bit_equal(to_host(dv[i]), ref.state[str(i)][1], f"v{i} it {it}")
+    t_g.close()
+    t_upd.close()
