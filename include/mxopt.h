@@ -118,8 +118,9 @@ typedef struct mxopt_norm_result {
   float    norm_f32;  /* (float)norm: what clip_grad_norm_with_norm returns          */
   float    scale;     /* clip factor, see mxopt_clip_mode                           */
   uint64_t nonfinite; /* 1 when the sum of squares is not finite (a NaN/Inf element, or
-                         squares beyond float32 range), else 0: the reference's sum-based
-                         validity check (grpo/engine.rs:1692-1698)                   */
+                         squares beyond float32 range) or when prep's clamp_pre met a raw
+                         +-Inf (which the clamp would have hidden), else 0: the engines'
+                         validity checks (grpo/engine.rs:563-569, :1692-1698)          */
 } mxopt_norm_result;
 
 /* How `scale` is derived from the norm. */
@@ -243,6 +244,13 @@ int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxop
  * Pair with mxopt_adam_with_pending. */
 int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep, double max_norm,
                                int clip_mode, mxopt_norm_result* d_result);
+
+/* g_out = first ? prep(g) : g_out + prep(g): the engines' per-micro-batch "clamp, clip by norm,
+ * then accumulate" (grpo/engine.rs:636-661, :1737-1754) without materialising the clipped
+ * gradient.  prep(g) is float32 (clip and the scale multiply promote); the sum is one float32
+ * add, rounded once to dtype(g_out).  Honours prep->d_skip_if_nonzero: a micro-batch flagged
+ * non-finite by mxopt_global_norm leaves the buffer untouched (grpo/engine.rs:561-562). */
+int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep);
 
 /* ---- small host<->device helpers (each synchronises the context's stream) --------- */
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out);

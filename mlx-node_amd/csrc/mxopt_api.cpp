@@ -550,7 +550,16 @@ int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_
   if (rc) return rc;
   const DevPrep dp = make_prep(prep);
   return run_update(ctx, t, "mxopt_grad_transform",
-                    [&](const Group& g, const Launch& L) { return launch_transform(g.gd, g.god, L, dp); });
+                    [&](const Group& g, const Launch& L) { return launch_transform(g.gd, g.god, L, dp, 0); });
+}
+
+int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_accumulate_transformed");
+  if (rc) return rc;
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_accumulate_transformed", [&](const Group& g, const Launch& L) {
+    return launch_transform(g.gd, g.god, L, dp, first ? 0 : 1);
+  });
 }
 
 int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep, double max_norm,

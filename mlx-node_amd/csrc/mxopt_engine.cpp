@@ -1,0 +1,501 @@
+// The optimizer side of the training engines: bookkeeping on the host, arithmetic in the kernels.
+// Declarations, and the reference lines each entry point stands behind, are in
+// include/mxopt_engine.h.
+#include "mxopt_engine.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "mxopt_internal.h"
+
+using namespace mxopt;
+
+namespace {
+
+struct Slot {
+  std::string name;
+  mxopt_array param{};
+  void* acc = nullptr;  // accumulation buffer, allocated on first use, reused by every cycle
+  int acc_dtype = -1;
+  bool in_acc = false;  // holds a value in the current accumulation cycle
+};
+
+int dtype_bytes(int dt) { return dt == MXOPT_F32 ? 4 : 2; }
+
+}  // namespace
+
+struct mxopt_engine {
+  mxopt_ctx* ctx = nullptr;
+  mxopt_engine_config cfg{};
+  std::vector<Slot> slots;
+  std::unordered_map<std::string, size_t> index;
+  mxopt_optimizer* adamw = nullptr;       // APPLY_ADAMW: moments by parameter name
+  mxopt_norm_result* d_result = nullptr;  // device slot of the norm pass
+  // EngineState (grpo/engine.rs:227-271, sft/engine.rs:114-145), optimizer-side fields
+  bool have_acc = false;
+  int32_t micro_step = 0;
+  int64_t step = 0;
+  uint64_t nan_gradient_count = 0;
+  uint32_t consecutive_nan_count = 0;
+  bool needs_emergency_save = false;
+};
+
+namespace {
+
+int32_t acc_steps(const mxopt_engine* e) {
+  return e->cfg.gradient_accumulation_steps < 1 ? 1 : e->cfg.gradient_accumulation_steps;
+}
+uint64_t max_nan(const mxopt_engine* e) {
+  return e->cfg.max_nan_gradients < 1 ? 100u : (uint64_t)e->cfg.max_nan_gradients;
+}
+uint32_t emergency_threshold(const mxopt_engine* e) {
+  return e->cfg.emergency_save_threshold < 1 ? 5u : (uint32_t)e->cfg.emergency_save_threshold;
+}
+
+void fill_metrics(const mxopt_engine* e, mxopt_engine_metrics* m, int applied, int skipped) {
+  if (!m) return;
+  std::memset(m, 0, sizeof *m);
+  m->step = e->step;
+  m->micro_step = e->micro_step;
+  m->gradients_applied = applied;
+  m->skipped = skipped;
+  m->needs_emergency_save = e->needs_emergency_save ? 1 : 0;
+  m->consecutive_nan_count = e->consecutive_nan_count;
+  m->nan_gradient_count = e->nan_gradient_count;
+  m->grad_sumsq = m->grad_norm = NAN;
+  m->clip_scale = 1.0f;
+}
+
+void add_norm(mxopt_engine_metrics* m, const mxopt_norm_result& h) {
+  if (!m) return;
+  m->norm_measured = 1;
+  m->grad_sumsq = h.sumsq;
+  m->grad_norm = h.norm;
+  m->clip_scale = h.scale;
+}
+
+int ensure_acc(mxopt_engine* e, Slot& s, int dtype) {
+  if (s.acc && s.acc_dtype == dtype) return MXOPT_OK;
+  DeviceGuard guard(e->ctx->device);
+  if (s.acc) {
+    HIP_TRY(e->ctx, hipStreamSynchronize(e->ctx->stream));
+    (void)hipFree(s.acc);
+    s.acc = nullptr;
+  }
+  if (s.param.n) HIP_TRY(e->ctx, hipMalloc(&s.acc, s.param.n * (size_t)dtype_bytes(dtype)));
+  s.acc_dtype = dtype;
+  return MXOPT_OK;
+}
+
+// Checks names and sizes; on success idx[i] is the slot of gradient i.
+int resolve(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads, std::vector<size_t>* idx) {
+  mxopt_ctx* ctx = e->ctx;
+  if (n && (!names || !grads)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "engine: null names or gradients");
+  idx->resize(n);
+  for (size_t i = 0; i < n; ++i) {
+    if (!names[i]) return fail(ctx, MXOPT_ERR_INVALID_ARG, "engine: null gradient name");
+    auto it = e->index.find(names[i]);
+    if (it == e->index.end())  // models/qwen3/model.rs:2427-2432
+      return fail(ctx, MXOPT_ERR_FAILURE, std::string("Parameter '") + names[i] + "' not found in model");
+    int rc = check_array(ctx, &grads[i], "engine: gradient");
+    if (rc) return rc;
+    if (grads[i].n != e->slots[it->second].param.n)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("engine: gradient '") + names[i] + "' has the wrong size");
+    (*idx)[i] = it->second;
+  }
+  return MXOPT_OK;
+}
+
+mxopt_grad_prep no_prep() {
+  mxopt_grad_prep p;
+  std::memset(&p, 0, sizeof p);
+  return p;
+}
+
+// The parameter update over every slot that holds an accumulated value.  `prep` turns the
+// accumulated sum into the gradient that is applied.
+int apply_accumulated(mxopt_engine* e, double lr, double weight_decay, const mxopt_grad_prep& prep) {
+  mxopt_ctx* ctx = e->ctx;
+  std::vector<mxopt_tensor> rows;
+  std::vector<const char*> names;
+  std::vector<mxopt_array> params, grads;
+  for (Slot& s : e->slots) {
+    if (!s.in_acc) continue;
+    if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {
+      names.push_back(s.name.c_str());
+      params.push_back(s.param);
+      grads.push_back(mxopt_array{s.acc, s.param.n, s.acc_dtype});
+    } else {
+      mxopt_tensor r = blank_tensor();
+      r.p = s.param.data; r.p_out = s.param.data;
+      r.p_dtype = r.p_out_dtype = (uint8_t)s.param.dtype;
+      r.g = s.acc; r.g_dtype = (uint8_t)s.acc_dtype;
+      r.n = s.param.n;
+      rows.push_back(r);
+    }
+  }
+  if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {
+    if (names.empty()) return MXOPT_OK;
+    return mxopt_optimizer_update_many(e->adamw, names.size(), names.data(), params.data(), grads.data(),
+                                       params.data(), &prep);
+  }
+  if (rows.empty()) return MXOPT_OK;
+  mxopt_table* t = nullptr;
+  int rc = cached_table(ctx, rows, &t);
+  if (rc) return rc;
+  return mxopt_sgd_plain(ctx, t, lr, weight_decay, &prep);
+}
+
+void end_cycle(mxopt_engine* e) {
+  for (Slot& s : e->slots) s.in_acc = false;
+  e->have_acc = false;
+  e->micro_step = 0;
+}
+
+// ---- GRPO: grpo/engine.rs:561-704 ------------------------------------------------------
+
+int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_array* grads,
+                     mxopt_engine_metrics* out) {
+  mxopt_ctx* ctx = e->ctx;
+  const size_t n = idx.size();
+  const double clip_value = e->cfg.has_gradient_clip_value ? e->cfg.gradient_clip_value : 1.0;  // engine.rs:636
+  mxopt_grad_prep prep = no_prep();
+  prep.has_clamp_pre = 1;
+  prep.pre_lo = (float)(-clip_value);
+  prep.pre_hi = (float)clip_value;
+  mxopt_norm_result h;
+  std::memset(&h, 0, sizeof h);
+  h.scale = 1.0f;
+  int rc;
+  if (n) {
+    // One read of the gradients: validity of the raw values and the norm of the clamped ones.
+    std::vector<mxopt_tensor> rows(n, blank_tensor());
+    for (size_t i = 0; i < n; ++i) {
+      rows[i].g = grads[i].data; rows[i].g_dtype = (uint8_t)grads[i].dtype; rows[i].n = grads[i].n;
+    }
+    mxopt_table* t = nullptr;
+    if ((rc = cached_table(ctx, rows, &t))) return rc;
+    const double max_norm = e->cfg.has_gradient_clip_norm ? e->cfg.gradient_clip_norm : -1.0;
+    if ((rc = mxopt_global_norm(ctx, t, 0, &prep, max_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, e->d_result))) return rc;
+    if ((rc = mxopt_read_norm_result(ctx, e->d_result, &h))) return rc;
+  }
+  if (h.nonfinite) {  // engine.rs:571-633: skip the whole micro-batch, touch nothing
+    e->nan_gradient_count += 1;
+    e->consecutive_nan_count += 1;
+    if (e->nan_gradient_count >= max_nan(e)) {
+      fill_metrics(e, out, 0, 1);
+      return fail(ctx, MXOPT_ERR_FAILURE,
+                  "Training stopped: exceeded maximum NaN gradient count (" + std::to_string(e->nan_gradient_count) +
+                      "/" + std::to_string(max_nan(e)) + ")");
+    }
+    if (e->consecutive_nan_count >= emergency_threshold(e)) e->needs_emergency_save = true;
+    e->step += 1;
+    fill_metrics(e, out, 0, 1);
+    return MXOPT_OK;
+  }
+  e->consecutive_nan_count = 0;  // engine.rs:660
+
+  // acc (+)= clip_norm(clamp(g)) in float32 (engine.rs:636-661, :2632-2666)
+  if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result->scale;
+  std::vector<mxopt_tensor> first_rows, add_rows;
+  for (size_t i = 0; i < n; ++i) {
+    Slot& s = e->slots[idx[i]];
+    if ((rc = ensure_acc(e, s, MXOPT_F32))) return rc;
+    mxopt_tensor r = blank_tensor();
+    r.g = grads[i].data; r.g_dtype = (uint8_t)grads[i].dtype;
+    r.g_out = s.acc; r.g_out_dtype = MXOPT_F32;
+    r.n = grads[i].n;
+    (s.in_acc ? add_rows : first_rows).push_back(r);
+    s.in_acc = true;
+  }
+  for (int pass = 0; pass < 2; ++pass) {
+    std::vector<mxopt_tensor>& rows = pass == 0 ? first_rows : add_rows;
+    if (rows.empty()) continue;
+    mxopt_table* t = nullptr;
+    if ((rc = cached_table(ctx, rows, &t))) return rc;
+    if ((rc = mxopt_accumulate_transformed(ctx, t, pass == 0, &prep))) return rc;
+  }
+  e->have_acc = true;
+  e->micro_step += 1;
+
+  int applied = 0;
+  const int32_t N = acc_steps(e);
+  if (e->micro_step >= N) {  // engine.rs:666-692
+    mxopt_grad_prep ap = no_prep();
+    if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {
+      ap.has_pre_mul = 1;
+      ap.pre_mul = (float)(1.0 / (double)N);
+      rc = apply_accumulated(e, e->cfg.learning_rate, 0.0, ap);
+    } else {
+      rc = apply_accumulated(e, e->cfg.learning_rate / (double)N, 0.0, ap);  // engine.rs:672
+    }
+    if (rc) return rc;
+    end_cycle(e);
+    applied = 1;
+  }
+  e->step += 1;  // engine.rs:690, :696
+  fill_metrics(e, out, applied, 0);
+  if (n) add_norm(out, h);
+  return MXOPT_OK;
+}
+
+// ---- SFT: sft/engine.rs:268-371, :459-553 ------------------------------------------------
+
+// Average by `count`, clip by norm, clamp, decay, update (sft/engine.rs:293-371).  `norm_ready`:
+// *d_result already describes acc/count.
+int sft_apply(mxopt_engine* e, int32_t count, bool norm_ready, mxopt_engine_metrics* out, mxopt_norm_result* h_out,
+              bool* measured) {
+  mxopt_ctx* ctx = e->ctx;
+  mxopt_grad_prep prep = no_prep();
+  prep.has_pre_mul = 1;
+  prep.pre_mul = (float)(1.0 / (double)count);  // mul_scalar(scale): float64, then one cast
+  int rc;
+  *measured = false;
+  if (e->cfg.has_gradient_clip_norm) {
+    if (!norm_ready) {
+      std::vector<mxopt_tensor> rows;
+      for (Slot& s : e->slots) {
+        if (!s.in_acc) continue;
+        mxopt_tensor r = blank_tensor();
+        r.g_out = s.acc; r.g_out_dtype = (uint8_t)s.acc_dtype; r.n = s.param.n;
+        rows.push_back(r);
+      }
+      if (!rows.empty()) {
+        mxopt_table* t = nullptr;
+        if ((rc = cached_table(ctx, rows, &t))) return rc;
+        if ((rc = mxopt_global_norm(ctx, t, 1, &prep, e->cfg.gradient_clip_norm, MXOPT_CLIP_ALWAYS_MULTIPLY,
+                                    e->d_result)))
+          return rc;
+        norm_ready = true;
+      }
+    }
+    if (norm_ready) {
+      prep.d_scale = &e->d_result->scale;
+      if (out) {  // only a caller that wants the figures pays for the read-back
+        if ((rc = mxopt_read_norm_result(ctx, e->d_result, h_out))) return rc;
+        *measured = true;
+      }
+    }
+  }
+  if (e->cfg.has_gradient_clip_value) {
+    prep.has_clamp_post = 1;
+    prep.post_lo = (float)(-e->cfg.gradient_clip_value);
+    prep.post_hi = (float)e->cfg.gradient_clip_value;
+  }
+  if ((rc = apply_accumulated(e, e->cfg.learning_rate, e->cfg.weight_decay, prep))) return rc;
+  end_cycle(e);
+  e->step += 1;
+  return MXOPT_OK;
+}
+
+int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_array* grads,
+                    mxopt_engine_metrics* out) {
+  mxopt_ctx* ctx = e->ctx;
+  const size_t n = idx.size();
+  e->consecutive_nan_count = 0;  // sft/engine.rs:261-267
+  const bool first_cycle_step = !e->have_acc;
+  std::vector<mxopt_tensor> rows;
+  int rc;
+  size_t held = 0;
+  for (const Slot& s : e->slots) held += s.in_acc ? 1 : 0;
+  for (size_t i = 0; i < n; ++i) {
+    Slot& s = e->slots[idx[i]];
+    if (!first_cycle_step && !s.in_acc) continue;  // sft/engine.rs:283-287: silently dropped
+    const int want = e->cfg.accumulate_in_f32 ? MXOPT_F32 : grads[i].dtype;
+    if (first_cycle_step) {
+      if (s.in_acc) continue;  // the same name twice in one call: the map keeps one
+      if ((rc = ensure_acc(e, s, want))) return rc;
+      s.in_acc = true;
+    } else if (s.acc_dtype != want && !(s.acc_dtype == MXOPT_F32)) {
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  "engine: gradient '" + s.name + "' changed dtype inside an accumulation cycle");
+    }
+    mxopt_tensor r = blank_tensor();
+    r.g = grads[i].data; r.g_dtype = (uint8_t)grads[i].dtype;
+    r.g_out = s.acc; r.g_out_dtype = (uint8_t)s.acc_dtype;
+    r.n = grads[i].n;
+    rows.push_back(r);
+  }
+  if (first_cycle_step) held = rows.size();
+  const int32_t N = acc_steps(e);
+  const bool boundary = e->micro_step + 1 >= N;
+  // The norm of acc/N rides on the last accumulation pass when that pass touches every held tensor.
+  const bool fuse_norm = boundary && e->cfg.has_gradient_clip_norm && !rows.empty() && rows.size() == held;
+  if (!rows.empty()) {
+    mxopt_table* t = nullptr;
+    if ((rc = cached_table(ctx, rows, &t))) return rc;
+    mxopt_grad_prep prep = no_prep();
+    prep.has_pre_mul = 1;
+    prep.pre_mul = (float)(1.0 / (double)N);
+    rc = mxopt_accumulate(ctx, t, first_cycle_step ? 1 : 0, fuse_norm ? &prep : nullptr,
+                          fuse_norm ? e->cfg.gradient_clip_norm : -1.0, MXOPT_CLIP_ALWAYS_MULTIPLY,
+                          fuse_norm ? e->d_result : nullptr);
+    if (rc) return rc;
+  }
+  e->have_acc = true;  // Some(map), possibly empty
+  e->micro_step += 1;
+  int applied = 0;
+  mxopt_norm_result h;
+  bool measured = false;
+  if (boundary) {
+    if ((rc = sft_apply(e, N, fuse_norm, out, &h, &measured))) return rc;
+    applied = 1;
+  }
+  fill_metrics(e, out, applied, 0);
+  if (measured) add_norm(out, h);
+  return MXOPT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+void mxopt_engine_config_default(int32_t kind, mxopt_engine_config* c) {
+  if (!c) return;
+  std::memset(c, 0, sizeof *c);
+  c->kind = kind;
+  c->gradient_accumulation_steps = 1;
+  c->has_gradient_clip_norm = 1;
+  c->gradient_clip_norm = 1.0;
+  c->max_nan_gradients = 100;
+  c->emergency_save_threshold = 5;
+  c->apply = MXOPT_ENGINE_APPLY_SGD;
+  c->beta1 = 0.9; c->beta2 = 0.999; c->eps = 1e-8;
+  if (kind == MXOPT_ENGINE_SFT) {  // sft/engine.rs:50-66
+    c->learning_rate = 2e-5;
+    c->weight_decay = 0.01;
+  } else {                         // grpo/engine.rs:114-141
+    c->learning_rate = 1e-6;
+    c->has_gradient_clip_value = 1;
+    c->gradient_clip_value = 1.0;
+  }
+}
+
+int mxopt_engine_new(mxopt_ctx* ctx, const mxopt_engine_config* config, size_t n, const char* const* names,
+                     const mxopt_array* params, mxopt_engine** out) {
+  if (!ctx || !config || !out || (n && (!names || !params)))
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: null argument");
+  *out = nullptr;
+  if (config->kind != MXOPT_ENGINE_GRPO && config->kind != MXOPT_ENGINE_SFT)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: unknown engine kind");
+  if (config->apply != MXOPT_ENGINE_APPLY_SGD && config->apply != MXOPT_ENGINE_APPLY_ADAMW)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: unknown apply mode");
+  mxopt_engine* e = new (std::nothrow) mxopt_engine();
+  if (!e) return fail(ctx, MXOPT_ERR_OOM, "mxopt_engine_new: out of host memory");
+  e->ctx = ctx;
+  e->cfg = *config;
+  e->slots.resize(n);
+  for (size_t i = 0; i < n; ++i) {
+    int rc = names[i] ? check_array(ctx, &params[i], "mxopt_engine_new: parameter")
+                      : fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: null parameter name");
+    if (!rc && !e->index.emplace(names[i], i).second)
+      rc = fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("mxopt_engine_new: duplicate parameter '") + names[i] + "'");
+    if (rc) {
+      delete e;
+      return rc;
+    }
+    e->slots[i].name = names[i];
+    e->slots[i].param = params[i];
+  }
+  int rc = MXOPT_OK;
+  {
+    DeviceGuard guard(ctx->device);
+    hipError_t err = hipMalloc((void**)&e->d_result, sizeof(mxopt_norm_result));
+    if (err != hipSuccess) rc = hip_fail(ctx, err, "mxopt_engine_new: hipMalloc");
+  }
+  if (!rc && config->apply == MXOPT_ENGINE_APPLY_ADAMW) {
+    const int no_bias_correction = 0;  // the reference's default (adamw.rs:57)
+    rc = mxopt_adamw_new(ctx, &config->learning_rate, &config->beta1, &config->beta2, &config->eps,
+                         &config->weight_decay, &no_bias_correction, &e->adamw);
+  }
+  if (rc) {
+    mxopt_engine_free(e);
+    return rc;
+  }
+  *out = e;
+  return MXOPT_OK;
+}
+
+void mxopt_engine_free(mxopt_engine* e) {
+  if (!e) return;
+  DeviceGuard guard(e->ctx->device);
+  (void)hipStreamSynchronize(e->ctx->stream);
+  for (Slot& s : e->slots)
+    if (s.acc) (void)hipFree(s.acc);
+  if (e->d_result) (void)hipFree(e->d_result);
+  if (e->adamw) mxopt_optimizer_free(e->adamw);
+  delete e;
+}
+
+int mxopt_engine_micro_batch(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads,
+                             mxopt_engine_metrics* out) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_micro_batch: null engine");
+  std::vector<size_t> idx;
+  int rc = resolve(e, n, names, grads, &idx);
+  if (rc) return rc;
+  return e->cfg.kind == MXOPT_ENGINE_GRPO ? grpo_micro_batch(e, idx, grads, out) : sft_micro_batch(e, idx, grads, out);
+}
+
+int mxopt_engine_flush_gradients(mxopt_engine* e, int* flushed, mxopt_engine_metrics* out) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_flush_gradients: null engine");
+  if (e->cfg.kind != MXOPT_ENGINE_SFT)
+    return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_flush_gradients: only the SFT engine flushes");
+  if (flushed) *flushed = 0;
+  if (e->micro_step == 0 || !e->have_acc) {  // sft/engine.rs:469-472
+    fill_metrics(e, out, 0, 0);
+    return MXOPT_OK;
+  }
+  mxopt_norm_result h;
+  bool measured = false;
+  int rc = sft_apply(e, e->micro_step, false, out, &h, &measured);
+  if (rc) return rc;
+  if (flushed) *flushed = 1;
+  fill_metrics(e, out, 1, 0);
+  if (measured) add_norm(out, h);
+  return MXOPT_OK;
+}
+
+int mxopt_engine_report_nonfinite_loss(mxopt_engine* e, mxopt_engine_metrics* out) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_report_nonfinite_loss: null engine");
+  e->nan_gradient_count += 1;
+  e->consecutive_nan_count += 1;
+  if (e->consecutive_nan_count >= emergency_threshold(e)) e->needs_emergency_save = true;  // sft/engine.rs:228-235
+  fill_metrics(e, out, 0, 1);
+  if (e->nan_gradient_count >= max_nan(e))                                                  // sft/engine.rs:237-243
+    return fail(e->ctx, MXOPT_ERR_FAILURE,
+                "Training stopped: exceeded " + std::to_string(max_nan(e)) + " NaN gradient limit");
+  return MXOPT_OK;
+}
+
+int mxopt_engine_get_metrics(const mxopt_engine* e, mxopt_engine_metrics* out) {
+  if (!e || !out) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_get_metrics: null argument");
+  fill_metrics(e, out, 0, 0);
+  return MXOPT_OK;
+}
+
+int mxopt_engine_clear_emergency_save_flag(mxopt_engine* e) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_clear_emergency_save_flag: null engine");
+  e->needs_emergency_save = false;
+  return MXOPT_OK;
+}
+
+int mxopt_engine_reset(mxopt_engine* e) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_reset: null engine");
+  for (Slot& s : e->slots) s.in_acc = false;
+  e->have_acc = false;
+  e->micro_step = 0;
+  e->step = 0;
+  e->nan_gradient_count = 0;
+  e->consecutive_nan_count = 0;
+  e->needs_emergency_save = false;
+  if (e->adamw) return mxopt_optimizer_reset(e->adamw);
+  return MXOPT_OK;
+}
+
+}  // extern "C"

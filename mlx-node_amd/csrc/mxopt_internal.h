@@ -4,8 +4,10 @@
 #include <hip/hip_runtime_api.h>
 
 #include <string>
+#include <vector>
 
 #include "mxopt.h"
+#include "mxopt_optimizers.h"
 #include "mxopt_host_types.h"
 #include "mxopt_launch.h"
 
@@ -45,5 +47,14 @@ void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d);
 uint64_t chunks_of(const DevTensor& d);  // chunk-table entries (= workgroups of work) of one tensor
 // A launch over the single tensor `t` (descriptor passed in the kernel arguments).
 Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool persistent);
+
+
+// Shared by the host-layer translation units (mxopt_optimizers.cpp, mxopt_engine.cpp).
+mxopt_tensor blank_tensor();  // all pointers NULL, bc1 = bc2 = 1
+int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, bool allow_null_data = false);
+// Finds or builds the table for `rows` (compared bytewise, per-step scalars excluded); the context
+// keeps the most recently used few.
+int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** out);
+int norm_scratch(mxopt_ctx* ctx, mxopt_norm_result** out);
 
 }  // namespace mxopt

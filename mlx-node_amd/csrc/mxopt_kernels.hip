@@ -255,10 +255,13 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 // Gradient transform: g_out = prep(g)
 // ------------------------------------------------------------------------------------
 
+// add != 0: g_out = g_out + prep(g) (one float32 add, rounded to g_out's dtype by the store): the
+// engines' "clamp, clip-norm, then accumulate" (grpo/engine.rs:636-661) without materialising the
+// clipped gradient.
 template <int GD, int OD, bool NT>
 __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __restrict__ T,
                                                              const DevChunk* __restrict__ C, DevTensor one,
-                                                             uint32_t nchunks, DevPrep prep) {
+                                                             uint32_t nchunks, DevPrep prep, int add) {
   constexpr int E = (GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
   if (skip_requested(prep)) return;
@@ -269,29 +272,44 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
     const uint64_t start = cv.start;
     const void* G = cv.t.g;
     void* GO = cv.t.g_out;
+    auto one_element = [&](uint64_t off) {
+      float t = prep_all(pr, Elem<GD>::load(G, off));
+      if (add) t = Elem<OD>::load(GO, off) + t;
+      Elem<OD>::store(GO, off, t);
+    };
     if (cv.fast) {
-      float g[U][E];
+      float g[U][E], a[U][E];
 #pragma unroll
-      for (int j = 0; j < U; ++j) load_group<GD, E, NT>(G, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
+        load_group<GD, E, NT>(G, off, g[j]);
+        if (add) load_group<OD, E, NT>(GO, off, a[j]);
+      }
 #pragma unroll
       for (int j = 0; j < U; ++j) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) g[j][e] = prep_all(pr, g[j][e]);
+        for (int e = 0; e < E; ++e) {
+          g[j][e] = prep_all(pr, g[j][e]);
+          if (add) g[j][e] = a[j][e] + g[j][e];
+        }
         store_group<OD, E, NT>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
       }
     } else {
       const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
       for (uint32_t q = tid; q < ngroups; q += kThreads) {
-        float g[E];
+        float g[E], a[E];
         load_group<GD, E, false>(G, start + (uint64_t)q * E, g);
+        if (add) load_group<OD, E, false>(GO, start + (uint64_t)q * E, a);
 #pragma unroll
-        for (int e = 0; e < E; ++e) g[e] = prep_all(pr, g[e]);
+        for (int e = 0; e < E; ++e) {
+          g[e] = prep_all(pr, g[e]);
+          if (add) g[e] = a[e] + g[e];
+        }
         store_group<OD, E, false>(GO, start + (uint64_t)q * E, g);
       }
-      for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads)
-        Elem<OD>::store(GO, start + i, prep_all(pr, Elem<GD>::load(G, start + i)));
+      for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) one_element(start + i);
     }
-    if (tid < cv.head) Elem<OD>::store(GO, tid, prep_all(pr, Elem<GD>::load(G, tid)));
+    if (tid < cv.head) one_element(tid);
   }
 }
 
@@ -304,6 +322,10 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
 //   MODE 3: square (g_out + g) without storing it (the update kernel adds g again itself)
 // AD: dtype of the stream that is squared / accumulated into; GD: dtype of g (MODE 2, 3).
 // ------------------------------------------------------------------------------------
+
+// A value clamp would turn +-Inf into a finite bound and hide it from the sum-based validity
+// check; the engines test the raw values (grpo/engine.rs:563-569), so such a lane poisons its partial.
+__device__ __forceinline__ bool is_inf(float x) { return __builtin_isinf(x); }
 
 template <int AD, int GD>
 __device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
@@ -343,18 +365,21 @@ struct SumsqChunk {
   // Returns this lane's float32 sum of squares over the chunk; stores the new sum in MODE 2.
   __device__ __forceinline__ float finish(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
     float s32 = 0.0f;
+    const bool clamped = (pr.flags & kPrepClampPre) != 0;
+    bool hidden_inf = false;
 #pragma unroll
     for (int j = 0; j < U; ++j) {
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
         if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
+        if (clamped) hidden_inf |= is_inf(x[j][e]);
         const float y = prep_pre(pr, x[j][e]);
         s32 = fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
     }
-    return s32;
+    return hidden_inf ? __builtin_nanf("") : s32;
   }
 
   // Partial or unaligned chunk.
@@ -363,6 +388,7 @@ struct SumsqChunk {
     const void* G = cv.t.g;
     void* A = cv.t.g_out;
     float s32 = 0.0f;
+    const bool clamped = (pr.flags & kPrepClampPre) != 0;
     const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
     for (uint32_t q = tid; q < ngroups; q += kThreads) {
       const uint64_t off = cv.start + (uint64_t)q * E;
@@ -379,7 +405,7 @@ struct SumsqChunk {
         if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
         if (MODE == 3) x[e] = accumulate_op<AD, GD>(x[e], g[e], false);
         const float y = prep_pre(pr, x[e]);
-        s32 = fmaf(y, y, s32);
+        s32 = (clamped && is_inf(x[e])) ? __builtin_nanf("") : fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, false>(A, off, x);
     }
@@ -398,6 +424,7 @@ struct SumsqChunk {
     }
     if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), false);
     const float y = prep_pre(pr, x);
+    if ((pr.flags & kPrepClampPre) && is_inf(x)) return __builtin_nanf("");
     return fmaf(y, y, s32);
   }
 };
@@ -577,25 +604,25 @@ bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float
 }
 
 template <int GD>
-static bool transform_for_gd(int od, const Launch& L, const DevPrep& prep) {
+static bool transform_for_gd(int od, const Launch& L, const DevPrep& prep, int add) {
   if (od == MXOPT_F32) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, true>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, false>), L, prep);
+    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, true>), L, prep, add);
+    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, false>), L, prep, add);
     return true;
   }
   if (od == GD) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, GD, true>), L, prep);
-    else MXOPT_LAUNCH((transform_kernel<GD, GD, false>), L, prep);
+    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, GD, true>), L, prep, add);
+    else MXOPT_LAUNCH((transform_kernel<GD, GD, false>), L, prep, add);
     return true;
   }
   return false;
 }
 
-bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep) {
+bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep, int add) {
   switch (gd) {
-    case MXOPT_F32: return transform_for_gd<MXOPT_F32>(od, L, prep);
-    case MXOPT_BF16: return transform_for_gd<MXOPT_BF16>(od, L, prep);
-    case MXOPT_F16: return transform_for_gd<MXOPT_F16>(od, L, prep);
+    case MXOPT_F32: return transform_for_gd<MXOPT_F32>(od, L, prep, add);
+    case MXOPT_BF16: return transform_for_gd<MXOPT_BF16>(od, L, prep, add);
+    case MXOPT_F16: return transform_for_gd<MXOPT_F16>(od, L, prep, add);
   }
   return false;
 }

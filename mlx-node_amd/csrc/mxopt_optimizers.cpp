@@ -25,14 +25,14 @@ struct StateEntry {
 
 enum class Kind { Adam, AdamW, Sgd, Rmsprop };
 
-static mxopt_tensor blank_tensor() {
+mxopt_tensor blank_tensor() {
   mxopt_tensor t;
   std::memset(&t, 0, sizeof t);
   t.bc1 = t.bc2 = 1.0f;
   return t;
 }
 
-static int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, bool allow_null_data = false) {
+int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, bool allow_null_data) {
   if (!a) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(what) + " is NULL");
   if (!float_dtype(a->dtype)) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(what) + ": unsupported dtype code");
   if (!a->data && a->n && !allow_null_data)
@@ -41,7 +41,7 @@ static int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, b
 }
 
 // Finds or builds the table for `rows` (compared bytewise, per-step scalars excluded).
-static int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** out) {
+int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** out) {
   std::vector<mxopt_tensor> key = rows;
   for (auto& r : key) { r.bc1 = r.bc2 = 1.0f; r.flags = 0; }
   auto& cache = ctx->table_cache;
@@ -68,7 +68,7 @@ static int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_t
   return MXOPT_OK;
 }
 
-static int norm_scratch(mxopt_ctx* ctx, mxopt_norm_result** out) {
+int norm_scratch(mxopt_ctx* ctx, mxopt_norm_result** out) {
   if (!ctx->d_norm_scratch) {
     DeviceGuard guard(ctx->device);
     HIP_TRY(ctx, hipMalloc((void**)&ctx->d_norm_scratch, sizeof(mxopt_norm_result)));
@@ -515,7 +515,7 @@ static int clamp_arrays(mxopt_ctx* ctx, size_t n, const mxopt_array* grads, doub
     if (rows[0].n == 0) return MXOPT_OK;
     DeviceGuard guard(ctx->device);
     const Launch L = make_single_launch(ctx, rows[0], ctx->persistent != 0);
-    if (!launch_transform(rows[0].g_dtype, rows[0].g_out_dtype, L, make_prep(&prep)))
+    if (!launch_transform(rows[0].g_dtype, rows[0].g_out_dtype, L, make_prep(&prep), 0))
       return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes");
     return check_launch(ctx, op);
   }

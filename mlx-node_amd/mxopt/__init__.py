@@ -7,5 +7,6 @@ from .core import (Context, NormResultBuffer, Table, TensorSpec, adam_hp, bias_c
 from .optimizers import (SGD, Adam, AdamW, GradientAccumulator, GradientUtils, LRScheduler, RMSprop,
                          accumulate_gradients, apply_gradients, clip_gradients_by_global_norm,
                          clip_gradients_by_value, default_context)
+from .engine import GRPOEngineOptimizerSide, SFTEngineOptimizerSide, TrainingStopped
 
 load()

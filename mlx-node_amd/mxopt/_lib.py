@@ -93,6 +93,7 @@ SIGNATURES = {
     "mxopt_global_norm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
                                     C.c_void_p]),
     "mxopt_grad_transform": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep)]),
+    "mxopt_accumulate_transformed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep)]),
     "mxopt_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
                                    C.c_void_p]),
     "mxopt_accumulate_norm_only": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
@@ -144,6 +145,44 @@ SIGNATURES.update({
 
 _lib = None
 
+
+
+class EngineConfig(C.Structure):
+    """mxopt_engine_config (include/mxopt_engine.h)."""
+    _fields_ = [("kind", C.c_int32), ("gradient_accumulation_steps", C.c_int32), ("learning_rate", C.c_double),
+                ("has_gradient_clip_norm", C.c_int32), ("gradient_clip_norm", C.c_double),
+                ("has_gradient_clip_value", C.c_int32), ("gradient_clip_value", C.c_double),
+                ("weight_decay", C.c_double), ("max_nan_gradients", C.c_int64),
+                ("emergency_save_threshold", C.c_int32), ("apply", C.c_int32),
+                ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
+                ("accumulate_in_f32", C.c_int32)]
+
+
+class EngineMetrics(C.Structure):
+    """mxopt_engine_metrics (include/mxopt_engine.h)."""
+    _fields_ = [("step", C.c_int64), ("micro_step", C.c_int32), ("gradients_applied", C.c_int32),
+                ("skipped", C.c_int32), ("needs_emergency_save", C.c_int32), ("consecutive_nan_count", C.c_uint32),
+                ("nan_gradient_count", C.c_uint64), ("norm_measured", C.c_int32), ("clip_scale", C.c_float),
+                ("grad_sumsq", C.c_double), ("grad_norm", C.c_double)]
+
+
+ENGINE_GRPO, ENGINE_SFT = 0, 1
+ENGINE_APPLY_SGD, ENGINE_APPLY_ADAMW = 0, 1
+_PM = C.POINTER(EngineMetrics)
+
+# every symbol declared in include/mxopt_engine.h
+SIGNATURES.update({
+    "mxopt_engine_config_default": (None, [C.c_int32, C.POINTER(EngineConfig)]),
+    "mxopt_engine_new": (C.c_int, [C.c_void_p, C.POINTER(EngineConfig), C.c_size_t, C.POINTER(C.c_char_p), _PA,
+                                   C.POINTER(C.c_void_p)]),
+    "mxopt_engine_free": (None, [C.c_void_p]),
+    "mxopt_engine_micro_batch": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA, _PM]),
+    "mxopt_engine_flush_gradients": (C.c_int, [C.c_void_p, _PI, _PM]),
+    "mxopt_engine_report_nonfinite_loss": (C.c_int, [C.c_void_p, _PM]),
+    "mxopt_engine_get_metrics": (C.c_int, [C.c_void_p, _PM]),
+    "mxopt_engine_clear_emergency_save_flag": (C.c_int, [C.c_void_p]),
+    "mxopt_engine_reset": (C.c_int, [C.c_void_p]),
+})
 
 def load() -> C.CDLL:
     global _lib

@@ -192,6 +192,11 @@ class Context:
                                           max_norm, clip_mode, C.c_void_p(out.ptr) if out else None), self.handle)
 
 
+def _accumulate_transformed(self, table: "Table", first: bool, prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_accumulate_transformed(self.handle, table.handle, int(first),
+                                                  C.byref(prep) if prep else None), self.handle)
+
+
 def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Optional[L.GradPrep] = None,
                           max_norm: float = -1.0, clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
     L.check(self.lib.mxopt_accumulate_norm_only(self.handle, table.handle, C.byref(prep) if prep else None,
@@ -199,6 +204,7 @@ def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Opt
 
 
 Context.accumulate_norm_only = _accumulate_norm_only
+Context.accumulate_transformed = _accumulate_transformed
 
 
 class Table:

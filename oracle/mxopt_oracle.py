@@ -38,7 +38,15 @@ PARITY UNPINNED (no reference test, fixture or buildable reference covers it):
   exact float64 sum, rounded once);
 * NaN handling of ``clip`` (NaN is propagated here);
 * the per-call ``step`` quirk, Nesterov's stored state and the
-  ``(m/(sqrt(v)+eps))*lr`` association are pinned only by reading the source.
+  ``(m/(sqrt(v)+eps))*lr`` association are pinned only by reading the source;
+* the engines' optimizer-side state machines (GRPOEngineOptimizerSide,
+  SFTEngineOptimizerSide: skip-on-NaN counters, emergency flag, step counting,
+  flush): no reference test exercises them; their arithmetic is a composition of
+  the pinned functions above (the lr/N and accumulate-then-apply identities are
+  the reference's own known answers, grpo-gradient-accumulation.test.ts:48-68,134-171),
+  their bookkeeping is pinned only by reading the source;
+* the ``apply="adamw"`` mode of those two classes has no counterpart in the
+  reference at all (it is this build's fused replacement for apply_gradients).
 """
 from __future__ import annotations
 
@@ -413,6 +421,201 @@ def apply_gradients(params: Dict[str, np.ndarray], gradients: Dict[str, np.ndarr
         else:
             out[name] = as_f32(p) - lr32 * as_f32(g)
     return out
+
+
+# --------------------------------------------------------------------------
+# The optimizer side of the training engines (what runs between the backward pass and the
+# next forward pass): grpo/engine.rs:561-704 (and :1691-1790), sft/engine.rs:215-371, :459-553
+# --------------------------------------------------------------------------
+
+class TrainingStopped(RuntimeError):
+    """Error::new(Status::GenericFailure, "Training stopped: exceeded ...") of both engines."""
+
+
+def _has_invalid(g: np.ndarray) -> bool:
+    """grpo/engine.rs:563-569: any NaN or Inf element of the float32 read-back."""
+    return not bool(np.isfinite(as_f32(g)).all())
+
+
+class _EngineState:
+    """EngineState (grpo/engine.rs:227-271, sft/engine.rs:114-145), optimizer-side fields only."""
+
+    def __init__(self):
+        self.accumulated: Optional[Dict[str, np.ndarray]] = None
+        self.micro_step = 0
+        self.step = 0
+        self.nan_gradient_count = 0
+        self.consecutive_nan_count = 0
+        self.needs_emergency_save = False
+
+
+class _EngineBase:
+    def __init__(self, params: Dict[str, np.ndarray], learning_rate, gradient_accumulation_steps,
+                 gradient_clip_norm, gradient_clip_value, weight_decay, max_nan_gradients,
+                 emergency_save_threshold, apply, beta1, beta2, eps):
+        self.params = dict(params)
+        self.learning_rate = learning_rate
+        self.n_acc = 1 if gradient_accumulation_steps is None else int(gradient_accumulation_steps)
+        self.clip_norm = gradient_clip_norm
+        self.clip_value = gradient_clip_value
+        self.weight_decay = weight_decay
+        self.max_nan = 100 if max_nan_gradients is None else int(max_nan_gradients)
+        self.emergency_threshold = 5 if emergency_save_threshold is None else int(emergency_save_threshold)
+        self.apply = apply
+        self.adamw = AdamW(learning_rate, beta1, beta2, eps, weight_decay) if apply == "adamw" else None
+        self.state = _EngineState()
+
+    # getters of both engines (grpo/engine.rs:2460-2600, sft/engine.rs:590-625)
+    @property
+    def step(self): return self.state.step
+    @property
+    def micro_step(self): return self.state.micro_step
+    @property
+    def nan_gradient_count(self): return self.state.nan_gradient_count
+    @property
+    def needs_emergency_save(self): return self.state.needs_emergency_save
+
+    def clear_emergency_save_flag(self) -> None:
+        self.state.needs_emergency_save = False
+
+    def reset(self) -> None:
+        """grpo/engine.rs:2533-2546, sft/engine.rs:671-: *state = EngineState::default()."""
+        self.state = _EngineState()
+
+    def _adamw_apply(self, grads: Dict[str, np.ndarray]) -> None:
+        """This build's replacement for apply_gradients: AdamW on the prepared gradient, parameter
+        written back in its own dtype with one round-to-nearest-even."""
+        for name, g in grads.items():
+            if name not in self.params:
+                raise KeyError(f"Parameter '{name}' not found in model")
+            p = self.params[name]
+            new_p = self.adamw.update_single(name, p, g)
+            self.params[name] = f32_to_bf16(new_p) if is_bf16(p) else new_p
+
+
+class GRPOEngineOptimizerSide(_EngineBase):
+    """GRPOTrainingEngine, everything after the backward pass of one micro-batch
+    (grpo/engine.rs:561-704; :1691-1790 is the same arithmetic through clip_grad_value_and_norm).
+    ``gradient_clip_norm=None`` means no norm clipping (the config default is Some(1.0));
+    ``gradient_clip_value=None`` means 1.0 (engine.rs:636)."""
+
+    def __init__(self, params, learning_rate: Optional[float] = None, gradient_accumulation_steps: Optional[int] = None,
+                 gradient_clip_norm: Optional[float] = 1.0, gradient_clip_value: Optional[float] = None,
+                 max_nan_gradients: Optional[int] = None, emergency_save_threshold: Optional[int] = None,
+                 apply: str = "sgd", weight_decay: float = 0.01, beta1: float = 0.9, beta2: float = 0.999,
+                 eps: float = 1e-8):
+        super().__init__(params, 1e-6 if learning_rate is None else learning_rate, gradient_accumulation_steps,
+                         gradient_clip_norm, 1.0 if gradient_clip_value is None else gradient_clip_value,
+                         weight_decay, max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps)
+
+    def micro_batch(self, gradients: Dict[str, np.ndarray], norm_sumsq: Optional[float] = None) -> Dict[str, object]:
+        """One micro-batch of gradients.  ``norm_sumsq``: use this sum of squares of the clamped
+        gradients in place of the exact one (a checker passes the device's own value, which it has
+        compared with the exact one, so that the comparison downstream can be bit for bit)."""
+        st = self.state
+        # Step 1 (engine.rs:561-633): any NaN/Inf anywhere => skip the whole micro-batch
+        if any(_has_invalid(g) for g in gradients.values()):
+            st.nan_gradient_count += 1
+            st.consecutive_nan_count += 1
+            if st.nan_gradient_count >= self.max_nan:                          # engine.rs:588-596
+                raise TrainingStopped(f"Training stopped: exceeded maximum NaN gradient count "
+                                      f"({st.nan_gradient_count}/{self.max_nan})")
+            if st.consecutive_nan_count >= self.emergency_threshold:           # engine.rs:599-606
+                st.needs_emergency_save = True
+            st.step += 1                                                       # engine.rs:608
+            return {"step": st.step, "gradients_applied": False, "skipped": True}
+        # Step 2 (engine.rs:636-644): clamp; Step 3 (:647-653): clip by global norm of the clamped values
+        clamped = {k: clip_value(g, -self.clip_value, self.clip_value) for k, g in gradients.items()}
+        if self.clip_norm is not None:
+            sumsq = exact_sumsq(clamped.values()) if norm_sumsq is None else norm_sumsq
+            _, scale = norm_scale_c1(sumsq, self.clip_norm)
+            grads = {k: g * scale for k, g in clamped.items()}
+        else:
+            grads = clamped
+        st.consecutive_nan_count = 0                                           # engine.rs:660
+        # engine.rs:2632-2666
+        if st.accumulated is None:
+            st.accumulated = dict(grads)
+        else:
+            for name, g in grads.items():
+                st.accumulated[name] = _add_promoted(st.accumulated[name], g) if name in st.accumulated else g
+        st.micro_step += 1
+        applied = False
+        if st.micro_step >= self.n_acc:                                        # engine.rs:666-692
+            acc, st.accumulated = st.accumulated, None
+            if self.apply == "adamw":
+                self._adamw_apply({k: mul_scalar(g, 1.0 / self.n_acc) for k, g in acc.items()})
+            else:
+                self.params.update(apply_gradients(self.params, acc, self.learning_rate / self.n_acc))
+            st.micro_step = 0
+            applied = True
+        st.step += 1                                                           # engine.rs:690, :696
+        return {"step": st.step, "gradients_applied": applied, "skipped": False}
+
+
+class SFTEngineOptimizerSide(_EngineBase):
+    """SftTrainingEngine, everything after the backward pass of one micro-batch
+    (sft/engine.rs:268-371) plus flush_gradients (:459-553) and the NaN-loss bookkeeping
+    (:221-258).  ``gradient_clip_norm=None`` / ``gradient_clip_value=None`` mean "not configured"."""
+
+    def __init__(self, params, learning_rate: Optional[float] = None, gradient_accumulation_steps: Optional[int] = None,
+                 gradient_clip_norm: Optional[float] = 1.0, gradient_clip_value: Optional[float] = None,
+                 weight_decay: Optional[float] = None, max_nan_gradients: Optional[int] = None,
+                 emergency_save_threshold: Optional[int] = None, apply: str = "sgd", beta1: float = 0.9,
+                 beta2: float = 0.999, eps: float = 1e-8):
+        super().__init__(params, 2e-5 if learning_rate is None else learning_rate, gradient_accumulation_steps,
+                         gradient_clip_norm, gradient_clip_value, 0.0 if weight_decay is None else weight_decay,
+                         max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps)
+
+    def report_nonfinite_loss(self) -> int:
+        """sft/engine.rs:221-258: the loss was NaN/Inf, nothing is accumulated."""
+        st = self.state
+        st.nan_gradient_count += 1
+        st.consecutive_nan_count += 1
+        if st.consecutive_nan_count >= self.emergency_threshold:
+            st.needs_emergency_save = True
+        if st.nan_gradient_count >= self.max_nan:
+            raise TrainingStopped(f"Training stopped: exceeded {self.max_nan} NaN gradient limit")
+        return st.step
+
+    def micro_batch(self, gradients: Dict[str, np.ndarray], norm_sumsq: Optional[float] = None) -> Dict[str, object]:
+        st = self.state
+        st.consecutive_nan_count = 0                                           # sft/engine.rs:261-267
+        st.accumulated = accumulate_gradients_sft(st.accumulated, gradients)   # :282-290
+        st.micro_step += 1
+        applied = False
+        if st.micro_step >= self.n_acc:
+            self._apply(self.n_acc, norm_sumsq)
+            applied = True
+        return {"step": st.step, "gradients_applied": applied, "skipped": False}
+
+    def flush_gradients(self, norm_sumsq: Optional[float] = None) -> bool:
+        """sft/engine.rs:459-553: leftover micro-batches are averaged by their actual count."""
+        st = self.state
+        if st.micro_step == 0 or st.accumulated is None:
+            return False
+        self._apply(st.micro_step, norm_sumsq)
+        return True
+
+    def _apply(self, count: int, norm_sumsq: Optional[float]) -> None:
+        st = self.state
+        acc, st.accumulated = st.accumulated, None
+        averaged = {k: mul_scalar(g, 1.0 / count) for k, g in acc.items()}     # :297-305
+        if self.clip_norm is not None:                                         # :308-314
+            sumsq = exact_sumsq(averaged.values()) if norm_sumsq is None else norm_sumsq
+            _, scale = norm_scale_c1(sumsq, self.clip_norm)
+            averaged = {k: g * scale for k, g in averaged.items()}
+        if self.clip_value is not None:                                        # :317-329
+            averaged = {k: clip_value(g, -self.clip_value, self.clip_value) for k, g in averaged.items()}
+        if self.apply == "adamw":
+            self._adamw_apply(averaged)                                        # decoupled decay inside AdamW
+        else:
+            if self.weight_decay > 0.0:                                        # :345-365
+                averaged = {k: (g + mul_scalar(self.params[k], self.weight_decay)) if k in self.params else g
+                            for k, g in averaged.items()}
+            self.params.update(apply_gradients(self.params, averaged, self.learning_rate))
+        st.step += 1
+        st.micro_step = 0
 
 
 # --------------------------------------------------------------------------

@@ -16,7 +16,7 @@ sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
 
 import mxopt_oracle as O
 
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("mxopt.h", "mxopt_optimizers.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("mxopt.h", "mxopt_optimizers.h", "mxopt_engine.h")]
 
 
 @pytest.fixture(scope="module")
@@ -49,7 +49,7 @@ def test_ctypes_structs_match_c_layout(L, tmp_path):
     src.write_text(r'''
 #include <stdio.h>
 #include <stddef.h>
-#include "mxopt_optimizers.h"
+#include "mxopt_engine.h"
 #define S(T) printf(#T " %zu\n", sizeof(T))
 #define F(T, f) printf(#T "." #f " %zu\n", offsetof(T, f))
 int main(void) {
@@ -60,13 +60,18 @@ int main(void) {
   S(mxopt_sgd_hp); F(mxopt_sgd_hp, nesterov);
   S(mxopt_rmsprop_hp); F(mxopt_rmsprop_hp, has_weight_decay);
   S(mxopt_array); F(mxopt_array, dtype);
+  S(mxopt_engine_config); F(mxopt_engine_config, gradient_clip_norm); F(mxopt_engine_config, max_nan_gradients);
+  F(mxopt_engine_config, apply); F(mxopt_engine_config, eps); F(mxopt_engine_config, accumulate_in_f32);
+  S(mxopt_engine_metrics); F(mxopt_engine_metrics, nan_gradient_count); F(mxopt_engine_metrics, clip_scale);
+  F(mxopt_engine_metrics, grad_norm);
   return 0;
 }''')
     exe = tmp_path / "layout"
     subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     want = dict(line.rsplit(" ", 1) for line in subprocess.check_output([str(exe)], text=True).splitlines())
     py = {"mxopt_tensor": L.Tensor, "mxopt_norm_result": L.NormResult, "mxopt_grad_prep": L.GradPrep,
-          "mxopt_adam_hp": L.AdamHp, "mxopt_sgd_hp": L.SgdHp, "mxopt_rmsprop_hp": L.RmspropHp, "mxopt_array": L.Array}
+          "mxopt_adam_hp": L.AdamHp, "mxopt_sgd_hp": L.SgdHp, "mxopt_rmsprop_hp": L.RmspropHp, "mxopt_array": L.Array,
+          "mxopt_engine_config": L.EngineConfig, "mxopt_engine_metrics": L.EngineMetrics}
     for key, val in want.items():
         if "." in key:
             t, f = key.split(".")

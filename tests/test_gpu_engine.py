@@ -1,0 +1,183 @@
+"""GPU parity of the engines' optimizer side (include/mxopt_engine.h) against the oracle's restatement
+of grpo/engine.rs:561-704 and sft/engine.rs:215-371, 459-553, through the C ABI: parameters bit for
+bit after every micro-batch, counters and flags equal, the measured norm within rel 1e-5 of the exact
+one (the oracle is then handed the device's sum of squares so that the clip factor is the same scalar)."""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mxopt_oracle as O
+from gpu_util import assert_bit_equal, to_dev, to_host
+
+F = np.float32
+SIZES = {"embed": 100003, "ln": 64, "tiny": 7, "w1": 3 * 4096, "w2": 4097}
+
+
+@pytest.fixture(scope="module")
+def mx():
+    import mxopt
+    return mxopt
+
+
+def make_params(rng, bf16):
+    ps = {k: rng.normal(0, 0.5, n).astype(F) for k, n in SIZES.items()}
+    return {k: O.f32_to_bf16(v) for k, v in ps.items()} if bf16 else ps
+
+
+def make_grads(rng, bf16, std, names=SIZES):
+    gs = {k: rng.normal(0, std, SIZES[k]).astype(F) for k in names}
+    return {k: O.f32_to_bf16(v) for k, v in gs.items()} if bf16 else gs
+
+
+def check_state(dev, ref, dparams, what):
+    m = dev.metrics()
+    st = ref.state
+    assert (m.step, m.micro_step, m.nan_gradient_count, m.consecutive_nan_count, bool(m.needs_emergency_save)) == \
+           (st.step, st.micro_step, st.nan_gradient_count, st.consecutive_nan_count, st.needs_emergency_save), what
+    for k in dparams:
+        assert_bit_equal(to_host(dparams[k]), ref.params[k], f"{what}: {k}")
+
+
+def exact_clamped_sumsq(grads, cv):
+    return O.exact_sumsq([O.clip_value(g, -cv, cv) for g in grads.values()])
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("apply", ["sgd", "adamw"])
+@pytest.mark.parametrize("n_acc", [1, 3])
+def test_grpo_sequence(mx, bf16, apply, n_acc):
+    rng = np.random.default_rng(7 + n_acc)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=2.0, gradient_clip_value=0.02,
+              max_nan_gradients=50, emergency_save_threshold=2, apply=apply, weight_decay=0.01)
+    dev = mx.GRPOEngineOptimizerSide(dparams, **kw)
+    ref = O.GRPOEngineOptimizerSide(params, **kw)
+    script = ["ok", "ok", "nan", "inf", "ok", "ok", "-inf", "ok", "ok", "ok"]
+    for it, kind in enumerate(script):
+        grads = make_grads(rng, bf16, 0.01 * (1 + it % 3))
+        if kind != "ok":
+            bad = {"nan": np.nan, "inf": np.inf, "-inf": -np.inf}[kind]
+            v = O.as_f32(grads["w1"]).copy()
+            v[4096 + 5] = bad                     # +-Inf would be clamped to a finite bound: the raw value counts
+            grads["w1"] = O.f32_to_bf16(v) if bf16 else v
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        if kind == "ok":
+            exact = exact_clamped_sumsq(grads, 0.02)
+            assert m.norm_measured and abs(m.grad_norm - math.sqrt(exact)) <= 1e-5 * math.sqrt(exact)
+            r = ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
+            assert F(m.clip_scale) == O.norm_scale_c1(m.grad_sumsq, 2.0)[1]
+        else:
+            r = ref.micro_batch(grads)
+        assert (bool(m.skipped), bool(m.gradients_applied), m.step) == (r["skipped"], r["gradients_applied"], r["step"])
+        check_state(dev, ref, dparams, f"micro-batch {it} ({kind})")
+    assert ref.state.nan_gradient_count == 3 and ref.needs_emergency_save
+    dev.clear_emergency_save_flag()
+    ref.clear_emergency_save_flag()
+    dev.reset()
+    ref.reset()
+    check_state(dev, ref, dparams, "after reset")
+
+
+def test_grpo_defaults_new_names_and_errors(mx):
+    """Default config (lr 1e-6, clamp 1.0, clip 1.0, N 1); a name that shows up only in a later
+    micro-batch of a cycle is inserted (engine.rs:2650-2654); unknown names are refused."""
+    rng = np.random.default_rng(11)
+    params = make_params(rng, True)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    dev = mx.GRPOEngineOptimizerSide(dparams, gradient_accumulation_steps=2, learning_rate=0.01)
+    ref = O.GRPOEngineOptimizerSide(params, gradient_accumulation_steps=2, learning_rate=0.01)
+    for names in (["embed", "w1"], ["embed", "w1", "ln", "tiny"], ["w2"], ["embed", "w2"]):
+        grads = make_grads(rng, True, 0.4, names)          # large enough for clamp and clip to act
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
+        assert m.clip_scale < 1.0
+        check_state(dev, ref, dparams, str(names))
+    before = {k: to_host(v) for k, v in dparams.items()}
+    with pytest.raises(KeyError, match="Parameter 'nope' not found in model"):
+        dev.micro_batch({"embed": to_dev(np.zeros(SIZES["embed"], F)), "nope": to_dev(np.zeros(3, F))})
+    with pytest.raises(ValueError):
+        dev.micro_batch({"ln": to_dev(np.zeros(SIZES["ln"] + 1, F))})
+    check_state(dev, ref, dparams, "after refused calls")
+    for k in dparams:
+        assert_bit_equal(to_host(dparams[k]), before[k], k)
+
+
+def test_grpo_training_stopped(mx):
+    params = {"w": np.ones(100, F)}
+    dparams = {"w": to_dev(params["w"])}
+    dev = mx.GRPOEngineOptimizerSide(dparams, max_nan_gradients=3)
+    ref = O.GRPOEngineOptimizerSide(params, max_nan_gradients=3)
+    bad = np.zeros(100, F)
+    bad[3] = np.nan
+    for _ in range(2):
+        dev.micro_batch({"w": to_dev(bad)})
+        ref.micro_batch({"w": bad})
+    with pytest.raises(mx.TrainingStopped, match=r"exceeded maximum NaN gradient count \(3/3\)"):
+        dev.micro_batch({"w": to_dev(bad)})
+    with pytest.raises(O.TrainingStopped):
+        ref.micro_batch({"w": bad})
+    check_state(dev, ref, dparams, "after the limit")
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("apply", ["sgd", "adamw"])
+@pytest.mark.parametrize("acc_f32", [False, True])
+def test_sft_sequence(mx, bf16, apply, acc_f32):
+    if acc_f32 and not bf16:
+        pytest.skip("float32 gradients already accumulate in float32")
+    rng = np.random.default_rng(23)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.02, gradient_accumulation_steps=3, gradient_clip_norm=0.5, gradient_clip_value=0.002,
+              weight_decay=0.01, apply=apply)
+    dev = mx.SFTEngineOptimizerSide(dparams, accumulate_in_f32=acc_f32, **kw)
+    ref = O.SFTEngineOptimizerSide(params, **kw)
+    widen = (lambda g: O.as_f32(g)) if acc_f32 else (lambda g: g)   # a float32 buffer = float32 gradients to the oracle
+    for it in range(7):                                            # two full cycles + one leftover micro-batch
+        names = list(SIZES) if it != 4 else ["embed", "w1"]        # a micro-batch that misses some names
+        grads = make_grads(rng, bf16, 0.01, names)
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        boundary = ref.state.micro_step + 1 >= 3
+        if boundary:
+            assert m.norm_measured and m.gradients_applied
+            r = ref.micro_batch({k: widen(g) for k, g in grads.items()}, norm_sumsq=m.grad_sumsq)
+        else:
+            r = ref.micro_batch({k: widen(g) for k, g in grads.items()})
+        assert (bool(m.gradients_applied), m.step) == (r["gradients_applied"], r["step"])
+        check_state(dev, ref, dparams, f"micro-batch {it}")
+    assert ref.state.micro_step == 1
+    assert dev.flush_gradients() is True
+    assert ref.flush_gradients(norm_sumsq=dev.last_metrics.grad_sumsq) is True
+    check_state(dev, ref, dparams, "after flush")
+    assert dev.flush_gradients() is False and ref.flush_gradients() is False
+    # NaN-loss bookkeeping
+    for _ in range(5):
+        dev.report_nonfinite_loss()
+        ref.report_nonfinite_loss()
+    check_state(dev, ref, dparams, "after NaN losses")
+    assert dev.needs_emergency_save
+
+
+def test_sft_norm_is_of_the_averaged_sum(mx):
+    """The fused norm (last accumulation pass) and the separate one (a micro-batch that misses names)
+    both describe acc / N."""
+    rng = np.random.default_rng(31)
+    params = make_params(rng, False)
+    for partial_last in (False, True):
+        dparams = {k: to_dev(v) for k, v in params.items()}
+        dev = mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=2, gradient_clip_norm=1e-3, learning_rate=0.1)
+        ref = O.SFTEngineOptimizerSide(params, gradient_accumulation_steps=2, gradient_clip_norm=1e-3, learning_rate=0.1)
+        g1 = make_grads(rng, False, 0.01)
+        g2 = make_grads(rng, False, 0.01, ["embed", "ln"] if partial_last else SIZES)
+        dev.micro_batch({k: to_dev(g) for k, g in g1.items()})
+        ref.micro_batch(g1)
+        m = dev.micro_batch({k: to_dev(g) for k, g in g2.items()})
+        acc = {k: g1[k] + g2[k] if k in g2 else g1[k] for k in g1}
+        exact = O.exact_sumsq([a * F(0.5) for a in acc.values()])
+        assert abs(m.grad_sumsq - exact) <= 1e-6 * exact
+        ref.micro_batch(g2, norm_sumsq=m.grad_sumsq)
+        check_state(dev, ref, dparams, f"partial_last={partial_last}")
