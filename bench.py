@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
                     choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
-                             "cfg4", "cfg4-flat", "cfg5", "copy"])
+                             "cfg4", "cfg4-flat", "cfg5", "copy", "grpo-engine", "sft-engine"])
     ap.add_argument("--cpu-sample", type=int, default=128 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -62,7 +62,7 @@ def parse_args():
 
 def tensor_sizes(args):
     from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B"}.get(args.workload)
+    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B", "grpo-engine": "8B", "sft-engine": "8B"}.get(args.workload)
     if model:
         sizes = []
         for _, shape in param_list(QWEN3[model]):
@@ -306,6 +306,46 @@ class Workload:
     def _step_cfg3_rmsprop(self):
         self._timed("rmsprop", lambda: self.ctx.rmsprop(self.t_upd, self.hp))
 
+    # -- the engines' optimizer side (include/mxopt_engine.h) on the 8B list: 4 micro-batches of bf16
+    #    gradients per optimizer step, bf16 parameters updated in place by the reference's plain SGD
+    def _setup_engine(self, kind):
+        from mxopt.qwen3_shapes import QWEN3, param_list
+        t, mx = self.torch, self.mx
+        bf = t.bfloat16
+        self.names = [name for name, _ in param_list(QWEN3["8B"])]
+        self.p = self._randn_list(bf, 0.02)
+        self.g = self._randn_list(bf, 1e-3)
+        params = dict(zip(self.names, self.p))
+        self.grads = dict(zip(self.names, self.g))
+        self.n_micro = 4
+        if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
+            self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=4,
+                                                     ctx=self.ctx)
+            self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10 + 8}
+            self.note = "per micro-batch: validity+norm of clamp(g) (2 B), acc += clip(clamp(g)) (6/10 B), 32-byte read-back"
+        else:                # acc += g in float32, last pass carries the norm of acc/N; p -= lr*(clip(acc/N) + wd*p)
+            self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=4,
+                                                    weight_decay=0.01, accumulate_in_f32=True, ctx=self.ctx)
+            self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 10 + 8}
+            self.note = "float32 accumulation buffer; norm fused into the last accumulation pass"
+        self.step_bytes_per_elem = (self.bytes_per_elem["micro_batch_first"] + 2 * self.bytes_per_elem["micro_batch"] +
+                                    self.bytes_per_elem["micro_batch_apply"])
+        self.dominant = "micro_batch_apply"
+        self.dtype = "bf16 params/grads, f32 accumulate + arithmetic"
+
+    def _setup_grpo_engine(self):
+        self._setup_engine("grpo")
+
+    def _setup_sft_engine(self):
+        self._setup_engine("sft")
+
+    def _step_grpo_engine(self):
+        for k in range(self.n_micro):
+            name = "micro_batch_first" if k == 0 else ("micro_batch_apply" if k == self.n_micro - 1 else "micro_batch")
+            self._timed(name, lambda: self.engine.micro_batch(self.grads))
+
+    _step_sft_engine = _step_grpo_engine
+
     # -- copy: g_out = g (float32, no pre-processing): the plain copy that calibrates HBM counters
     def _setup_copy(self):
         t, mx = self.torch, self.mx
@@ -451,7 +491,8 @@ def main():
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
-    cpu = cpu_baseline(args, n) if args.cpu_sample > 0 and args.workload != "copy" else None
+    no_cpu_leg = ("copy", "grpo-engine", "sft-engine")
+    cpu = cpu_baseline(args, n) if args.cpu_sample > 0 and args.workload not in no_cpu_leg else None
 
     out = {
         "metric": "optimizer steps/s + achieved HBM GB/s (% of 8 TB/s), AdamW on Qwen3-8B shapes",
