@@ -321,7 +321,7 @@ class Workload:
         if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
             self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=4,
                                                      ctx=self.ctx)
-            self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10 + 8}
+            self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10}
             self.note = "per micro-batch: validity+norm of clamp(g) (2 B), acc += clip(clamp(g)) (6/10 B), 32-byte read-back"
         else:                # acc += g in float32, last pass carries the norm of acc/N; p -= lr*(clip(acc/N) + wd*p)
             self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=4,

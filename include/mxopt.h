@@ -210,6 +210,15 @@ int mxopt_rmsprop(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* 
 int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
                     const mxopt_grad_prep* prep);
 
+/* mxopt_sgd_plain on (g + prep(g_out)): g is the float32 accumulation buffer of already-clipped
+ * micro-batches, g_out the last micro-batch, which is clamped / scaled by `pending_prep` in
+ * registers and added (one float32 add, the value mxopt_accumulate_transformed would have stored)
+ * instead of being written back first: r(p, acc, g) + w(p) instead of an accumulation pass plus
+ * an apply pass.  The buffer is left without the last micro-batch.  Same arithmetic as
+ * grpo/engine.rs:636-692 (accumulate, then Qwen3Model::apply_gradients). */
+int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                 const mxopt_grad_prep* pending_prep);
+
 /* ---- global norm ------------------------------------------------------------------ */
 
 /* Sum of squares of the gradients (after prep's pre_mul / clamp_pre) over the whole

@@ -545,6 +545,18 @@ int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, 
   });
 }
 
+int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                 const mxopt_grad_prep* pending_prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedGOut, "mxopt_sgd_plain_with_pending");
+  if (rc) return rc;
+  DevPrep dp = make_prep(pending_prep);
+  dp.flags |= kPrepPendingOnly;
+  const float lr32 = (float)learning_rate;
+  return run_update(ctx, t, "mxopt_sgd_plain_with_pending", [&](const Group& g, const Launch& L) {
+    return launch_sgd_plain_pending(g.pd, g.gd, g.pod, g.god, L, round_to_dtype(lr32, g.pd), dp);
+  });
+}
+
 int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep) {
   int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_grad_transform");
   if (rc) return rc;

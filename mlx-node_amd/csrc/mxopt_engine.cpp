@@ -200,9 +200,60 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     return MXOPT_OK;
   }
   e->consecutive_nan_count = 0;  // engine.rs:660
+  if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result->scale;
+  const int32_t N = acc_steps(e);
+
+  if (e->micro_step + 1 >= N && e->cfg.apply == MXOPT_ENGINE_APPLY_SGD) {
+    // Last micro-batch of the cycle: p -= (lr/N) * (acc + clip(clamp(g))) in one pass over p, acc and
+    // g; the sum is formed in registers exactly as the accumulation pass would have stored it.
+    const double lr = e->cfg.learning_rate / (double)N;  // engine.rs:672
+    std::vector<char> in_batch(e->slots.size(), 0);
+    std::vector<mxopt_tensor> pending, direct, acc_only;
+    for (size_t i = 0; i < n; ++i) {
+      Slot& s = e->slots[idx[i]];
+      if (in_batch[idx[i]]) continue;
+      in_batch[idx[i]] = 1;
+      mxopt_tensor r = blank_tensor();
+      r.p = s.param.data; r.p_out = s.param.data;
+      r.p_dtype = r.p_out_dtype = (uint8_t)s.param.dtype;
+      r.n = s.param.n;
+      if (s.in_acc) {
+        r.g = s.acc; r.g_dtype = MXOPT_F32;
+        r.g_out = grads[i].data; r.g_out_dtype = (uint8_t)grads[i].dtype;
+        pending.push_back(r);
+      } else {
+        r.g = grads[i].data; r.g_dtype = (uint8_t)grads[i].dtype;
+        direct.push_back(r);
+      }
+    }
+    for (size_t k = 0; k < e->slots.size(); ++k) {
+      Slot& s = e->slots[k];
+      if (!s.in_acc || in_batch[k]) continue;
+      mxopt_tensor r = blank_tensor();
+      r.p = s.param.data; r.p_out = s.param.data;
+      r.p_dtype = r.p_out_dtype = (uint8_t)s.param.dtype;
+      r.g = s.acc; r.g_dtype = MXOPT_F32;
+      r.n = s.param.n;
+      acc_only.push_back(r);
+    }
+    mxopt_table* t = nullptr;
+    if (!pending.empty()) {
+      if ((rc = cached_table(ctx, pending, &t)) || (rc = mxopt_sgd_plain_with_pending(ctx, t, lr, &prep))) return rc;
+    }
+    if (!direct.empty()) {
+      if ((rc = cached_table(ctx, direct, &t)) || (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, &prep))) return rc;
+    }
+    if (!acc_only.empty()) {
+      if ((rc = cached_table(ctx, acc_only, &t)) || (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, nullptr))) return rc;
+    }
+    end_cycle(e);
+    e->step += 1;
+    fill_metrics(e, out, 1, 0);
+    if (n) add_norm(out, h);
+    return MXOPT_OK;
+  }
 
   // acc (+)= clip_norm(clamp(g)) in float32 (engine.rs:636-661, :2632-2666)
-  if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result->scale;
   std::vector<mxopt_tensor> first_rows, add_rows;
   for (size_t i = 0; i < n; ++i) {
     Slot& s = e->slots[idx[i]];
@@ -225,17 +276,11 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
   e->micro_step += 1;
 
   int applied = 0;
-  const int32_t N = acc_steps(e);
-  if (e->micro_step >= N) {  // engine.rs:666-692
+  if (e->micro_step >= N) {  // engine.rs:666-692, with AdamW on the averaged sum in place of apply_gradients
     mxopt_grad_prep ap = no_prep();
-    if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {
-      ap.has_pre_mul = 1;
-      ap.pre_mul = (float)(1.0 / (double)N);
-      rc = apply_accumulated(e, e->cfg.learning_rate, 0.0, ap);
-    } else {
-      rc = apply_accumulated(e, e->cfg.learning_rate / (double)N, 0.0, ap);  // engine.rs:672
-    }
-    if (rc) return rc;
+    ap.has_pre_mul = 1;
+    ap.pre_mul = (float)(1.0 / (double)N);
+    if ((rc = apply_accumulated(e, e->cfg.learning_rate, 0.0, ap))) return rc;
     end_cycle(e);
     applied = 1;
   }

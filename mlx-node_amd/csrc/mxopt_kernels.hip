@@ -171,6 +171,14 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
   if (skip_requested(prep)) return;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
+  // The gradient the update sees: prep(g), prep(g + g2) (an accumulation buffer plus the micro-batch
+  // that was not written back to it), or g + prep(g2) (the buffer holds already-clipped gradients and
+  // the pending micro-batch still has to be clipped: grpo/engine.rs:636-661).
+  const bool pending_only = kHasG2 && (pr.flags & kPrepPendingOnly);
+  auto combine = [&](float g, float g2) {
+    if (!kHasG2) return prep_all(pr, g);
+    return pending_only ? g + prep_all(pr, g2) : prep_all(pr, g + g2);
+  };
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
     const ChunkView cv = locate(T, C, one, c);
@@ -186,11 +194,10 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
     const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
     auto one_element = [&](uint64_t off) {
       float p = Elem<PD>::load(P, off);
-      float ge = Elem<GD>::load(G, off);
-      if (kHasG2) ge = ge + Elem<G2D>::load(G2P, off);
+      const float ge = combine(Elem<GD>::load(G, off), kHasG2 ? Elem<G2D>::load(G2P, off) : 0.0f);
       float m = Math::kM ? M[off] : 0.0f;
       float v = read_v ? V[off] : 0.0f;
-      math(p, prep_all(pr, ge), m, v, bc1, bc2, flags);
+      math(p, ge, m, v, bc1, bc2, flags);
       Elem<OD>::store(PO, off, p);
       if (Math::kM) M[off] = m;
       if (use_v) V[off] = v;
@@ -212,9 +219,7 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float ge = g[j][e];
-          if (kHasG2) ge = ge + g2[j][e];
-          math(p[j][e], prep_all(pr, ge), m[j][e], v[j][e], bc1, bc2, flags);
+          math(p[j][e], combine(g[j][e], g2[j][e]), m[j][e], v[j][e], bc1, bc2, flags);
         }
       }
 #pragma unroll
@@ -237,9 +242,7 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
         if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float ge = g[e];
-          if (kHasG2) ge = ge + g2[e];
-          math(p[e], prep_all(pr, ge), m[e], v[e], bc1, bc2, flags);
+          math(p[e], combine(g[e], g2[e]), m[e], v[e], bc1, bc2, flags);
         }
         store_group<OD, E, false>(PO, off, p);
         if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
@@ -591,6 +594,28 @@ static bool plain_for_pd(int gd, int od, const Launch& L, float lr_p, float wd, 
   }
   PlainSgdMath<PD, false> m{lr_p, wd, has_wd};
   return dispatch_gd<PD>(gd, od, L, m, prep);
+}
+
+// Plain SGD on (float32 accumulation buffer + prep(pending gradient)); output in the parameter's dtype.
+template <int PD>
+static bool plain_pending_for_pd(int g2d, const Launch& L, float lr_p, const DevPrep& prep) {
+  PlainSgdMath<PD, false> m{lr_p, 0.0f, 0};
+  switch (g2d) {
+    case MXOPT_F32: launch_update_t<PD, MXOPT_F32, PD, MXOPT_F32>(L, m, prep); return true;
+    case MXOPT_BF16: launch_update_t<PD, MXOPT_F32, PD, MXOPT_BF16>(L, m, prep); return true;
+    case MXOPT_F16: launch_update_t<PD, MXOPT_F32, PD, MXOPT_F16>(L, m, prep); return true;
+  }
+  return false;
+}
+
+bool launch_sgd_plain_pending(int pd, int gd, int od, int g2d, const Launch& L, float lr_p, const DevPrep& prep) {
+  if (gd != MXOPT_F32 || od != pd) return false;
+  switch (pd) {
+    case MXOPT_F32: return plain_pending_for_pd<MXOPT_F32>(g2d, L, lr_p, prep);
+    case MXOPT_BF16: return plain_pending_for_pd<MXOPT_BF16>(g2d, L, lr_p, prep);
+    case MXOPT_F16: return plain_pending_for_pd<MXOPT_F16>(g2d, L, lr_p, prep);
+  }
+  return false;
 }
 
 bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float wd, int has_wd, bool g_promoted,

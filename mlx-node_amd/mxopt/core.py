@@ -192,6 +192,11 @@ class Context:
                                           max_norm, clip_mode, C.c_void_p(out.ptr) if out else None), self.handle)
 
 
+def _sgd_plain_with_pending(self, table: "Table", learning_rate: float, pending_prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_sgd_plain_with_pending(self.handle, table.handle, learning_rate,
+                                                  C.byref(pending_prep) if pending_prep else None), self.handle)
+
+
 def _accumulate_transformed(self, table: "Table", first: bool, prep: Optional[L.GradPrep] = None) -> None:
     L.check(self.lib.mxopt_accumulate_transformed(self.handle, table.handle, int(first),
                                                   C.byref(prep) if prep else None), self.handle)
@@ -205,6 +210,7 @@ def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Opt
 
 Context.accumulate_norm_only = _accumulate_norm_only
 Context.accumulate_transformed = _accumulate_transformed
+Context.sgd_plain_with_pending = _sgd_plain_with_pending
 
 
 class Table:
