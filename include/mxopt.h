@@ -100,6 +100,11 @@ typedef struct mxopt_tensor {
 int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxopt_table** out);
 /* Per-step scalars, `n` entries each; a NULL array leaves that field unchanged. */
 int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* bc2, const uint32_t* flags);
+/* Same tensors (sizes, dtypes, which pointers are set, alignment class), new buffers: swaps the
+ * pointers of an existing table without rebuilding its chunk list (hosts whose arrays move every
+ * step, as MLX's do).  Stream-ordered like a kernel.  Returns MXOPT_ERR_INVALID_ARG and changes
+ * nothing when the layout differs; build a new table then. */
+int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n);
 void mxopt_table_destroy(mxopt_table* t);
 uint64_t mxopt_table_total_elems(const mxopt_table* t);
 uint64_t mxopt_table_num_chunks(const mxopt_table* t);

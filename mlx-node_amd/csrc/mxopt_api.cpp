@@ -387,6 +387,27 @@ int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxo
   return MXOPT_OK;
 }
 
+// Copies t->dev to the device.  Staged through one of two pinned buffers so that the call returns
+// without waiting for the copy; a buffer is reused only after the copy issued from it two calls ago
+// has finished.  Stream-ordered: kernels already enqueued still see the old descriptors.
+static int upload_descriptors(mxopt_table* t) {
+  mxopt_ctx* ctx = t->ctx;
+  const size_t n = t->dev.size();
+  if (!n) return MXOPT_OK;
+  const size_t bytes = n * sizeof(DevTensor);
+  const int k = t->turn ^= 1;
+  if (!t->pinned[k]) {
+    HIP_TRY(ctx, hipHostMalloc((void**)&t->pinned[k], bytes, hipHostMallocDefault));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&t->copied[k], hipEventDisableTiming));
+  } else {
+    HIP_TRY(ctx, hipEventSynchronize(t->copied[k]));
+  }
+  std::memcpy(t->pinned[k], t->dev.data(), bytes);
+  HIP_TRY(ctx, hipMemcpyAsync(t->d_tensors, t->pinned[k], bytes, hipMemcpyHostToDevice, ctx->stream));
+  HIP_TRY(ctx, hipEventRecord(t->copied[k], ctx->stream));
+  return MXOPT_OK;
+}
+
 int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* bc2, const uint32_t* flags) {
   if (!t) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_set_step_scalars: null table");
   mxopt_ctx* ctx = t->ctx;
@@ -398,22 +419,30 @@ int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* 
     if (flags) t->host[i].flags = flags[i];
     fill_dev_tensor(t->host[i], t->dev[i]);
   }
-  if (n) {
-    // Stage through one of two pinned buffers so that the call returns without waiting for the
-    // copy; a buffer is reused only after the copy issued from it two calls ago has finished.
-    const size_t bytes = n * sizeof(DevTensor);
-    const int k = t->turn ^= 1;
-    if (!t->pinned[k]) {
-      HIP_TRY(ctx, hipHostMalloc((void**)&t->pinned[k], bytes, hipHostMallocDefault));
-      HIP_TRY(ctx, hipEventCreateWithFlags(&t->copied[k], hipEventDisableTiming));
-    } else {
-      HIP_TRY(ctx, hipEventSynchronize(t->copied[k]));
-    }
-    std::memcpy(t->pinned[k], t->dev.data(), bytes);
-    HIP_TRY(ctx, hipMemcpyAsync(t->d_tensors, t->pinned[k], bytes, hipMemcpyHostToDevice, ctx->stream));
-    HIP_TRY(ctx, hipEventRecord(t->copied[k], ctx->stream));
+  return upload_descriptors(t);
+}
+
+int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n) {
+  if (!t || (n && !tensors)) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: null argument");
+  mxopt_ctx* ctx = t->ctx;
+  if (n != t->host.size()) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: different number of tensors");
+  std::vector<DevTensor> dev(n);
+  for (size_t i = 0; i < n; ++i) {
+    const mxopt_tensor& a = t->host[i];
+    const mxopt_tensor& b = tensors[i];
+    const bool same = a.n == b.n && !a.p == !b.p && !a.p_out == !b.p_out && !a.g == !b.g && !a.g_out == !b.g_out &&
+                      !a.m == !b.m && !a.v == !b.v && (!a.p || a.p_dtype == b.p_dtype) &&
+                      (!a.p_out || a.p_out_dtype == b.p_out_dtype) && (!a.g || a.g_dtype == b.g_dtype) &&
+                      (!a.g_out || a.g_out_dtype == b.g_out_dtype);
+    fill_dev_tensor(b, dev[i]);
+    // The chunk list depends on the head and on which path the tensor takes.
+    if (!same || dev[i].head != t->dev[i].head || ((dev[i].flags ^ t->dev[i].flags) & kTfUnaligned))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: tensor " + std::to_string(i) + " has a different layout");
   }
-  return MXOPT_OK;
+  DeviceGuard guard(ctx->device);
+  t->host.assign(tensors, tensors + n);
+  t->dev.swap(dev);
+  return upload_descriptors(t);
 }
 
 void mxopt_table_destroy(mxopt_table* t) {

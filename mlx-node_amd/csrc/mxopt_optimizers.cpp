@@ -55,6 +55,22 @@ int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** 
       return MXOPT_OK;
     }
   }
+  // Same layout, other buffers (the caller's arrays moved): keep the chunk list, swap the pointers.
+  // The least recently used candidate goes first so that alternating buffer sets each keep a table.
+  for (size_t i = 0; i < cache.size(); ++i) {
+    if (cache[i].key.size() != key.size() || key.empty()) continue;
+    const std::string saved = ctx->err;
+    if (mxopt_table_retarget(cache[i].table, rows.data(), rows.size()) != MXOPT_OK) {
+      ctx->err = saved;  // a layout mismatch here is not the caller's error
+      continue;
+    }
+    mxopt_ctx::CachedTable hit = std::move(cache[i]);
+    hit.key = std::move(key);
+    cache.erase(cache.begin() + i);
+    cache.push_back(std::move(hit));
+    *out = cache.back().table;
+    return MXOPT_OK;
+  }
   mxopt_table* t = nullptr;
   int rc = mxopt_table_build(ctx, rows.data(), rows.size(), &t);
   if (rc) return rc;

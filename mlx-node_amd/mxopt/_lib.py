@@ -78,6 +78,7 @@ SIGNATURES = {
     "mxopt_table_total_elems": (C.c_uint64, [C.c_void_p]),
     "mxopt_table_num_chunks": (C.c_uint64, [C.c_void_p]),
     "mxopt_table_num_tensors": (C.c_uint64, [C.c_void_p]),
+    "mxopt_table_retarget": (C.c_int, [C.c_void_p, C.POINTER(Tensor), C.c_size_t]),
     "mxopt_tensor_layout": (C.c_int, [C.POINTER(Tensor), C.POINTER(C.c_uint32), C.POINTER(C.c_int),
                                       C.POINTER(C.c_uint64)]),
     "mxopt_adam_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int,

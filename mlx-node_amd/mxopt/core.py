@@ -232,6 +232,15 @@ class Table:
 
     __del__ = close
 
+    def retarget(self, rows: Sequence[TensorSpec]) -> None:
+        """Same tensors in new buffers: swaps the pointers, keeps the chunk list."""
+        rows = list(rows)
+        arr = (L.Tensor * max(len(rows), 1))()
+        for i, r in enumerate(rows):
+            arr[i] = r.to_c()
+        L.check(self.ctx.lib.mxopt_table_retarget(self.handle, arr, len(rows)), self.ctx.handle)
+        self.rows = rows
+
     @property
     def total_elems(self) -> int:
         return self.ctx.lib.mxopt_table_total_elems(self.handle)

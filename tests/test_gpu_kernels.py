@@ -601,3 +601,47 @@ def test_mixed_dtype_table(mx, ctx):
             assert_bit_equal(to_host(dv[i]), ref.state[str(i)][1], f"v{i} it {it}")
     t_g.close()
     t_upd.close()
+
+
+# ---------------------------------------------------------------------------------
+# A table follows its tensors to new buffers
+# ---------------------------------------------------------------------------------
+
+def test_table_retarget(mx, ctx):
+    import torch
+    hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    sizes = [5, 4096, 12289, 100003]
+    table = None
+    for rnd in range(3):
+        ps, gs = make_lists(500 + rnd, sizes=sizes, bf16=True)
+        dp, dg = [to_dev(p) for p in ps], [to_dev(g) for g in gs]
+        dm = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in sizes]
+        dv = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in sizes]
+        rows = [mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)]
+        if table is None:
+            table = ctx.table(rows)
+            chunks = table.num_chunks
+        else:
+            table.retarget(rows)
+            assert table.num_chunks == chunks
+        ctx.adam(table, hp)
+        ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+        for i in range(len(sizes)):
+            assert_bit_equal(to_host(dp[i]), O.f32_to_bf16(ref.update_single(str(i), ps[i], gs[i])), f"round {rnd} p{i}")
+            assert_bit_equal(to_host(dm[i]), ref.state[str(i)][0], f"round {rnd} m{i}")
+    # a different layout is refused and leaves the table as it was
+    other = [mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)]
+    other[1] = mx.TensorSpec(p=dp[1][:100], p_out=dp[1][:100], g=dg[1][:100], m=dm[1][:100], v=dv[1][:100])
+    with pytest.raises(ValueError, match="different layout"):
+        table.retarget(other)
+    shifted = list(rows)
+    shifted[2] = mx.TensorSpec(p=dp[2][1:], p_out=dp[2][1:], g=dg[2][1:], m=dm[2][1:], v=dv[2][1:])
+    with pytest.raises(ValueError):
+        table.retarget(shifted)
+    before = [to_host(p) for p in dp]
+    ctx.adam(table, hp)
+    ref2 = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    ref2.state = ref.state
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(dp[i]), O.f32_to_bf16(ref2.update_single(str(i), before[i], gs[i])), f"after refusal p{i}")
+    table.close()
