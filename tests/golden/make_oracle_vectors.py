@@ -1,6 +1,8 @@
 #!/usr/bin/env python3
 """Writes tests/golden/oracle_vectors.npz: small seeded inputs and the CPU oracle's outputs for
-every optimizer and utility of the path, float32 and bf16 (bf16 as uint16 bit patterns).
+every optimizer and utility of the path, float32 and bf16 (bf16 as uint16 bit patterns), and
+tests/golden/engine_vectors.npz: scripted micro-batch sequences through the oracle's restatement
+of the two training engines' optimizer side (parameters and counters after every micro-batch).
 
 The vectors freeze the oracle (a later edit that changes a result fails tests/test_golden.py)
 and let the GPU tests check the HIP path against committed data without importing the oracle.
@@ -107,6 +109,63 @@ def main():
         out[f"utils.{tag}.apply.out"] = O.apply_gradients({"w": p}, {"w": gs[3]}, 2e-2)["w"]
     np.savez_compressed(os.path.join(HERE, "oracle_vectors.npz"), **out)
     print(f"wrote {len(out)} arrays")
+    eng = engine_vectors()
+    np.savez_compressed(os.path.join(HERE, "engine_vectors.npz"), **eng)
+    print(f"wrote {len(eng)} engine arrays")
+
+
+ENGINE_SIZES = {"a": 261, "b": 70, "c": 517}
+ENGINE_CASES = {
+    # name: (oracle class, keyword arguments, script: which names each micro-batch carries / "nan" / "flush")
+    "grpo_sgd": ("GRPOEngineOptimizerSide",
+                 dict(learning_rate=0.05, gradient_accumulation_steps=2, gradient_clip_norm=0.5,
+                      gradient_clip_value=0.02, emergency_save_threshold=1),
+                 ["abc", "abc", "ab", "nan", "bc", "abc"]),
+    "grpo_adamw": ("GRPOEngineOptimizerSide",
+                   dict(learning_rate=1e-3, gradient_accumulation_steps=3, gradient_clip_norm=None, apply="adamw",
+                        weight_decay=0.1),
+                   ["abc", "abc", "abc", "abc", "nan", "abc", "abc"]),
+    "sft_sgd": ("SFTEngineOptimizerSide",
+                dict(learning_rate=0.02, gradient_accumulation_steps=2, gradient_clip_norm=0.3,
+                     gradient_clip_value=0.004, weight_decay=0.01),
+                ["abc", "abc", "ab", "abc", "abc", "flush"]),
+    "sft_adamw": ("SFTEngineOptimizerSide",
+                  dict(learning_rate=1e-3, gradient_accumulation_steps=2, gradient_clip_norm=1.0, apply="adamw",
+                       weight_decay=0.05),
+                  ["abc", "abc", "abc", "flush"]),
+}
+
+
+def engine_vectors():
+    out = {}
+    for case, (cls, kw, script) in ENGINE_CASES.items():
+        for bf16 in (False, True):
+            tag = f"{case}.{'bf16' if bf16 else 'f32'}"
+            rng = np.random.default_rng(sum(map(ord, tag)))
+            cast = O.f32_to_bf16 if bf16 else (lambda x: x)
+            params = {k: cast(rng.normal(0, 0.5, n).astype(F)) for k, n in ENGINE_SIZES.items()}
+            for k, v in params.items():
+                out[f"{tag}.param.{k}"] = v
+            eng = getattr(O, cls)(params, **kw)
+            for i, what in enumerate(script):
+                if what == "flush":
+                    applied = eng.flush_gradients()
+                else:
+                    names = "abc" if what == "nan" else what
+                    grads = {k: rng.normal(0, 0.01, ENGINE_SIZES[k]).astype(F) for k in names}
+                    if what == "nan":
+                        grads["b"][7] = np.inf
+                    grads = {k: cast(g) for k, g in grads.items()}
+                    for k, g in grads.items():
+                        out[f"{tag}.mb{i}.grad.{k}"] = g
+                    applied = eng.micro_batch(grads)["gradients_applied"]
+                st = eng.state
+                out[f"{tag}.mb{i}.state"] = np.array([st.step, st.micro_step, st.nan_gradient_count,
+                                                      st.consecutive_nan_count, int(st.needs_emergency_save),
+                                                      int(applied)], np.int64)
+                for k in ENGINE_SIZES:
+                    out[f"{tag}.mb{i}.param.{k}"] = eng.params[k]
+    return out
 
 
 if __name__ == "__main__":

@@ -233,3 +233,88 @@ def test_float32_accumulation_buffer_against_committed_vectors(vec):
         for _ in range(3):
             acc.accumulate({"w": g})
         same(impl.host(acc.take()["w"]), vec[f"utils.{dt}.acc_f32"], f"f32 accumulate {dt}")
+
+
+# ---- engines' optimizer side: scripted micro-batch sequences (tests/golden/engine_vectors.npz) ----
+
+@pytest.fixture(scope="module")
+def engine_vec():
+    return np.load(os.path.join(GOLDEN, "engine_vectors.npz"))
+
+
+def engine_cases():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_oracle_vectors", os.path.join(GOLDEN, "make_oracle_vectors.py"))
+    # only the case table is needed; the generator module imports the oracle, which CPU tests may do
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.ENGINE_CASES, mod.ENGINE_SIZES
+
+
+# the case table, restated so that the GPU half does not import the generator (and with it the oracle)
+ENGINE_CASES = {
+    "grpo_sgd": ("GRPOEngineOptimizerSide", dict(learning_rate=0.05, gradient_accumulation_steps=2, gradient_clip_norm=0.5,
+                                                gradient_clip_value=0.02, emergency_save_threshold=1),
+                 ["abc", "abc", "ab", "nan", "bc", "abc"]),
+    "grpo_adamw": ("GRPOEngineOptimizerSide", dict(learning_rate=1e-3, gradient_accumulation_steps=3, gradient_clip_norm=None,
+                                                  apply="adamw", weight_decay=0.1),
+                   ["abc", "abc", "abc", "abc", "nan", "abc", "abc"]),
+    "sft_sgd": ("SFTEngineOptimizerSide", dict(learning_rate=0.02, gradient_accumulation_steps=2, gradient_clip_norm=0.3,
+                                              gradient_clip_value=0.004, weight_decay=0.01),
+                ["abc", "abc", "ab", "abc", "abc", "flush"]),
+    "sft_adamw": ("SFTEngineOptimizerSide", dict(learning_rate=1e-3, gradient_accumulation_steps=2, gradient_clip_norm=1.0,
+                                                apply="adamw", weight_decay=0.05),
+                  ["abc", "abc", "abc", "flush"]),
+}
+
+
+def test_engine_case_table_matches_the_generator():
+    cases, _ = engine_cases()
+    assert cases == ENGINE_CASES
+
+
+def close_params(got, want, exact):
+    got, want = np.asarray(got), np.asarray(want)
+    assert got.dtype == want.dtype
+    if exact:
+        return np.array_equal(bits(got), bits(want))
+    if got.dtype == np.uint16:      # the device's norm may differ in the last float32 place: <= 1 bf16 ulp
+        return np.abs(got.astype(np.int32) - want.astype(np.int32)).max() <= 1
+    return np.allclose(got, want, rtol=1e-6, atol=1e-9)
+
+
+def run_engine_vectors(make_engine, tensor, host, vec, exact):
+    for case, (cls, kw, script) in ENGINE_CASES.items():
+        for dt in ("f32", "bf16"):
+            tag = f"{case}.{dt}"
+            params = {k: tensor(vec[f"{tag}.param.{k}"]) for k in "abc"}
+            eng, live = make_engine(cls, params, kw)
+            for i, what in enumerate(script):
+                if what == "flush":
+                    applied = eng.flush_gradients()
+                else:
+                    names = "abc" if what == "nan" else what
+                    m = eng.micro_batch({k: tensor(vec[f"{tag}.mb{i}.grad.{k}"]) for k in names})
+                    applied = m["gradients_applied"] if isinstance(m, dict) else bool(m.gradients_applied)
+                st = vec[f"{tag}.mb{i}.state"]
+                assert (eng.step, eng.micro_step, eng.nan_gradient_count, int(eng.needs_emergency_save),
+                        int(applied)) == (st[0], st[1], st[2], st[4], st[5]), (tag, i)
+                for k in "abc":
+                    assert close_params(host(live(eng)[k]), vec[f"{tag}.mb{i}.param.{k}"], exact), (tag, i, k)
+
+
+def test_oracle_engines_are_frozen_by_committed_vectors(engine_vec):
+    import mxopt_oracle as O
+    run_engine_vectors(lambda cls, params, kw: (getattr(O, cls)(params, **kw), lambda e: e.params),
+                       np.asarray, np.asarray, engine_vec, exact=True)
+
+
+@pytest.mark.gpu
+def test_library_engines_against_committed_vectors(engine_vec):
+    impl = GpuImpl()
+
+    def make(cls, params, kw):
+        eng = getattr(impl.mx, cls)(params, **kw)
+        return eng, lambda e: params          # updated in place
+
+    run_engine_vectors(make, impl.tensor, impl.host, engine_vec, exact=False)
