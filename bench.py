@@ -326,8 +326,8 @@ class Workload:
         else:                # acc += g in float32, last pass carries the norm of acc/N; p -= lr*(clip(acc/N) + wd*p)
             self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=4,
                                                     weight_decay=0.01, accumulate_in_f32=True, ctx=self.ctx)
-            self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 10 + 8}
-            self.note = "float32 accumulation buffer; norm fused into the last accumulation pass"
+            self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 6 + 10}
+            self.note = "float32 accumulation buffer; last micro-batch: norm of (acc+g)/N read-only, then folded into the update"
         self.step_bytes_per_elem = (self.bytes_per_elem["micro_batch_first"] + 2 * self.bytes_per_elem["micro_batch"] +
                                     self.bytes_per_elem["micro_batch_apply"])
         self.dominant = "micro_batch_apply"

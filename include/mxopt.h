@@ -215,14 +215,19 @@ int mxopt_rmsprop(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* 
 int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
                     const mxopt_grad_prep* prep);
 
-/* mxopt_sgd_plain on (g + prep(g_out)): g is the float32 accumulation buffer of already-clipped
- * micro-batches, g_out the last micro-batch, which is clamped / scaled by `pending_prep` in
- * registers and added (one float32 add, the value mxopt_accumulate_transformed would have stored)
- * instead of being written back first: r(p, acc, g) + w(p) instead of an accumulation pass plus
- * an apply pass.  The buffer is left without the last micro-batch.  Same arithmetic as
- * grpo/engine.rs:636-692 (accumulate, then Qwen3Model::apply_gradients). */
-int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
-                                 const mxopt_grad_prep* pending_prep);
+/* mxopt_sgd_plain with the last micro-batch still pending: g is the float32 accumulation buffer,
+ * g_out the micro-batch that was NOT added to it.  The sum is formed in registers (one float32
+ * add, the value an accumulation pass would have stored) instead of being written back and read
+ * again: r(p, acc, g) + w(p) replaces an accumulation pass plus an apply pass.  The buffer is
+ * left without the last micro-batch.
+ *   prep_covers_sum = 0: gradient = g + prep(g_out)   the buffer holds already clipped
+ *                        micro-batches, the pending one is clamped / scaled here
+ *                        (grpo/engine.rs:636-692: clip, accumulate, apply_gradients);
+ *   prep_covers_sum = 1: gradient = prep(g + g_out)   average, clip and clamp act on the sum
+ *                        (sft/engine.rs:293-371), pair with mxopt_accumulate_norm_only.
+ * weight_decay as in mxopt_sgd_plain. */
+int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
+                                 const mxopt_grad_prep* prep, int prep_covers_sum);
 
 /* ---- global norm ------------------------------------------------------------------ */
 

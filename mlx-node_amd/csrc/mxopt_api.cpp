@@ -574,15 +574,17 @@ int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, 
   });
 }
 
-int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
-                                 const mxopt_grad_prep* pending_prep) {
+int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
+                                 const mxopt_grad_prep* prep, int prep_covers_sum) {
   int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedGOut, "mxopt_sgd_plain_with_pending");
   if (rc) return rc;
-  DevPrep dp = make_prep(pending_prep);
-  dp.flags |= kPrepPendingOnly;
+  DevPrep dp = make_prep(prep);
+  if (!prep_covers_sum) dp.flags |= kPrepPendingOnly;
   const float lr32 = (float)learning_rate;
+  const float wd32 = (float)weight_decay;
+  const int has_wd = weight_decay > 0.0;  // sft/engine.rs:345
   return run_update(ctx, t, "mxopt_sgd_plain_with_pending", [&](const Group& g, const Launch& L) {
-    return launch_sgd_plain_pending(g.pd, g.gd, g.pod, g.god, L, round_to_dtype(lr32, g.pd), dp);
+    return launch_sgd_plain_pending(g.pd, g.gd, g.pod, g.god, L, round_to_dtype(lr32, g.pd), wd32, has_wd, dp);
   });
 }
 

@@ -200,6 +200,8 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     return MXOPT_OK;
   }
   e->consecutive_nan_count = 0;  // engine.rs:660
+  if (!e->have_acc)
+    for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
   if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result->scale;
   const int32_t N = acc_steps(e);
 
@@ -238,7 +240,7 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     }
     mxopt_table* t = nullptr;
     if (!pending.empty()) {
-      if ((rc = cached_table(ctx, pending, &t)) || (rc = mxopt_sgd_plain_with_pending(ctx, t, lr, &prep))) return rc;
+      if ((rc = cached_table(ctx, pending, &t)) || (rc = mxopt_sgd_plain_with_pending(ctx, t, lr, 0.0, &prep, 0))) return rc;
     }
     if (!direct.empty()) {
       if ((rc = cached_table(ctx, direct, &t)) || (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, &prep))) return rc;
@@ -345,6 +347,11 @@ int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt
   const size_t n = idx.size();
   e->consecutive_nan_count = 0;  // sft/engine.rs:261-267
   const bool first_cycle_step = !e->have_acc;
+  if (first_cycle_step)
+    for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
+  const int32_t N = acc_steps(e);
+  const bool boundary = e->micro_step + 1 >= N;
+  const bool direct = boundary && first_cycle_step;  // N = 1: no accumulator is needed at all
   std::vector<mxopt_tensor> rows;
   int rc;
   size_t held = 0;
@@ -355,7 +362,7 @@ int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt
     const int want = e->cfg.accumulate_in_f32 ? MXOPT_F32 : grads[i].dtype;
     if (first_cycle_step) {
       if (s.in_acc) continue;  // the same name twice in one call: the map keeps one
-      if ((rc = ensure_acc(e, s, want))) return rc;
+      if (!direct && (rc = ensure_acc(e, s, want))) return rc;
       s.in_acc = true;
     } else if (s.acc_dtype != want && !(s.acc_dtype == MXOPT_F32)) {
       return fail(ctx, MXOPT_ERR_INVALID_ARG,
@@ -363,13 +370,81 @@ int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt
     }
     mxopt_tensor r = blank_tensor();
     r.g = grads[i].data; r.g_dtype = (uint8_t)grads[i].dtype;
-    r.g_out = s.acc; r.g_out_dtype = (uint8_t)s.acc_dtype;
+    if (!direct) { r.g_out = s.acc; r.g_out_dtype = (uint8_t)s.acc_dtype; }
     r.n = grads[i].n;
     rows.push_back(r);
   }
   if (first_cycle_step) held = rows.size();
-  const int32_t N = acc_steps(e);
-  const bool boundary = e->micro_step + 1 >= N;
+
+  // Last micro-batch of the cycle, every held tensor has a gradient in it: the sum acc + g is formed
+  // in registers by the norm pass and again by the update, instead of being written back and read
+  // twice.  With no accumulator yet (N = 1) the gradient is applied straight from where it lies.
+  bool all_f32 = true;
+  for (const mxopt_tensor& r : rows) all_f32 = all_f32 && r.g_out_dtype == MXOPT_F32;
+  const bool pending = boundary && !first_cycle_step && e->cfg.apply == MXOPT_ENGINE_APPLY_SGD && all_f32 &&
+                       rows.size() == held;
+  if ((direct || pending) && !rows.empty()) {
+    mxopt_grad_prep prep = no_prep();
+    prep.has_pre_mul = 1;
+    prep.pre_mul = (float)(1.0 / (double)N);  // mul_scalar(scale): float64, then one cast
+    mxopt_table* t = nullptr;
+    mxopt_norm_result h;
+    bool measured = false;
+    if (e->cfg.has_gradient_clip_norm) {
+      if ((rc = cached_table(ctx, rows, &t))) return rc;
+      rc = direct ? mxopt_global_norm(ctx, t, 0, &prep, e->cfg.gradient_clip_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, e->d_result)
+                  : mxopt_accumulate_norm_only(ctx, t, &prep, e->cfg.gradient_clip_norm, MXOPT_CLIP_ALWAYS_MULTIPLY,
+                                               e->d_result);
+      if (rc) return rc;
+      prep.d_scale = &e->d_result->scale;
+      if (out) {
+        if ((rc = mxopt_read_norm_result(ctx, e->d_result, &h))) return rc;
+        measured = true;
+      }
+    }
+    if (e->cfg.has_gradient_clip_value) {
+      prep.has_clamp_post = 1;
+      prep.post_lo = (float)(-e->cfg.gradient_clip_value);
+      prep.post_hi = (float)e->cfg.gradient_clip_value;
+    }
+    std::vector<mxopt_tensor> urows;
+    std::vector<const char*> unames;
+    std::vector<mxopt_array> uparams, ugrads;
+    size_t k = 0;
+    for (size_t i = 0; i < n && k < rows.size(); ++i) {
+      Slot& s = e->slots[idx[i]];
+      if (rows[k].g != grads[i].data || !s.in_acc) continue;  // rows follow the batch order, minus dropped names
+      mxopt_tensor r = blank_tensor();
+      r.p = s.param.data; r.p_out = s.param.data;
+      r.p_dtype = r.p_out_dtype = (uint8_t)s.param.dtype;
+      r.n = s.param.n;
+      if (direct) {
+        r.g = grads[i].data; r.g_dtype = (uint8_t)grads[i].dtype;
+      } else {
+        r.g = s.acc; r.g_dtype = MXOPT_F32;
+        r.g_out = grads[i].data; r.g_out_dtype = (uint8_t)grads[i].dtype;
+      }
+      urows.push_back(r);
+      unames.push_back(s.name.c_str());
+      uparams.push_back(s.param);
+      ugrads.push_back(grads[i]);
+      ++k;
+    }
+    if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {  // direct only
+      rc = mxopt_optimizer_update_many(e->adamw, unames.size(), unames.data(), uparams.data(), ugrads.data(),
+                                       uparams.data(), &prep);
+    } else {
+      if ((rc = cached_table(ctx, urows, &t))) return rc;
+      rc = direct ? mxopt_sgd_plain(ctx, t, e->cfg.learning_rate, e->cfg.weight_decay, &prep)
+                  : mxopt_sgd_plain_with_pending(ctx, t, e->cfg.learning_rate, e->cfg.weight_decay, &prep, 1);
+    }
+    if (rc) return rc;
+    end_cycle(e);
+    e->step += 1;
+    fill_metrics(e, out, 1, 0);
+    if (measured) add_norm(out, h);
+    return MXOPT_OK;
+  }
   // The norm of acc/N rides on the last accumulation pass when that pass touches every held tensor.
   const bool fuse_norm = boundary && e->cfg.has_gradient_clip_norm && !rows.empty() && rows.size() == held;
   if (!rows.empty()) {

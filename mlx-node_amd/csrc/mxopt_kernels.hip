@@ -598,8 +598,8 @@ static bool plain_for_pd(int gd, int od, const Launch& L, float lr_p, float wd, 
 
 // Plain SGD on (float32 accumulation buffer + prep(pending gradient)); output in the parameter's dtype.
 template <int PD>
-static bool plain_pending_for_pd(int g2d, const Launch& L, float lr_p, const DevPrep& prep) {
-  PlainSgdMath<PD, false> m{lr_p, 0.0f, 0};
+static bool plain_pending_for_pd(int g2d, const Launch& L, float lr_p, float wd, int has_wd, const DevPrep& prep) {
+  PlainSgdMath<PD, false> m{lr_p, wd, has_wd};
   switch (g2d) {
     case MXOPT_F32: launch_update_t<PD, MXOPT_F32, PD, MXOPT_F32>(L, m, prep); return true;
     case MXOPT_BF16: launch_update_t<PD, MXOPT_F32, PD, MXOPT_BF16>(L, m, prep); return true;
@@ -608,12 +608,13 @@ static bool plain_pending_for_pd(int g2d, const Launch& L, float lr_p, const Dev
   return false;
 }
 
-bool launch_sgd_plain_pending(int pd, int gd, int od, int g2d, const Launch& L, float lr_p, const DevPrep& prep) {
+bool launch_sgd_plain_pending(int pd, int gd, int od, int g2d, const Launch& L, float lr_p, float wd, int has_wd,
+                              const DevPrep& prep) {
   if (gd != MXOPT_F32 || od != pd) return false;
   switch (pd) {
-    case MXOPT_F32: return plain_pending_for_pd<MXOPT_F32>(g2d, L, lr_p, prep);
-    case MXOPT_BF16: return plain_pending_for_pd<MXOPT_BF16>(g2d, L, lr_p, prep);
-    case MXOPT_F16: return plain_pending_for_pd<MXOPT_F16>(g2d, L, lr_p, prep);
+    case MXOPT_F32: return plain_pending_for_pd<MXOPT_F32>(g2d, L, lr_p, wd, has_wd, prep);
+    case MXOPT_BF16: return plain_pending_for_pd<MXOPT_BF16>(g2d, L, lr_p, wd, has_wd, prep);
+    case MXOPT_F16: return plain_pending_for_pd<MXOPT_F16>(g2d, L, lr_p, wd, has_wd, prep);
   }
   return false;
 }

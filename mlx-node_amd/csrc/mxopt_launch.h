@@ -31,8 +31,10 @@ bool launch_rmsprop(int pd, int gd, int od, const Launch& L, const mxopt_rmsprop
 bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float wd, int has_wd, bool g_promoted,
                       const DevPrep& prep);
 // add != 0: g_out = g_out + prep(g) instead of g_out = prep(g).
-// g: float32 accumulation buffer, tensor.g_out: pending gradient of dtype g2d, prep on the pending one only.
-bool launch_sgd_plain_pending(int pd, int gd, int od, int g2d, const Launch& L, float lr_p, const DevPrep& prep);
+// g: float32 accumulation buffer, tensor.g_out: pending gradient of dtype g2d; prep's kPrepPendingOnly
+// flag says whether prep covers the pending gradient alone or the sum.
+bool launch_sgd_plain_pending(int pd, int gd, int od, int g2d, const Launch& L, float lr_p, float wd, int has_wd,
+                              const DevPrep& prep);
 bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep, int add);
 // mode 0: square g; 1: square g_out; 2: g_out = first ? g : g_out + g, square the result;
 // 3: square g_out + g without storing it.

@@ -91,7 +91,8 @@ SIGNATURES = {
     "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
     "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),
     "mxopt_sgd_plain": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double, C.POINTER(GradPrep)]),
-    "mxopt_sgd_plain_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.POINTER(GradPrep)]),
+    "mxopt_sgd_plain_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double, C.POINTER(GradPrep),
+                                               C.c_int]),
     "mxopt_global_norm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
                                     C.c_void_p]),
     "mxopt_grad_transform": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep)]),

@@ -192,9 +192,11 @@ class Context:
                                           max_norm, clip_mode, C.c_void_p(out.ptr) if out else None), self.handle)
 
 
-def _sgd_plain_with_pending(self, table: "Table", learning_rate: float, pending_prep: Optional[L.GradPrep] = None) -> None:
-    L.check(self.lib.mxopt_sgd_plain_with_pending(self.handle, table.handle, learning_rate,
-                                                  C.byref(pending_prep) if pending_prep else None), self.handle)
+def _sgd_plain_with_pending(self, table: "Table", learning_rate: float, weight_decay: float = 0.0,
+                            prep: Optional[L.GradPrep] = None, prep_covers_sum: bool = False) -> None:
+    L.check(self.lib.mxopt_sgd_plain_with_pending(self.handle, table.handle, learning_rate, weight_decay,
+                                                  C.byref(prep) if prep else None, int(prep_covers_sum)),
+            self.handle)
 
 
 def _accumulate_transformed(self, table: "Table", first: bool, prep: Optional[L.GradPrep] = None) -> None:

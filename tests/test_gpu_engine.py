@@ -181,3 +181,27 @@ def test_sft_norm_is_of_the_averaged_sum(mx):
         assert abs(m.grad_sumsq - exact) <= 1e-6 * exact
         ref.micro_batch(g2, norm_sumsq=m.grad_sumsq)
         check_state(dev, ref, dparams, f"partial_last={partial_last}")
+
+
+@pytest.mark.parametrize("kind", ["grpo", "sft"])
+@pytest.mark.parametrize("apply", ["sgd", "adamw"])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_one_micro_batch_per_step(mx, kind, apply, bf16):
+    """gradient_accumulation_steps = 1 (both engines' default): the gradient is applied from where it
+    lies, no accumulator is involved."""
+    rng = np.random.default_rng(41)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    if kind == "grpo":
+        kw = dict(learning_rate=0.05, gradient_clip_norm=1.5, gradient_clip_value=0.03, apply=apply, weight_decay=0.02)
+        dev, ref = mx.GRPOEngineOptimizerSide(dparams, **kw), O.GRPOEngineOptimizerSide(params, **kw)
+    else:
+        kw = dict(learning_rate=0.05, gradient_clip_norm=1.5, gradient_clip_value=0.003, apply=apply, weight_decay=0.02)
+        dev, ref = mx.SFTEngineOptimizerSide(dparams, **kw), O.SFTEngineOptimizerSide(params, **kw)
+    for it in range(4):
+        names = list(SIZES) if it != 2 else ["embed", "tiny"]
+        grads = make_grads(rng, bf16, 0.02, names)
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        assert m.gradients_applied and m.norm_measured and m.clip_scale < 1.0
+        ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
+        check_state(dev, ref, dparams, f"{kind} step {it}")
