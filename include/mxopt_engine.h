@@ -106,6 +106,11 @@ int mxopt_engine_get_metrics(const mxopt_engine* e, mxopt_engine_metrics* out);
 int mxopt_engine_clear_emergency_save_flag(mxopt_engine* e);
 int mxopt_engine_reset(mxopt_engine* e);
 
+/* MXOPT_ENGINE_APPLY_ADAMW only: the AdamW moments as a safetensors file
+ * (mxopt_optimizer_save_file / mxopt_optimizer_load_file of the engine's optimizer). */
+int mxopt_engine_save_optimizer_state(mxopt_engine* e, const char* path);
+int mxopt_engine_load_optimizer_state(mxopt_engine* e, const char* path);
+
 #ifdef __cplusplus
 }
 #endif

@@ -92,6 +92,16 @@ int mxopt_optimizer_save_state(mxopt_optimizer* opt, const char* param_name, flo
 int mxopt_optimizer_load_state(mxopt_optimizer* opt, const char* param_name, const float* m, const float* v,
                                uint64_t n, int64_t step_count);
 
+/* Optimizer-state checkpoint on disk, in the safetensors layout of the reference's own writer
+ * (crates/mlx-core/src/utils/safetensors.rs:312-385): tensors "<param_name>.m" / "<param_name>.v",
+ * float32, shape [elements], sorted by name; __metadata__ carries the optimizer kind and the call
+ * counter `step`.  The reference saves no optimizer state at all (saveCheckpoint,
+ * packages/trl/src/trainers/grpo-trainer.ts:1146-1206 writes the model only), so resuming there
+ * restarts the moments from zero.  Both calls synchronise the context's stream; load replaces the
+ * optimizer's current state and refuses a file written for another optimizer kind. */
+int mxopt_optimizer_save_file(mxopt_optimizer* opt, const char* path);
+int mxopt_optimizer_load_file(mxopt_optimizer* opt, const char* path);
+
 /* ---- GradientUtils (optimizers/mod.rs:33-227) -------------------------------------- */
 /* compute_gradient_norm (:43-55): sqrt of the float64 sum of squares.  Synchronises. */
 int mxopt_compute_gradient_norm(mxopt_ctx* ctx, size_t n, const mxopt_array* grads, double* norm_out);

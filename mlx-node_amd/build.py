@@ -17,7 +17,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxopt.so")
 
-SOURCES = ["mxopt_kernels.hip", "mxopt_api.cpp", "mxopt_optimizers.cpp", "mxopt_engine.cpp"]
+SOURCES = ["mxopt_kernels.hip", "mxopt_api.cpp", "mxopt_optimizers.cpp", "mxopt_engine.cpp", "mxopt_checkpoint.cpp"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -618,4 +618,16 @@ int mxopt_engine_reset(mxopt_engine* e) {
   return MXOPT_OK;
 }
 
+int mxopt_engine_save_optimizer_state(mxopt_engine* e, const char* path) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_save_optimizer_state: null engine");
+  if (!e->adamw) return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "this engine applies plain SGD: there is no optimizer state");
+  return mxopt_optimizer_save_file(e->adamw, path);
+}
+
+int mxopt_engine_load_optimizer_state(mxopt_engine* e, const char* path) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_load_optimizer_state: null engine");
+  if (!e->adamw) return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "this engine applies plain SGD: there is no optimizer state");
+  return mxopt_optimizer_load_file(e->adamw, path);
+}
+
 }  // extern "C"

@@ -12,6 +12,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "mxopt_checkpoint_internal.h"
 #include "mxopt_internal.h"
 
 namespace mxopt {
@@ -440,6 +441,56 @@ int mxopt_optimizer_load_state(mxopt_optimizer* opt, const char* param_name, con
     st->has_velocity = true;
   }
   if (is_adam(opt)) opt->step = step_count;
+  return MXOPT_OK;
+}
+
+static const char* kind_name(Kind k) {
+  switch (k) {
+    case Kind::Adam: return "adam";
+    case Kind::AdamW: return "adamw";
+    case Kind::Sgd: return "sgd";
+    default: return "rmsprop";
+  }
+}
+
+int mxopt_optimizer_save_file(mxopt_optimizer* opt, const char* path) {
+  if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "optimizer_save_file: null optimizer");
+  std::vector<CheckpointTensor> tensors;
+  for (const auto& kv : opt->state) {
+    const StateEntry& st = kv.second;
+    if (st.m) tensors.push_back({kv.first + ".m", st.m, st.n});
+    if (st.v && (opt->kind != Kind::Sgd || st.has_velocity)) tensors.push_back({kv.first + ".v", st.v, st.n});
+  }
+  return save_state_file(opt->ctx, path, kind_name(opt->kind), opt->step, tensors);
+}
+
+int mxopt_optimizer_load_file(mxopt_optimizer* opt, const char* path) {
+  if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "optimizer_load_file: null optimizer");
+  free_state(opt);  // a checkpoint replaces whatever state there was
+  int64_t step = 0;
+  int rc = load_state_file(opt->ctx, path, kind_name(opt->kind), &step,
+                           [&](const std::string& key, uint64_t n, float** device) -> int {
+    if (key.size() < 3 || key[key.size() - 2] != '.' || (key.back() != 'm' && key.back() != 'v'))
+      return fail(opt->ctx, MXOPT_ERR_INVALID_ARG, "optimizer_load_file: unexpected tensor '" + key + "'");
+    const std::string name = key.substr(0, key.size() - 2);
+    StateEntry* st = nullptr;
+    int r = get_state(opt, name.c_str(), n, &st);
+    if (r) return r;
+    if (key.back() == 'm') {
+      *device = st->m;
+    } else {
+      *device = st->v;
+      st->has_velocity = true;
+    }
+    if (!*device && n)
+      return fail(opt->ctx, MXOPT_ERR_INVALID_ARG, "optimizer_load_file: this optimizer keeps no '" + key + "'");
+    return MXOPT_OK;
+  });
+  if (rc) {
+    free_state(opt);
+    return rc;
+  }
+  if (is_adam(opt)) opt->step = step;
   return MXOPT_OK;
 }
 

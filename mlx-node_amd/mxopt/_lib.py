@@ -132,6 +132,8 @@ SIGNATURES.update({
     "mxopt_optimizer_save_state": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p]),
     "mxopt_optimizer_load_state": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_uint64,
                                              C.c_int64]),
+    "mxopt_optimizer_save_file": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "mxopt_optimizer_load_file": (C.c_int, [C.c_void_p, C.c_char_p]),
     "mxopt_compute_gradient_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, _PD]),
     "mxopt_clip_grad_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, _PA, _PD]),
     "mxopt_clip_grad_value": (C.c_int, [C.c_void_p, _PA, C.c_double, C.c_double, _PA]),
@@ -185,6 +187,8 @@ SIGNATURES.update({
     "mxopt_engine_get_metrics": (C.c_int, [C.c_void_p, _PM]),
     "mxopt_engine_clear_emergency_save_flag": (C.c_int, [C.c_void_p]),
     "mxopt_engine_reset": (C.c_int, [C.c_void_p]),
+    "mxopt_engine_save_optimizer_state": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "mxopt_engine_load_optimizer_state": (C.c_int, [C.c_void_p, C.c_char_p]),
 })
 
 def load() -> C.CDLL:

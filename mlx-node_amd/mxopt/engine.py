@@ -91,6 +91,12 @@ class _EngineOptimizerSide:
     def reset(self) -> None:
         self._check(self.lib.mxopt_engine_reset(self.handle))
 
+    def save_optimizer_state(self, path) -> None:
+        self._check(self.lib.mxopt_engine_save_optimizer_state(self.handle, str(path).encode()))
+
+    def load_optimizer_state(self, path) -> None:
+        self._check(self.lib.mxopt_engine_load_optimizer_state(self.handle, str(path).encode()))
+
 
 def _config(kind, learning_rate, gradient_accumulation_steps, gradient_clip_norm, gradient_clip_value, weight_decay,
             max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps, accumulate_in_f32) -> L.EngineConfig:

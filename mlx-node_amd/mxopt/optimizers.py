@@ -119,6 +119,14 @@ class _Optimizer:
             vo = None     # SGD before its first momentum step: no velocity yet
         return mo, vo
 
+    def save_file(self, path: str) -> None:
+        """Writes every moment / velocity and the call counter to a safetensors file."""
+        L.check(self.lib.mxopt_optimizer_save_file(self.handle, str(path).encode()), self.ctx.handle)
+
+    def load_file(self, path: str) -> None:
+        """Replaces this optimizer's state with a checkpoint written by save_file."""
+        L.check(self.lib.mxopt_optimizer_load_file(self.handle, str(path).encode()), self.ctx.handle)
+
     def load_state(self, param_name: str, m: Optional[torch.Tensor], v: Optional[torch.Tensor],
                    step_count: int = 0) -> None:
         n = (m if m is not None else v).numel()
