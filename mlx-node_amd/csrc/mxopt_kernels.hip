@@ -328,7 +328,16 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
 
 // A value clamp would turn +-Inf into a finite bound and hide it from the sum-based validity
 // check; the engines test the raw values (grpo/engine.rs:563-569), so such a lane poisons its partial.
-__device__ __forceinline__ bool is_inf(float x) { return __builtin_isinf(x); }
+
+// The value whose square enters the norm.  Under a clamp the lane only has to remember that it met
+// a NaN or an infinity (its partial is poisoned afterwards), so the clamp itself can be a single
+// median-of-three that does not care about NaN.
+__device__ __forceinline__ float norm_value(const PrepRegs& pr, float x, bool clamped, bool& bad) {
+  if (!clamped) return prep_pre(pr, x);
+  bad |= !__builtin_isfinite(x);
+  if (pr.flags & kPrepPreMul) x = x * pr.pre_mul;
+  return __builtin_amdgcn_fmed3f(x, pr.pre_lo, pr.pre_hi);
+}
 
 template <int AD, int GD>
 __device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
@@ -376,8 +385,7 @@ struct SumsqChunk {
       for (int e = 0; e < E; ++e) {
         if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
         if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
-        if (clamped) hidden_inf |= is_inf(x[j][e]);
-        const float y = prep_pre(pr, x[j][e]);
+        const float y = norm_value(pr, x[j][e], clamped, hidden_inf);
         s32 = fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
@@ -407,8 +415,9 @@ struct SumsqChunk {
       for (int e = 0; e < E; ++e) {
         if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
         if (MODE == 3) x[e] = accumulate_op<AD, GD>(x[e], g[e], false);
-        const float y = prep_pre(pr, x[e]);
-        s32 = (clamped && is_inf(x[e])) ? __builtin_nanf("") : fmaf(y, y, s32);
+        bool bad = false;
+        const float y = norm_value(pr, x[e], clamped, bad);
+        s32 = bad ? __builtin_nanf("") : fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, false>(A, off, x);
     }
@@ -426,9 +435,9 @@ struct SumsqChunk {
       Elem<AD>::store(cv.t.g_out, off, x);
     }
     if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), false);
-    const float y = prep_pre(pr, x);
-    if ((pr.flags & kPrepClampPre) && is_inf(x)) return __builtin_nanf("");
-    return fmaf(y, y, s32);
+    bool bad = false;
+    const float y = norm_value(pr, x, (pr.flags & kPrepClampPre) != 0, bad);
+    return bad ? __builtin_nanf("") : fmaf(y, y, s32);
   }
 };
 
