@@ -43,7 +43,26 @@ def build(verbose: bool = False) -> str:
     if verbose and err.strip():
         print(err)
     os.replace(LIB + ".tmp", LIB)
+    build_demo(verbose)
     return LIB
+
+
+DEMO = os.path.join(HERE, "bin", "cabi_demo")
+
+
+def build_demo(verbose: bool = False) -> str:
+    """examples/cabi_demo.c as plain C11 against the public headers: a host without Python, and the
+    proof that the headers are C."""
+    os.makedirs(os.path.dirname(DEMO), exist_ok=True)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-Werror", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.join(rocm, "include"), os.path.join(HERE, "examples", "cabi_demo.c"), "-o", DEMO,
+           "-L", HERE, "-lmxopt", "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return DEMO
 
 
 if __name__ == "__main__":

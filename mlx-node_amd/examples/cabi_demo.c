@@ -1,0 +1,186 @@
+/* A plain-C host of libmxopt.so: what a cgo / Rust / N-API binding does, without any Python.
+ *
+ *   cabi_demo            known-answer checks through the optimizer objects (the reference's own
+ *                        closed forms: __test__/core/optimizers.test.ts:151-203, 324-351) and the
+ *                        engine entry points, then a timing of updateSingle-per-tensor against
+ *                        one update_many call over the Qwen3-0.6B parameter list.
+ * Prints "PASS" lines and one "TIMING" line; exits non-zero on the first mismatch.
+ */
+#define _POSIX_C_SOURCE 200809L
+#include <hip/hip_runtime_api.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+
+#include "mxopt_engine.h"
+
+#define CHECK_HIP(call)                                                                  \
+  do {                                                                                   \
+    hipError_t e_ = (call);                                                              \
+    if (e_ != hipSuccess) { fprintf(stderr, "%s: %s\n", #call, hipGetErrorString(e_)); exit(2); } \
+  } while (0)
+#define CHECK_MX(call)                                                                   \
+  do {                                                                                   \
+    int rc_ = (call);                                                                    \
+    if (rc_ != MXOPT_OK) { fprintf(stderr, "%s -> %d: %s\n", #call, rc_, mxopt_last_error(ctx)); exit(3); } \
+  } while (0)
+
+static mxopt_ctx* ctx;
+
+static float* to_device(const float* host, size_t n) {
+  float* d = NULL;
+  CHECK_HIP(hipMalloc((void**)&d, (n ? n : 1) * sizeof(float)));
+  if (n) CHECK_HIP(hipMemcpy(d, host, n * sizeof(float), hipMemcpyHostToDevice));
+  return d;
+}
+
+static void expect_close(const char* what, const float* d, const double* want, size_t n, double tol) {
+  float host[16];
+  CHECK_MX(mxopt_synchronize(ctx));
+  CHECK_HIP(hipMemcpy(host, d, n * sizeof(float), hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < n; ++i) {
+    if (!(fabs((double)host[i] - want[i]) <= tol)) {
+      fprintf(stderr, "FAIL %s[%zu]: got %.9g want %.9g\n", what, i, host[i], want[i]);
+      exit(1);
+    }
+  }
+  printf("PASS %s\n", what);
+}
+
+static double now_ms(void) {
+  struct timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return ts.tv_sec * 1e3 + ts.tv_nsec * 1e-6;
+}
+
+static void known_answers(void) {
+  /* SGD, lr 0.1: [1,2,3] - 0.1*[0.1,0.2,0.3]  (optimizers.test.ts:151-164) */
+  const float p0[3] = {1.0f, 2.0f, 3.0f}, g0[3] = {0.1f, 0.2f, 0.3f};
+  float *p = to_device(p0, 3), *g = to_device(g0, 3), *out = to_device(p0, 3);
+  mxopt_optimizer* sgd = NULL;
+  CHECK_MX(mxopt_sgd_new(ctx, 0.1, NULL, NULL, NULL, NULL, &sgd));
+  mxopt_array ap = {p, 3, MXOPT_F32}, ag = {g, 3, MXOPT_F32}, ao = {out, 3, MXOPT_F32};
+  CHECK_MX(mxopt_optimizer_update_single(sgd, "param", &ap, &ag, &ao));
+  const double want_sgd[3] = {0.99, 1.98, 2.97};
+  expect_close("SGD basic step", out, want_sgd, 3, 5e-6);
+  mxopt_optimizer_free(sgd);
+
+  /* Nesterov without momentum is refused with InvalidArg (optimizers.test.ts:205-214) */
+  const int yes = 1;
+  const double zero = 0.0;
+  if (mxopt_sgd_new(ctx, 0.1, &zero, NULL, NULL, &yes, &sgd) != MXOPT_ERR_INVALID_ARG) {
+    fprintf(stderr, "FAIL: invalid Nesterov configuration was accepted\n");
+    exit(1);
+  }
+  printf("PASS SGD rejects Nesterov without momentum: %s\n", mxopt_last_error(ctx));
+
+  /* clip_grad_norm: [3,4] has norm 5, max 2.5 halves it (optimizers.test.ts:324-351) */
+  const float g1[2] = {3.0f, 4.0f};
+  float *dg = to_device(g1, 2), *dc = to_device(g1, 2);
+  mxopt_array cg = {dg, 2, MXOPT_F32}, co = {dc, 2, MXOPT_F32};
+  double norm = 0.0;
+  CHECK_MX(mxopt_clip_grad_norm(ctx, 1, &cg, 2.5, &co, &norm));
+  const double want_clip[2] = {1.5, 2.0};
+  expect_close("clip_grad_norm halves [3,4]", dc, want_clip, 2, 5e-6);
+  if (fabs(norm - 5.0) > 1e-5) { fprintf(stderr, "FAIL norm %.9g\n", norm); exit(1); }
+
+  /* GRPO engine, N = 4, lr 0.01, clips off: [10,20] - 0.0025*[10,14]
+   * (__test__/trainers/grpo-gradient-accumulation.test.ts:134-171) */
+  const float w0[2] = {10.0f, 20.0f};
+  const float gs[4][2] = {{1, 2}, {2, 3}, {3, 4}, {4, 5}};
+  float* w = to_device(w0, 2);
+  mxopt_engine_config cfg;
+  mxopt_engine_config_default(MXOPT_ENGINE_GRPO, &cfg);
+  cfg.learning_rate = 0.01;
+  cfg.gradient_accumulation_steps = 4;
+  cfg.has_gradient_clip_norm = 0;
+  cfg.gradient_clip_value = 100.0;
+  const char* names[1] = {"w"};
+  mxopt_array aw = {w, 2, MXOPT_F32};
+  mxopt_engine* eng = NULL;
+  CHECK_MX(mxopt_engine_new(ctx, &cfg, 1, names, &aw, &eng));
+  mxopt_engine_metrics m;
+  for (int k = 0; k < 4; ++k) {
+    float* d = to_device(gs[k], 2);
+    mxopt_array a = {d, 2, MXOPT_F32};
+    CHECK_MX(mxopt_engine_micro_batch(eng, 1, names, &a, &m));
+    if (m.gradients_applied != (k == 3) || m.step != k + 1) { fprintf(stderr, "FAIL engine bookkeeping at %d\n", k); exit(1); }
+    CHECK_MX(mxopt_synchronize(ctx));
+    CHECK_HIP(hipFree(d));
+  }
+  const double want_w[2] = {9.975, 19.965};
+  expect_close("GRPO engine: 4 micro-batches, lr/N", w, want_w, 2, 5e-6);
+  mxopt_engine_free(eng);
+}
+
+/* Qwen3-0.6B: vocab 151936, hidden 1024, 28 layers, q 2048x1024, k/v 1024x1024, o 1024x2048,
+ * gate/up 3072x1024, down 1024x3072, four norm vectors per layer, final norm, tied embedding. */
+static size_t qwen3_06b(size_t* sizes) {
+  size_t n = 0;
+  sizes[n++] = (size_t)151936 * 1024;
+  for (int l = 0; l < 28; ++l) {
+    sizes[n++] = 2048 * 1024; sizes[n++] = 1024 * 1024; sizes[n++] = 1024 * 1024; sizes[n++] = 1024 * 2048;
+    sizes[n++] = 3072 * 1024; sizes[n++] = 3072 * 1024; sizes[n++] = 1024 * 3072;
+    sizes[n++] = 1024; sizes[n++] = 1024; sizes[n++] = 128; sizes[n++] = 128;
+  }
+  sizes[n++] = 1024;
+  return n;
+}
+
+static void timing(void) {
+  size_t sizes[512];
+  const size_t nt = qwen3_06b(sizes);
+  size_t total = 0;
+  mxopt_array *p = calloc(nt, sizeof *p), *g = calloc(nt, sizeof *g);
+  char (*names)[32] = calloc(nt, 32);
+  const char** name_ptrs = calloc(nt, sizeof *name_ptrs);
+  for (size_t i = 0; i < nt; ++i) {
+    void *dp, *dg;
+    CHECK_HIP(hipMalloc(&dp, sizes[i] * 4));
+    CHECK_HIP(hipMalloc(&dg, sizes[i] * 4));
+    CHECK_HIP(hipMemset(dp, 0, sizes[i] * 4));
+    CHECK_HIP(hipMemset(dg, 0, sizes[i] * 4));
+    p[i] = (mxopt_array){dp, sizes[i], MXOPT_F32};
+    g[i] = (mxopt_array){dg, sizes[i], MXOPT_F32};
+    snprintf(names[i], 32, "t%zu", i);
+    name_ptrs[i] = names[i];
+    total += sizes[i];
+  }
+  mxopt_optimizer* opt = NULL;
+  CHECK_MX(mxopt_adamw_new(ctx, NULL, NULL, NULL, NULL, NULL, NULL, &opt));
+  const int steps = 20;
+  double wall[2], host[2];
+  for (int mode = 0; mode < 2; ++mode) {
+    double t0 = 0;
+    for (int it = -3; it < steps; ++it) {
+      if (it == 0) {
+        CHECK_MX(mxopt_synchronize(ctx));
+        t0 = now_ms();
+      }
+      if (mode == 0) {
+        for (size_t i = 0; i < nt; ++i) CHECK_MX(mxopt_optimizer_update_single(opt, names[i], &p[i], &g[i], &p[i]));
+      } else {
+        CHECK_MX(mxopt_optimizer_update_many(opt, nt, name_ptrs, p, g, p, NULL));
+      }
+    }
+    host[mode] = (now_ms() - t0) / steps;   /* time to enqueue */
+    CHECK_MX(mxopt_synchronize(ctx));
+    wall[mode] = (now_ms() - t0) / steps;   /* until the device has finished */
+  }
+  const double t_single = wall[0], t_many = wall[1], host_single = host[0] * steps, host_many = host[1] * steps;
+  printf("TIMING tensors=%zu elements=%zu update_single_loop_ms=%.3f (host enqueue %.3f) update_many_ms=%.3f "
+         "(host enqueue %.3f) bytes_per_step=%zu\n", nt, total, t_single, host_single / steps, t_many,
+         host_many / steps, total * 28);
+  mxopt_optimizer_free(opt);
+}
+
+int main(int argc, char** argv) {
+  CHECK_MX(mxopt_create(0, NULL, &ctx));
+  printf("%s\n", mxopt_version());
+  known_answers();
+  if (argc < 2 || strcmp(argv[1], "--no-timing") != 0) timing();
+  mxopt_destroy(ctx);
+  return 0;
+}
