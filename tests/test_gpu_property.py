@@ -1,0 +1,223 @@
+"""Property test of the update kernels: random table shapes (ragged sizes around the 8-element group
+and the 4096-element chunk, empty tensors), element shifts that are common to all streams or not,
+every dtype combination the kernels accept, every optimizer, every stage of the gradient
+pre-processing -- always bit for bit against the oracle.  Examples are derandomised: the same cases
+run every time."""
+import math
+
+import numpy as np
+import pytest
+from hypothesis import HealthCheck, given, settings
+from hypothesis import strategies as st
+
+pytestmark = pytest.mark.gpu
+
+import mxopt_oracle as O
+from gpu_util import assert_bit_equal, to_dev, to_host
+
+F = np.float32
+SIZES = st.one_of(st.integers(0, 20), st.integers(4088, 4104), st.integers(8185, 8200), st.integers(21, 30000))
+DTYPES = ["f32", "bf16", "f16"]
+
+
+def cast(x, dt):
+    return {"f32": lambda a: a.astype(F), "bf16": O.f32_to_bf16, "f16": lambda a: a.astype(np.float16)}[dt](x)
+
+
+def round_out(x, dt):
+    with np.errstate(over="ignore"):
+        return cast(np.asarray(x, F), dt)
+
+
+def torch_dtype(torch, dt):
+    return {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dt]
+
+
+def prep_oracle(g, pre_mul, clamp_pre, scale, clamp_post):
+    x = O.as_f32(g)
+    if pre_mul is not None:
+        x = x * F(pre_mul)
+    if clamp_pre is not None:
+        x = O.clip_value(x, -clamp_pre, clamp_pre)
+    pre = x
+    if scale is not None:
+        x = x * F(scale)
+    if clamp_post is not None:
+        x = O.clip_value(x, -clamp_post, clamp_post)
+    return pre, x
+
+
+@pytest.fixture(scope="module")
+def mx():
+    import mxopt
+    return mxopt
+
+
+@settings(max_examples=200, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@given(sizes=st.lists(SIZES, min_size=1, max_size=5), shift=st.integers(0, 9), common_shift=st.booleans(),
+       kind=st.sampled_from(["adam", "adamw", "adamw_bias", "sgd", "sgd_nesterov", "sgd_no_momentum", "rmsprop"]),
+       pd=st.sampled_from(DTYPES), gd=st.sampled_from(DTYPES), out_f32=st.booleans(), in_place=st.booleans(),
+       pre_mul=st.sampled_from([None, 0.25]), clamp_pre=st.sampled_from([None, 1.5e-3]),
+       clip=st.booleans(), clamp_post=st.sampled_from([None, 4e-4]), seed=st.integers(0, 2 ** 31))
+def test_update_kernels_match_the_oracle(mx, sizes, shift, common_shift, kind, pd, gd, out_f32, in_place, pre_mul,
+                                         clamp_pre, clip, clamp_post, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    od = "f32" if out_f32 else pd
+    in_place = in_place and od == pd
+    ctx = mx.default_context()
+    ps = [cast(rng.normal(0, 0.05, n).astype(F), pd) for n in sizes]
+    state_shift = shift if common_shift else 0
+    dp = [to_dev(p, shift) for p in ps]
+    do = dp if in_place else [torch.empty(n + 16, dtype=torch_dtype(torch, od), device="cuda")[state_shift:state_shift + n]
+                              for n in sizes]
+    dm = [to_dev(np.zeros(n, F), state_shift) for n in sizes]
+    dv = [to_dev(np.zeros(n, F), state_shift) for n in sizes]
+    dg = [torch.empty(n + 16, dtype=torch_dtype(torch, gd), device="cuda")[shift:shift + n] for n in sizes]
+    adam = kind.startswith("adam")
+    if adam:
+        bias = kind == "adamw_bias"
+        wd = None if kind == "adam" else 0.02
+        hp = mx.adam_hp(3e-3, 0.9, 0.99, 1e-8, wd)
+        ref = (O.Adam(3e-3, 0.9, 0.99, 1e-8, bias) if wd is None else O.AdamW(3e-3, 0.9, 0.99, 1e-8, wd, bias))
+        rows = [mx.TensorSpec(p=p, p_out=o, g=g, m=m, v=v) for p, o, g, m, v in zip(dp, do, dg, dm, dv)]
+    elif kind.startswith("sgd"):
+        mom = 0.0 if kind == "sgd_no_momentum" else 0.9
+        nest = kind == "sgd_nesterov"
+        hp = mx.sgd_hp(2e-2, mom, 1e-3, 0.0, nest)
+        ref = O.SGD(2e-2, mom, 1e-3, 0.0, nest)
+        rows = [mx.TensorSpec(p=p, p_out=o, g=g, v=(v if mom else None), flags=mx.TF_FIRST)
+                for p, o, g, v in zip(dp, do, dg, dv)]
+    else:
+        hp = mx.rmsprop_hp(1e-3, 0.95, 1e-8, 0.01)
+        ref = O.RMSprop(1e-3, 0.95, 1e-8, 0.01)
+        rows = [mx.TensorSpec(p=p, p_out=o, g=g, v=v) for p, o, g, v in zip(dp, do, dg, dv)]
+    table = ctx.table(rows)
+    t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
+    res = ctx.norm_result()
+    cur = list(ps)
+    step = 0
+    for it in range(2):
+        gs = [cast(rng.normal(0, 1e-3, n).astype(F), gd) for n in sizes]
+        for d, g in zip(dg, gs):
+            d.copy_(to_dev(g))
+        scale = None
+        if clip:
+            pre_only = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None)
+            ctx.global_norm(t_g, res, prep=pre_only, max_norm=5e-3)
+            r = ctx.read_norm_result(res)
+            exact = O.exact_sumsq([prep_oracle(g, pre_mul, clamp_pre, None, None)[0] for g in gs])
+            assert abs(r.sumsq - exact) <= 1e-6 * exact + 1e-300
+            assert F(r.scale) == O.norm_scale_c1(r.sumsq, 5e-3)[1]
+            scale = r.scale
+        prep = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None,
+                            scale=res if clip else None, clamp_post=(-clamp_post, clamp_post) if clamp_post else None)
+        if adam and kind == "adamw_bias":
+            bcs = [mx.bias_correction(0.9, 0.99, step + i + 1) for i in range(len(sizes))]
+            table.set_step_scalars([a for a, _ in bcs], [b for _, b in bcs])
+        if kind.startswith("sgd") and it == 1:
+            table.set_step_scalars(flags=[0] * len(sizes))
+        step += len(sizes)
+        if adam:
+            ctx.adam(table, hp, prep)
+        elif kind.startswith("sgd"):
+            ctx.sgd(table, hp, prep)
+        else:
+            ctx.rmsprop(table, hp, prep)
+        for i, n in enumerate(sizes):
+            g_eff = prep_oracle(gs[i], pre_mul, clamp_pre, scale, clamp_post)[1]
+            want = round_out(ref.update_single(str(i), cur[i], g_eff), od)
+            what = f"{kind} {pd}/{gd}->{od} n={n} shift={shift}/{state_shift} it={it} tensor {i}"
+            assert_bit_equal(to_host(do[i]), want, what)
+            if in_place:
+                cur[i] = want
+        ctx.synchronize()
+    table.close()
+    t_g.close()
+
+
+@settings(max_examples=150, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@given(sizes=st.lists(SIZES, min_size=1, max_size=5), shift=st.integers(0, 9), gd=st.sampled_from(DTYPES),
+       acc_f32=st.booleans(), pre_mul=st.sampled_from([None, 0.5]), clamp=st.sampled_from([None, 1.2e-3]),
+       poison=st.sampled_from([None, "nan", "inf", "-inf"]), seed=st.integers(0, 2 ** 31))
+def test_accumulation_and_transform_kernels_match_the_oracle(mx, sizes, shift, gd, acc_f32, pre_mul, clamp, poison, seed):
+    """acc = g0; acc += g1 with the norm of the new sum fused; the same sum measured without being
+    written (norm-only); acc2 = T(g0) + T(g1) with T = clamp and clip; g_out = T(g).  A NaN/Inf element
+    must raise the flag, also when the clamp would hide it, and then nothing may be written."""
+    import torch
+    rng = np.random.default_rng(seed)
+    ad = "f32" if acc_f32 else gd
+    ctx = mx.default_context()
+    g0 = [cast(rng.normal(0, 1e-3, n).astype(F), gd) for n in sizes]
+    g1 = [cast(rng.normal(0, 1e-3, n).astype(F), gd) for n in sizes]
+    total = sum(sizes)
+    if poison and total:
+        i = int(np.argmax(sizes))
+        v = O.as_f32(g1[i]).copy()
+        v[sizes[i] // 2] = {"nan": np.nan, "inf": np.inf, "-inf": -np.inf}[poison]
+        g1[i] = cast(v, gd)
+    dg = [torch.empty(n + 16, dtype=torch_dtype(torch, gd), device="cuda")[shift:shift + n] for n in sizes]
+    da = [torch.full((n + 16,), float("nan"), dtype=torch_dtype(torch, ad), device="cuda")[shift:shift + n] for n in sizes]
+    t_acc = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(dg, da)])
+    res = ctx.norm_result()
+    pre = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp, clamp) if clamp else None)
+
+    def load(gs):
+        for d, g in zip(dg, gs):
+            d.copy_(to_dev(g))
+
+    def add(a, b):          # promote(acc, g): equal 16-bit dtypes round the sum to that dtype
+        s = O.as_f32(a) + O.as_f32(b)
+        return round_out(s, ad)
+
+    load(g0)
+    ctx.accumulate(t_acc, first=True)
+    acc0 = [round_out(O.as_f32(g), ad) for g in g0]
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(da[i]), acc0[i], f"first {i}")
+    load(g1)
+    ctx.accumulate_norm_only(t_acc, res, prep=pre, max_norm=2e-3)
+    r_only = ctx.read_norm_result(res)
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(da[i]), acc0[i], f"norm-only wrote {i}")
+    ctx.accumulate(t_acc, first=False, out=res, prep=pre, max_norm=2e-3)
+    r = ctx.read_norm_result(res)
+    acc1 = [add(a, g) for a, g in zip(acc0, g1)]
+    for i in range(len(sizes)):
+        assert_bit_equal(to_host(da[i]), acc1[i], f"sum {i}")
+    bad = poison is not None and total > 0
+    assert r.nonfinite == int(bad) and r_only.nonfinite == int(bad)
+    if not bad:
+        exact = O.exact_sumsq([prep_oracle(a, pre_mul, clamp, None, None)[0] for a in acc1])
+        assert abs(r.sumsq - exact) <= 1e-6 * exact + 1e-300 and r.sumsq == r_only.sumsq
+        assert F(r.scale) == O.norm_scale_c1(r.sumsq, 2e-3)[1]
+
+    # clip-then-accumulate (float32 buffer) and the plain transform, with the skip flag wired in
+    db = [torch.full((n + 16,), 7.0, dtype=torch.float32, device="cuda")[shift:shift + n] for n in sizes]
+    dt = [torch.full((n + 16,), 7.0, dtype=torch.float32, device="cuda")[shift:shift + n] for n in sizes]
+    t_b = ctx.table([mx.TensorSpec(g=g, g_out=b) for g, b in zip(dg, db)])
+    t_t = ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(dg, dt)])
+    t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
+    want_b = None
+    for k, gs in enumerate((g0, g1)):
+        load(gs)
+        ctx.global_norm(t_g, res, prep=pre, max_norm=1e-3)
+        rk = ctx.read_norm_result(res)
+        full = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp, clamp) if clamp else None, scale=res,
+                            skip_if_nonfinite=res)
+        ctx.accumulate_transformed(t_b, first=(k == 0), prep=full)
+        ctx.grad_transform(t_t, full)
+        if k == 1 and bad:
+            assert rk.nonfinite == 1
+            for i in range(len(sizes)):     # skipped: still what the first micro-batch left
+                assert_bit_equal(to_host(db[i]), want_b[i], f"skipped accumulate {i}")
+                assert_bit_equal(to_host(dt[i]), want_t[i], f"skipped transform {i}")
+            break
+        tg = [prep_oracle(g, pre_mul, clamp, rk.scale, None)[1] for g in gs]
+        want_b = tg if k == 0 else [a + b for a, b in zip(want_b, tg)]
+        want_t = tg
+        for i in range(len(sizes)):
+            assert_bit_equal(to_host(db[i]), want_b[i], f"transformed accumulate {k} {i}")
+            assert_bit_equal(to_host(dt[i]), want_t[i], f"transform {k} {i}")
+    for t in (t_acc, t_b, t_t, t_g):
+        t.close()
