@@ -455,3 +455,62 @@ def test_error_cases(mx):
         a.update_single("v", arr(1, 2), arr(1, 2), out=torch.zeros(2, dtype=torch.float16, device="cuda"))
     with pytest.raises(ValueError):
         mx.Adam().update_single("w", torch.zeros(2), torch.zeros(2))   # host tensors: no CPU path
+
+
+# ---- __test__/core/training-demo-simple.test.ts ------------------------------------------------
+
+def test_demo_quadratic_with_four_optimizers(mx):  # :6-50
+    opts = {"adam": mx.Adam(0.1), "adamw": mx.AdamW(0.1, 0.9, 0.999, 1e-8, 0.01), "sgd": mx.SGD(0.1),
+            "sgdMomentum": mx.SGD(0.1, 0.9)}
+    refs = {"adam": O.Adam(0.1), "adamw": O.AdamW(0.1, 0.9, 0.999, 1e-8, 0.01), "sgd": O.SGD(0.1),
+            "sgdMomentum": O.SGD(0.1, 0.9)}
+    for name, opt in opts.items():
+        params, rp = arr(0.0, 0.0), np.zeros(2, F)
+        traj = []
+        for _ in range(50):
+            v = vals(params)
+            grad = np.array([2 * (v[0] - 2), 2 * (v[1] - 3)], F)      # f = (x-2)^2 + (y-3)^2
+            params = opt.update_single(f"{name}_params", params, to_dev(grad))
+            rp = refs[name].update_single(f"{name}_params", rp, grad)
+            assert_bit_equal(vals(params), rp, name)                    # and the whole trajectory is the oracle's
+            nv = vals(params)
+            traj.append(math.hypot(nv[0] - 2, nv[1] - 3))
+        assert traj[-1] < 0.5 and traj[-1] < traj[0], name
+
+
+def test_demo_learning_rate_schedule(mx):  # :91-140
+    rng = np.random.default_rng(0)
+    w, b = arr(0.0), arr(0.0)
+    losses = []
+    for step in range(100):
+        lr = mx.LRScheduler.cosine_annealing(0.1, 0.001, step, 100)
+        sgd = mx.SGD(lr)
+        x = rng.uniform(-1, 1, 10).astype(F)
+        y = 2 * x + 1
+        diff = x * vals(w)[0] + vals(b)[0] - y
+        losses.append(float((diff ** 2).mean()))
+        w = sgd.update_single("weight", w, arr(2 * float((x * diff).mean())))
+        b = sgd.update_single("bias", b, arr(2 * float(diff.mean())))
+    assert abs(vals(w)[0] - 2.0) < 0.5 and abs(vals(b)[0] - 1.0) < 0.5
+    assert sum(losses[-10:]) < sum(losses[:10])
+
+
+def test_demo_gradient_clipping(mx):  # :142-165
+    clipped = mx.GradientUtils.clip_grad_value(arr(10.0, -15.0, 20.0), -5.0, 5.0)
+    c = vals(clipped)
+    assert close(c[0], 5.0) and close(c[1], -5.0) and close(c[2], 5.0)
+    u = vals(mx.Adam(0.01).update_single("param", arr(1.0, 2.0, 3.0), clipped))
+    assert all(abs(u[i] - [1.0, 2.0, 3.0][i]) < 1.0 for i in range(3))
+
+
+def test_demo_weight_decay(mx):  # :220-251
+    no_wd, wd = mx.Adam(0.01), mx.AdamW(0.01, 0.9, 0.999, 1e-8, 0.1)
+    a, b = arr(10.0, 10.0), arr(10.0, 10.0)
+    z = arr(0.0, 0.0)
+    for _ in range(50):
+        a = no_wd.update_single("params", a, z)
+        b = wd.update_single("params", b, z)
+    va, vb = vals(a), vals(b)
+    assert close(va[0], 10.0, 2) and close(va[1], 10.0, 2)
+    assert vb[0] < va[0] and vb[1] < va[1]
+    assert abs(vb[0] - 10.0 * (1 - 0.01 * 0.1) ** 50) < 1e-4            # closed form of the decoupled decay
