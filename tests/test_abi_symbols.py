@@ -161,3 +161,20 @@ def test_tensor_layout_head_and_chunk_count(L):
     # streams that disagree: bf16 p one element in, float32 m on a boundary
     assert layout(5000, p=BASE + 2, g=BASE + 2, m=BASE + 65536, v=BASE + 131072) == (0, 0, 2)
     assert lib.mxopt_tensor_layout(None, None, None, None) == 1
+
+
+def test_engine_config_defaults_are_the_reference_defaults(L):
+    """GRPOEngineConfig::default (grpo/engine.rs:114-141) and SftEngineConfig::default (sft/engine.rs:50-66)."""
+    lib = L.load()
+    g, s = L.EngineConfig(), L.EngineConfig()
+    lib.mxopt_engine_config_default(L.ENGINE_GRPO, C.byref(g))
+    lib.mxopt_engine_config_default(L.ENGINE_SFT, C.byref(s))
+    assert (g.learning_rate, g.gradient_accumulation_steps, g.has_gradient_clip_norm, g.gradient_clip_norm,
+            g.has_gradient_clip_value, g.gradient_clip_value, g.max_nan_gradients, g.emergency_save_threshold,
+            g.apply) == (1e-6, 1, 1, 1.0, 1, 1.0, 100, 5, L.ENGINE_APPLY_SGD)
+    assert (s.learning_rate, s.gradient_accumulation_steps, s.has_gradient_clip_norm, s.gradient_clip_norm,
+            s.has_gradient_clip_value, s.weight_decay, s.max_nan_gradients, s.emergency_save_threshold,
+            s.apply) == (2e-5, 1, 1, 1.0, 0, 0.01, 100, 5, L.ENGINE_APPLY_SGD)
+    # entry points refuse a null engine without touching a device
+    assert lib.mxopt_engine_micro_batch(None, 0, None, None, None) == 1
+    assert lib.mxopt_engine_reset(None) == 1 and lib.mxopt_optimizer_save_file(None, b"/tmp/x") == 1
