@@ -361,11 +361,19 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
   const bool same = opt->many_table && key.size() == opt->many_key.size() &&
                     (key.empty() || std::memcmp(key.data(), opt->many_key.data(), key.size() * sizeof(mxopt_tensor)) == 0);
   if (!same) {
+    // The same tensors in other buffers (a functional host hands back new arrays every step): keep the
+    // chunk list and swap the pointers; anything else is a new table.
+    bool moved = false;
     if (opt->many_table) {
-      mxopt_table_destroy(opt->many_table);
-      opt->many_table = nullptr;
+      const std::string saved = ctx->err;
+      moved = mxopt_table_retarget(opt->many_table, rows.data(), rows.size()) == MXOPT_OK;
+      if (!moved) {
+        ctx->err = saved;
+        mxopt_table_destroy(opt->many_table);
+        opt->many_table = nullptr;
+      }
     }
-    if ((rc = mxopt_table_build(ctx, rows.data(), rows.size(), &opt->many_table))) return rc;
+    if (!moved && (rc = mxopt_table_build(ctx, rows.data(), rows.size(), &opt->many_table))) return rc;
     opt->many_key = std::move(key);
   } else {
     bool scalars_differ = false;
