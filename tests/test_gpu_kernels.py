@@ -645,3 +645,48 @@ def test_table_retarget(mx, ctx):
     for i in range(len(sizes)):
         assert_bit_equal(to_host(dp[i]), O.f32_to_bf16(ref2.update_single(str(i), before[i], gs[i])), f"after refusal p{i}")
     table.close()
+
+
+# ---------------------------------------------------------------------------------
+# Subnormal float32 intermediates (g*g around 1e-40, sqrt and divide of such values) are kept, as a
+# CPU float32 op chain keeps them: nothing is flushed to zero.
+# ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("kind", ["adamw", "rmsprop", "sgd"])
+def test_subnormal_intermediates(mx, ctx, kind):
+    import torch
+    rng = np.random.default_rng(77)
+    n = 9001
+    p = rng.normal(0, 1e-18, n).astype(F)
+    g = (rng.normal(0, 1, n) * 10.0 ** rng.uniform(-24, -18, n)).astype(F)     # squares between 1e-48 and 1e-36
+    g[:16] = (rng.normal(0, 1, 16) * 1e-41).astype(F)                           # subnormal gradients themselves
+    assert (np.abs(g[:16]) < np.finfo(F).tiny).any()
+    dp, dg = to_dev(p), to_dev(g)
+    dm = torch.zeros(n, dtype=torch.float32, device="cuda")
+    dv = torch.zeros(n, dtype=torch.float32, device="cuda")
+    do = torch.empty(n, dtype=torch.float32, device="cuda")
+    if kind == "adamw":
+        ref, run = O.AdamW(1e-3, 0.9, 0.999, 1e-30, 0.01), lambda t: ctx.adam(t, mx.adam_hp(1e-3, 0.9, 0.999, 1e-30, 0.01))
+        row = mx.TensorSpec(p=dp, p_out=do, g=dg, m=dm, v=dv)
+    elif kind == "rmsprop":
+        ref, run = O.RMSprop(1e-3, 0.99, 1e-30, 0.0), lambda t: ctx.rmsprop(t, mx.rmsprop_hp(1e-3, 0.99, 1e-30, 0.0))
+        row = mx.TensorSpec(p=dp, p_out=do, g=dg, v=dv)
+    else:
+        ref, run = O.SGD(1e-3, 0.9, 1e-4), lambda t: ctx.sgd(t, mx.sgd_hp(1e-3, 0.9, 1e-4))
+        row = mx.TensorSpec(p=dp, p_out=do, g=dg, v=dv, flags=mx.TF_FIRST)
+    table = ctx.table([row])
+    cur = p
+    for it in range(3):
+        if kind == "sgd" and it == 1:
+            table.set_step_scalars(flags=[0])
+        run(table)
+        with np.errstate(under="ignore"):
+            cur = ref.update_single("w", cur, g)
+        assert_bit_equal(to_host(do), cur, f"{kind} it {it}")
+        state = ref.state["w"]
+        v_ref = state[1] if isinstance(state, tuple) else state
+        assert_bit_equal(to_host(dv), v_ref, f"{kind} v it {it}")
+        if kind == "adamw":
+            assert (np.abs(v_ref[v_ref != 0]) < np.finfo(F).tiny).any()        # the test does reach subnormals
+        dp.copy_(do)
+    table.close()
