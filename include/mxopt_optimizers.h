@@ -101,6 +101,12 @@ int mxopt_optimizer_load_state(mxopt_optimizer* opt, const char* param_name, con
  * optimizer's current state and refuses a file written for another optimizer kind. */
 int mxopt_optimizer_save_file(mxopt_optimizer* opt, const char* path);
 int mxopt_optimizer_load_file(mxopt_optimizer* opt, const char* path);
+/* Host-only look at a checkpoint (no device, no optimizer needed): which optimizer kind wrote it
+ * ("adam", "adamw", "sgd", "rmsprop"), its call counter, how many tensors and float32 elements it
+ * holds.  Fails like load_file on anything that is not a well-formed checkpoint.  Any out pointer
+ * may be NULL. */
+int mxopt_checkpoint_inspect(const char* path, char* optimizer, size_t optimizer_capacity, int64_t* step,
+                             uint64_t* tensors, uint64_t* elements);
 
 /* ---- GradientUtils (optimizers/mod.rs:33-227) -------------------------------------- */
 /* compute_gradient_norm (:43-55): sqrt of the float64 sum of squares.  Synchronises. */

@@ -195,54 +195,96 @@ int save_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int
   return MXOPT_OK;
 }
 
+namespace {
+
+struct Entry { std::string key; uint64_t begin, end; };
+
+// Reads and validates the header: format tag, optimizer kind, step, and every tensor's byte range
+// against the size of the file.  No device involved.
+int read_header(mxopt_ctx* ctx, FILE* f, const char* path, std::string* optimizer, int64_t* step,
+                std::vector<Entry>* entries, uint64_t* data_start) {
+  unsigned char le[8];
+  if (std::fread(le, 1, 8, f) != 8) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: file is too short");
+  uint64_t hlen = 0;
+  for (int i = 0; i < 8; ++i) hlen |= (uint64_t)le[i] << (8 * i);
+  if (hlen < 2 || hlen > (256u << 20)) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: implausible header length");
+  std::string header(hlen, '\0');
+  if (std::fread(&header[0], 1, hlen, f) != hlen) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: truncated header");
+  JsonReader rd{header.data(), header.data() + header.size()};
+  const Json root = rd.value();
+  if (!rd.ok || root.type != Json::Object) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: header is not a JSON object");
+  const Json* meta = root.get("__metadata__");
+  const Json* fmt = meta && meta->type == Json::Object ? meta->get("format") : nullptr;
+  if (!fmt || fmt->string != "mxopt-optimizer-state")
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: not an optimizer-state checkpoint");
+  const Json* kind = meta->get("optimizer");
+  *optimizer = kind ? kind->string : "";
+  const Json* st = meta->get("step");
+  if (step) *step = st ? std::strtoll(st->string.c_str(), nullptr, 10) : 0;
+  if (std::fseek(f, 0, SEEK_END) != 0) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: seek failed");
+  const long size = std::ftell(f);
+  if (size < 0 || (uint64_t)size < 8 + hlen) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: truncated header");
+  const uint64_t data_bytes = (uint64_t)size - 8 - hlen;  // the file size bounds every offset
+  *data_start = 8 + hlen;
+  for (const auto& kv : root.object) {
+    if (kv.first == "__metadata__") continue;
+    const Json* dt = kv.second.type == Json::Object ? kv.second.get("dtype") : nullptr;
+    const Json* off = kv.second.type == Json::Object ? kv.second.get("data_offsets") : nullptr;
+    if (!dt || !off || off->array.size() != 2 || off->array[0].type != Json::Number || off->array[1].type != Json::Number)
+      return fail(ctx, MXOPT_ERR_FAILURE, "load_file: malformed entry '" + kv.first + "'");
+    if (dt->string != "F32") return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: '" + kv.first + "' is not float32");
+    const double da = off->array[0].number, db = off->array[1].number;
+    if (!(da >= 0) || !(db >= da) || db > (double)data_bytes)
+      return fail(ctx, MXOPT_ERR_FAILURE, "load_file: '" + kv.first + "' has offsets outside the file");
+    const uint64_t a = (uint64_t)da, b = (uint64_t)db;
+    if ((b - a) % 4) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: '" + kv.first + "' is not a whole number of floats");
+    entries->push_back({kv.first, a, b});
+  }
+  (void)path;
+  return MXOPT_OK;
+}
+
+}  // namespace
+
+int inspect_state_file(const char* path, std::string* optimizer, int64_t* step, uint64_t* tensors, uint64_t* elements) {
+  if (!path) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "checkpoint_inspect: path is NULL");
+  FileCloser file{std::fopen(path, "rb")};
+  if (!file.f) return fail(nullptr, MXOPT_ERR_FAILURE, std::string("load_file: cannot open ") + path);
+  std::vector<Entry> entries;
+  uint64_t data_start = 0;
+  int rc = read_header(nullptr, file.f, path, optimizer, step, &entries, &data_start);
+  if (rc) return rc;
+  if (tensors) *tensors = entries.size();
+  if (elements) {
+    *elements = 0;
+    for (const Entry& e : entries) *elements += (e.end - e.begin) / 4;
+  }
+  return MXOPT_OK;
+}
+
 int load_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int64_t* step,
                     const std::function<int(const std::string& key, uint64_t n, float** device)>& place) {
   if (!path) return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: path is NULL");
   FileCloser file{std::fopen(path, "rb")};
   if (!file.f) return fail(ctx, MXOPT_ERR_FAILURE, std::string("load_file: cannot open ") + path);
-  unsigned char le[8];
-  if (std::fread(le, 1, 8, file.f) != 8) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: file is too short");
-  uint64_t hlen = 0;
-  for (int i = 0; i < 8; ++i) hlen |= (uint64_t)le[i] << (8 * i);
-  if (hlen < 2 || hlen > (256u << 20)) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: implausible header length");
-  std::string header(hlen, '\0');
-  if (std::fread(&header[0], 1, hlen, file.f) != hlen) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: truncated header");
-  JsonReader rd{header.data(), header.data() + header.size()};
-  const Json root = rd.value();
-  if (!rd.ok || root.type != Json::Object) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: header is not a JSON object");
-  const Json* meta = root.get("__metadata__");
-  const Json* fmt = meta ? meta->get("format") : nullptr;
-  if (!fmt || fmt->string != "mxopt-optimizer-state")
-    return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: not an optimizer-state checkpoint");
-  const Json* kind = meta->get("optimizer");
-  if (!kind || kind->string != optimizer)
-    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("load_file: checkpoint is for optimizer '") +
-                (kind ? kind->string : "?") + "', this one is '" + optimizer + "'");
-  const Json* st = meta->get("step");
-  if (step) *step = st ? std::strtoll(st->string.c_str(), nullptr, 10) : 0;
-
-  // file size bounds every offset
-  if (std::fseek(file.f, 0, SEEK_END) != 0) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: seek failed");
-  const uint64_t data_bytes = (uint64_t)std::ftell(file.f) - 8 - hlen;
+  std::vector<Entry> entries;
+  std::string kind;
+  uint64_t data_start = 0;
+  int rc = read_header(ctx, file.f, path, &kind, step, &entries, &data_start);
+  if (rc) return rc;
+  if (kind != optimizer)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("load_file: checkpoint is for optimizer '") + kind +
+                "', this one is '" + optimizer + "'");
   DeviceGuard guard(ctx->device);
   Staging stage;
-  int rc = stage.ensure(ctx);
-  if (rc) return rc;
-  for (const auto& kv : root.object) {
-    if (kv.first == "__metadata__") continue;
-    const Json* dt = kv.second.get("dtype");
-    const Json* off = kv.second.get("data_offsets");
-    if (!dt || !off || off->array.size() != 2)
-      return fail(ctx, MXOPT_ERR_FAILURE, "load_file: malformed entry '" + kv.first + "'");
-    if (dt->string != "F32") return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: '" + kv.first + "' is not float32");
-    const uint64_t a = (uint64_t)off->array[0].number, b = (uint64_t)off->array[1].number;
-    if (b < a || b > data_bytes || (b - a) % 4)
-      return fail(ctx, MXOPT_ERR_FAILURE, "load_file: '" + kv.first + "' has offsets outside the file");
+  if ((rc = stage.ensure(ctx))) return rc;
+  for (const Entry& entry : entries) {
+    const uint64_t a = entry.begin, b = entry.end;
     const uint64_t n = (b - a) / 4;
     float* dst = nullptr;
-    if ((rc = place(kv.first, n, &dst))) return rc;
+    if ((rc = place(entry.key, n, &dst))) return rc;
     if (!dst || !n) continue;
-    if (std::fseek(file.f, (long)(8 + hlen + a), SEEK_SET) != 0) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: seek failed");
+    if (std::fseek(file.f, (long)(data_start + a), SEEK_SET) != 0) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: seek failed");
     char* d = (char*)dst;
     uint64_t left = b - a;
     while (left) {

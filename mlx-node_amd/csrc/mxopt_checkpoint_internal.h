@@ -25,4 +25,7 @@ int save_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int
 int load_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int64_t* step,
                     const std::function<int(const std::string& key, uint64_t n, float** device)>& place);
 
+// Header of a checkpoint without touching a device: optimizer kind, call counter, tensor and element counts.
+int inspect_state_file(const char* path, std::string* optimizer, int64_t* step, uint64_t* tensors, uint64_t* elements);
+
 }  // namespace mxopt

@@ -472,6 +472,18 @@ int mxopt_optimizer_save_file(mxopt_optimizer* opt, const char* path) {
   return save_state_file(opt->ctx, path, kind_name(opt->kind), opt->step, tensors);
 }
 
+int mxopt_checkpoint_inspect(const char* path, char* optimizer, size_t optimizer_capacity, int64_t* step,
+                             uint64_t* tensors, uint64_t* elements) {
+  std::string kind;
+  int rc = inspect_state_file(path, &kind, step, tensors, elements);
+  if (rc) return rc;
+  if (optimizer && optimizer_capacity) {
+    std::strncpy(optimizer, kind.c_str(), optimizer_capacity - 1);
+    optimizer[optimizer_capacity - 1] = '\0';
+  }
+  return MXOPT_OK;
+}
+
 int mxopt_optimizer_load_file(mxopt_optimizer* opt, const char* path) {
   if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "optimizer_load_file: null optimizer");
   free_state(opt);  // a checkpoint replaces whatever state there was

@@ -134,6 +134,8 @@ SIGNATURES.update({
                                              C.c_int64]),
     "mxopt_optimizer_save_file": (C.c_int, [C.c_void_p, C.c_char_p]),
     "mxopt_optimizer_load_file": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "mxopt_checkpoint_inspect": (C.c_int, [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_int64),
+                                           C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "mxopt_compute_gradient_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, _PD]),
     "mxopt_clip_grad_norm": (C.c_int, [C.c_void_p, C.c_size_t, _PA, C.c_double, _PA, _PD]),
     "mxopt_clip_grad_value": (C.c_int, [C.c_void_p, _PA, C.c_double, C.c_double, _PA]),
