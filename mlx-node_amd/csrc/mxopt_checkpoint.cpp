@@ -201,7 +201,7 @@ struct Entry { std::string key; uint64_t begin, end; };
 
 // Reads and validates the header: format tag, optimizer kind, step, and every tensor's byte range
 // against the size of the file.  No device involved.
-int read_header(mxopt_ctx* ctx, FILE* f, const char* path, std::string* optimizer, int64_t* step,
+int read_header(mxopt_ctx* ctx, FILE* f, std::string* optimizer, int64_t* step,
                 std::vector<Entry>* entries, uint64_t* data_start) {
   unsigned char le[8];
   if (std::fread(le, 1, 8, f) != 8) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: file is too short");
@@ -240,7 +240,6 @@ int read_header(mxopt_ctx* ctx, FILE* f, const char* path, std::string* optimize
     if ((b - a) % 4) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: '" + kv.first + "' is not a whole number of floats");
     entries->push_back({kv.first, a, b});
   }
-  (void)path;
   return MXOPT_OK;
 }
 
@@ -252,7 +251,7 @@ int inspect_state_file(const char* path, std::string* optimizer, int64_t* step, 
   if (!file.f) return fail(nullptr, MXOPT_ERR_FAILURE, std::string("load_file: cannot open ") + path);
   std::vector<Entry> entries;
   uint64_t data_start = 0;
-  int rc = read_header(nullptr, file.f, path, optimizer, step, &entries, &data_start);
+  int rc = read_header(nullptr, file.f, optimizer, step, &entries, &data_start);
   if (rc) return rc;
   if (tensors) *tensors = entries.size();
   if (elements) {
@@ -270,7 +269,7 @@ int load_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int
   std::vector<Entry> entries;
   std::string kind;
   uint64_t data_start = 0;
-  int rc = read_header(ctx, file.f, path, &kind, step, &entries, &data_start);
+  int rc = read_header(ctx, file.f, &kind, step, &entries, &data_start);
   if (rc) return rc;
   if (kind != optimizer)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("load_file: checkpoint is for optimizer '") + kind +
