@@ -44,6 +44,7 @@ def build(verbose: bool = False) -> str:
         print(err)
     os.replace(LIB + ".tmp", LIB)
     build_demo(verbose)
+    build_napi(verbose)
     return LIB
 
 
@@ -63,6 +64,29 @@ def build_demo(verbose: bool = False) -> str:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
     return DEMO
+
+
+NAPI = os.path.join(HERE, "bin", "mxopt.node")
+
+
+def build_napi(verbose: bool = False):
+    """napi/mxopt_napi.c -> bin/mxopt.node (the JavaScript surface), when node's headers are installed."""
+    include = next((d for d in ("/usr/include/node", "/usr/local/include/node") if os.path.exists(os.path.join(d, "node_api.h"))),
+                   None)
+    if include is None:
+        if verbose:
+            print("node_api.h not found: the N-API binding is not built")
+        return None
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c11", "-O2", "-Wall", "-Werror", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(rocm, "include"), "-I", include,
+           os.path.join(HERE, "napi", "mxopt_napi.c"), "-o", NAPI, "-L", HERE, "-lmxopt",
+           "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-lm", "-Wl,-rpath,$ORIGIN/..",
+           "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return NAPI
 
 
 if __name__ == "__main__":
