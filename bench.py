@@ -168,7 +168,8 @@ class Workload:
                                      for p, a, m, v in zip(self.p, self.acc, self.m, self.v)])
         self.hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
         self.prep = mx.make_prep(scale=self.res)
-        self.dtype = "bf16 params/grads, f32 accumulate + moments + arithmetic"
+        self.dtype = "f32"
+        self.storage = "bf16 parameters and gradients, float32 accumulation buffer and moments"
         self.fold_last = bool(self.args.fold_last)
         if self.fold_last:
             # the update reads the accumulation buffer AND the last micro-batch (24 + 2 B/elem); the last
@@ -259,7 +260,8 @@ class Workload:
                                      for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
         self.hp = mx.adam_hp(lr, 0.9, 0.999, 1e-8, wd)
         self.prep = mx.make_prep(scale=self.res)
-        self.dtype = "bf16 params/grads, f32 moments + arithmetic"
+        self.dtype = "f32"
+        self.storage = "bf16 parameters and gradients, float32 moments"
         self.bytes_per_elem = {"global_norm": 2, "adamw": 22}
         self.step_bytes_per_elem = 24
         self.dominant = "adamw"
@@ -331,7 +333,8 @@ class Workload:
         self.step_bytes_per_elem = (self.bytes_per_elem["micro_batch_first"] + 2 * self.bytes_per_elem["micro_batch"] +
                                     self.bytes_per_elem["micro_batch_apply"])
         self.dominant = "micro_batch_apply"
-        self.dtype = "bf16 params/grads, f32 accumulate + arithmetic"
+        self.dtype = "f32"
+        self.storage = "bf16 parameters and gradients, float32 accumulation buffer"
 
     def _setup_grpo_engine(self):
         self._setup_engine("grpo")
@@ -501,7 +504,8 @@ def main():
         "ms_per_step_min": round(step_ms[0], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
-                   "bytes_per_elem_per_step": wl.step_bytes_per_elem, "note": wl.note, "scale": args.scale,
+                   "bytes_per_elem_per_step": wl.step_bytes_per_elem,
+                   "storage": getattr(wl, "storage", "float32 everywhere"), "note": wl.note, "scale": args.scale,
                    "alloc": args.alloc},
         "elements_per_s": round(n * steps_per_s, 1),
         "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
