@@ -42,7 +42,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg5",
                     choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
                              "cfg4", "cfg4-flat", "cfg5", "copy", "grpo-engine", "sft-engine"])
-    ap.add_argument("--cpu-sample", type=int, default=128 * 1024 * 1024,
+    ap.add_argument("--cpu-sample", type=int, default=512 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
                     help="shrink every tensor's first dimension (for quick runs; invalid as a result)")
