@@ -89,5 +89,32 @@ def build_napi(verbose: bool = False):
     return NAPI
 
 
+SANITY = os.path.join(HERE, "bin", "host_sanity_asan")
+
+
+def build_sanitized(verbose: bool = False) -> str:
+    """examples/host_sanity.cpp + the whole host layer under AddressSanitizer and UBSan (host code only;
+    the device pass is not instrumented).  Not part of the default build: it takes a couple of minutes.
+    Run with ASAN_OPTIONS=detect_leaks=0 (the HIP runtime keeps its own allocations)."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    os.makedirs(os.path.dirname(SANITY), exist_ok=True)
+    srcs = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(HERE, "examples", "host_sanity.cpp")]
+    cmd = [hipcc, "--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-ffp-contract=off",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+           "-Xarch_host", "-fno-sanitize-recover=undefined",
+           "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-x", "hip"] + srcs + ["-o", SANITY]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write("\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l) + "\n")
+        raise RuntimeError("sanitized build failed")
+    return SANITY
+
+
 if __name__ == "__main__":
-    print(build(verbose=True))
+    if "--sanitize" in sys.argv:
+        print(build_sanitized(verbose=True))
+    else:
+        print(build(verbose=True))
