@@ -221,3 +221,51 @@ def test_accumulation_and_transform_kernels_match_the_oracle(mx, sizes, shift, g
             assert_bit_equal(to_host(dt[i]), want_t[i], f"transform {k} {i}")
     for t in (t_acc, t_b, t_t, t_g):
         t.close()
+
+
+@settings(max_examples=120, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@given(sizes=st.lists(SIZES, min_size=1, max_size=4), bf16=st.booleans(), max_norm=st.sampled_from([1e-3, 3e-2, 10.0]),
+       clip_val=st.sampled_from([2e-4, 1.0]), lr=st.sampled_from([1e-6, 2e-5, 0.3]), seed=st.integers(0, 2 ** 31))
+def test_host_layer_utilities_match_the_oracle(mx, sizes, bf16, max_norm, clip_val, lr, seed):
+    """GradientUtils, the Vec clip API, accumulate_gradients and apply_gradients over name-keyed maps of
+    random shape, against the oracle (clip outputs given the device's norm, everything else bit for bit)."""
+    rng = np.random.default_rng(seed)
+    dt = "bf16" if bf16 else "f32"
+    names = [f"t{i}" for i in range(len(sizes))]
+    gs = {k: cast(rng.normal(0, 1e-3, n).astype(F), dt) for k, n in zip(names, sizes)}
+    ps = {k: cast(rng.normal(0, 0.5, n).astype(F), dt) for k, n in zip(names, sizes)}
+    dg = {k: to_dev(v) for k, v in gs.items()}
+    exact = O.GradientUtils.compute_gradient_norm(gs)
+    got = mx.GradientUtils.compute_gradient_norm(dg)
+    assert abs(got - exact) <= 1e-5 * exact + 1e-30
+    # clip by norm (always multiplies) and the Vec API (unchanged when below)
+    clipped, n32 = mx.GradientUtils.clip_grad_norm_with_norm(dg, max_norm)
+    assert abs(n32 - exact) <= 1e-5 * exact + 1e-30
+    _, scale = O.norm_scale_c1(float(n32) ** 2, max_norm)
+    for k in names:
+        want = O.as_f32(gs[k]) * scale
+        assert np.allclose(to_host(clipped[k]), want, rtol=3e-7, atol=0), k
+    vec = mx.clip_gradients_by_global_norm([dg[k] for k in names], max_norm)
+    want_vec = O.clip_gradients_by_global_norm([gs[k] for k in names], max_norm)
+    for k, g, w in zip(names, vec, want_vec):
+        assert np.allclose(O.as_f32(to_host(g)), O.as_f32(w), rtol=3e-7, atol=0), k
+    # clamp: bit for bit, NaN kept
+    for k in names[:2]:
+        assert_bit_equal(to_host(mx.GradientUtils.clip_grad_value(dg[k], -clip_val, clip_val)),
+                         O.clip_value(gs[k], -clip_val, clip_val), f"clamp {k}")
+    # accumulate three times through the map API, with a name that appears late and one that stops
+    acc_d, acc_o = {}, {}
+    for it in range(3):
+        keep = names if it != 1 else names[:-1] or names
+        new_o = {k: cast(rng.normal(0, 1e-3, sizes[names.index(k)]).astype(F), dt) for k in keep}
+        acc_d = mx.accumulate_gradients(acc_d, {k: to_dev(v) for k, v in new_o.items()})
+        acc_o = O.accumulate_gradients(acc_o, new_o)
+    assert set(acc_d) == set(acc_o)
+    for k in acc_o:
+        assert_bit_equal(to_host(acc_d[k]), acc_o[k], f"accumulated {k}")
+    # apply: plain SGD in the parameter's dtype, in place
+    dp = {k: to_dev(v) for k, v in ps.items()}
+    mx.apply_gradients(dp, acc_d, lr)
+    want_p = O.apply_gradients(ps, acc_o, lr)
+    for k in names:
+        assert_bit_equal(to_host(dp[k]), want_p[k], f"applied {k}")
