@@ -75,7 +75,7 @@ int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** 
   mxopt_table* t = nullptr;
   int rc = mxopt_table_build(ctx, rows.data(), rows.size(), &t);
   if (rc) return rc;
-  constexpr size_t kMaxCached = 8;
+  constexpr size_t kMaxCached = 16;  // two engines and the gradient utilities fit side by side
   if (cache.size() >= kMaxCached) {
     mxopt_table_destroy(cache.front().table);
     cache.erase(cache.begin());
