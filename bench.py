@@ -97,8 +97,16 @@ class Workload:
         torch.cuda.synchronize()
 
     # -- helpers
-    def _randn(self, n, dtype, std):
-        return self.torch.empty(n, dtype=dtype, device="cuda").normal_(0.0, std)
+    SEED = 0x5EED0001
+    CONFIG_ID = {"cfg1": 1, "cfg1-update-single": 1, "cfg1-update-many": 1, "cfg2": 2, "cfg3-sgd": 3, "cfg3-rmsprop": 3,
+                 "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8}
+
+    def _fill(self, views, stream_id, dist, a, b=0.0):
+        """Counter-based synthetic data (mxopt_fill_synthetic): every element is a function of
+        (seed, configuration, stream, tensor, index), so a host program can regenerate any slice."""
+        cfg = self.CONFIG_ID[self.args.workload]
+        for i, v in enumerate(views):
+            self.ctx.fill_synthetic(v, self.mx.synthetic_key(self.SEED, cfg, 0, stream_id, i), dist, a, b)
 
     def _zeros(self, n):
         return self.torch.zeros(n, dtype=self.torch.float32, device="cuda")
@@ -117,13 +125,12 @@ class Workload:
         slab = t.empty(max(total, 1), dtype=dtype, device="cuda")
         return slab, [slab[o:o + n] for o, n in zip(offs, self.sizes)]
 
-    def _randn_list(self, dtype, std):
-        slab, views = self._carve(dtype)
-        if slab is not None:
-            slab.normal_(0.0, std)
-        else:
-            for v in views:
-                v.normal_(0.0, std)
+    def _randn_list(self, dtype, std, outliers=False):
+        """A list of tensors with bell-shaped values of standard deviation `std` (optionally 1 % x100)."""
+        _, views = self._carve(dtype)
+        self._next_stream = getattr(self, "_next_stream", 0) + 1
+        mx = self.mx
+        self._fill(views, self._next_stream, mx.SYNTH_NORMAL_OUTLIERS if outliers else mx.SYNTH_NORMAL, std, 100.0)
         return views
 
     def _zeros_list(self):
@@ -246,13 +253,11 @@ class Workload:
         t, mx = self.torch, self.mx
         bf = t.bfloat16
         if uniform_p:
-            self.p = [t.empty(n, dtype=bf, device="cuda").uniform_(0.9, 1.1) for n in self.sizes]
+            self.p = self._carve(bf)[1]
+            self._fill(self.p, 100, mx.SYNTH_UNIFORM, 0.9, 1.1)
         else:
             self.p = self._randn_list(bf, 0.02)
-        self.g = self._randn_list(bf, gstd)
-        if self.args.workload == "cfg2":   # 1 % of the elements are x100 outliers
-            for g in self.g:
-                g.mul_(t.where(t.rand(g.shape, device="cuda") < 0.01, 100.0, 1.0).to(bf))
+        self.g = self._randn_list(bf, gstd, outliers=self.args.workload == "cfg2")   # cfg2: 1 % of the elements x100
         self.m = self._zeros_list()
         self.v = self._zeros_list()
         self.t_g = self.ctx.table([mx.TensorSpec(g=g) for g in self.g])
@@ -455,7 +460,6 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X: mxopt has no CPU path")
     torch.cuda.set_device(0)
-    torch.manual_seed(0x5EED0001)
 
     wl = Workload(args, torch, mxopt)
     for _ in range(args.warmup):
@@ -502,7 +506,7 @@ def main():
         "value": round(steps_per_s, 4), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(step_ms[len(step_ms) // 2], 4),
         "ms_per_step_min": round(step_ms[0], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": wl.dtype, "data": "synthetic",
+        "dtype": wl.dtype, "data": "synthetic (counter-based generator of the library, seed 0x5EED0001; reproducible on the host)",
         "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
                    "bytes_per_elem_per_step": wl.step_bytes_per_elem,
                    "storage": getattr(wl, "storage", "float32 everywhere"), "note": wl.note, "scale": args.scale,

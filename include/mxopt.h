@@ -271,6 +271,23 @@ int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt
  * non-finite by mxopt_global_norm leaves the buffer untouched (grpo/engine.rs:561-562). */
 int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep);
 
+/* ---- synthetic data for benchmarks and parity tests ----------------------------------
+ * out[i] = f(hash(seed, first_index + i)), hash = splitmix64 finaliser of seed + (index+1)*golden:
+ *   MXOPT_SYNTH_NORMAL          (sum of four 16-bit fields of the hash - 131070) * f32(a / sqrt((65536^2-1)/3)):
+ *                               mean 0, standard deviation a, bell shaped, |x| <= 3.46 a
+ *   MXOPT_SYNTH_NORMAL_OUTLIERS the same, and on average every 100th element (second hash % 100 == 0) times f32(b)
+ *   MXOPT_SYNTH_UNIFORM         f32(top 24 bits) * f32((b - a) / 2^24) + f32(a): uniform on [a, b)
+ * then rounded once to out's dtype.  Only integer arithmetic, exact conversions and at most two rounded
+ * float32 operations: a host program regenerates any slice bit for bit (as the CPU checker in this
+ * repository does), so inputs never have to be copied or read back to compare results at full size.
+ * No counterpart in the reference (its tests build inputs on the host). */
+enum { MXOPT_SYNTH_NORMAL = 0, MXOPT_SYNTH_NORMAL_OUTLIERS = 1, MXOPT_SYNTH_UNIFORM = 2 };
+int mxopt_fill_synthetic(mxopt_ctx* ctx, void* out, uint64_t n, int dtype, uint64_t seed, uint64_t first_index,
+                         int distribution, double a, double b);
+/* The stream key used by this repository's benchmark and tests:
+ * splitmix64(seed ^ config ^ step << 32 ^ micro_batch << 48 ^ tensor_index).  Host only. */
+uint64_t mxopt_synthetic_key(uint64_t seed, uint64_t config, uint64_t step, uint64_t micro_batch, uint64_t tensor_index);
+
 /* ---- small host<->device helpers (each synchronises the context's stream) --------- */
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out);
 

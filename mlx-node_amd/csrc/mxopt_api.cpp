@@ -605,6 +605,40 @@ int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first
   });
 }
 
+uint64_t mxopt_synthetic_key(uint64_t seed, uint64_t config, uint64_t step, uint64_t micro_batch, uint64_t tensor_index) {
+  uint64_t z = (seed ^ config ^ (step << 32) ^ (micro_batch << 48) ^ tensor_index) + 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+int mxopt_fill_synthetic(mxopt_ctx* ctx, void* out, uint64_t n, int dtype, uint64_t seed, uint64_t first_index,
+                         int distribution, double a, double b) {
+  if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_fill_synthetic: null context");
+  if (!float_dtype(dtype)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_fill_synthetic: unsupported dtype code");
+  if (n == 0) return MXOPT_OK;
+  if (!out) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_fill_synthetic: out is NULL");
+  float fa, fb;
+  switch (distribution) {
+    case MXOPT_SYNTH_NORMAL:
+    case MXOPT_SYNTH_NORMAL_OUTLIERS:
+      fa = (float)(a / std::sqrt((65536.0 * 65536.0 - 1.0) / 3.0));
+      fb = (float)b;
+      break;
+    case MXOPT_SYNTH_UNIFORM:
+      fa = (float)((b - a) / 16777216.0);
+      fb = (float)a;
+      break;
+    default:
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_fill_synthetic: unknown distribution");
+  }
+  DeviceGuard guard(ctx->device);
+  const uint64_t blocks = (n + 4 * 256 - 1) / (4 * 256);  // about four elements per lane
+  const uint32_t grid = (uint32_t)std::min<uint64_t>(blocks, (uint64_t)ctx->num_cus * 64u);
+  launch_synth(dtype, out, n, seed, first_index, distribution, fa, fb, grid ? grid : 1u, ctx->stream);
+  return check_launch(ctx, "mxopt_fill_synthetic");
+}
+
 int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep, double max_norm,
                       int clip_mode, mxopt_norm_result* d_result) {
   if (which != 0 && which != 1) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm: which must be 0 or 1");

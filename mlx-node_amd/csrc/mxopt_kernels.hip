@@ -699,6 +699,49 @@ bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep
   return false;
 }
 
+// ------------------------------------------------------------------------------------
+// Synthetic data.  Element i = f(hash(seed, first_index + i)): integer hashing and exact integer
+// -> float conversions followed by one or two rounded float32 operations, so that a host
+// restatement produces the same bits for any slice of any buffer without materialising it.
+// ------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint64_t synth_hash(uint64_t seed, uint64_t idx) {
+  uint64_t z = seed + (idx + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <int OD>
+__global__ __launch_bounds__(kThreads) void synth_kernel(void* __restrict__ out, uint64_t n, uint64_t seed,
+                                                         uint64_t first_index, int dist, float a, float b) {
+  for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kThreads) {
+    const uint64_t z = synth_hash(seed, first_index + i);
+    float x;
+    if (dist == MXOPT_SYNTH_UNIFORM) {
+      x = (float)(uint32_t)(z >> 40) * a;   // a = (hi - lo) / 2^24, b = lo
+      x = x + b;
+    } else {
+      // sum of four 16-bit uniforms, centred: a bell shape on [-131070, 131070] with an exactly known variance
+      const int32_t sum = (int32_t)((z & 0xffffu) + ((z >> 16) & 0xffffu) + ((z >> 32) & 0xffffu) + (z >> 48)) - 131070;
+      x = (float)sum * a;                    // a = sigma / sqrt((65536^2 - 1) / 3)
+      if (dist == MXOPT_SYNTH_NORMAL_OUTLIERS && synth_hash(seed ^ 0xA5A5A5A5A5A5A5A5ull, first_index + i) % 100ull == 0ull)
+        x = x * b;                           // b = outlier multiplier
+    }
+    Elem<OD>::store(out, i, x);
+  }
+}
+
+bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
+                  uint32_t grid, hipStream_t stream) {
+  switch (od) {
+    case MXOPT_F32: hipLaunchKernelGGL(synth_kernel<MXOPT_F32>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+    case MXOPT_BF16: hipLaunchKernelGGL(synth_kernel<MXOPT_BF16>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+    case MXOPT_F16: hipLaunchKernelGGL(synth_kernel<MXOPT_F16>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+  }
+  return false;
+}
+
 void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,
                         int has_max, int clip_mode, mxopt_norm_result* d_out) {
   hipLaunchKernelGGL(norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, partial_sum, npartials, max_norm,

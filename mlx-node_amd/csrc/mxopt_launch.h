@@ -40,6 +40,8 @@ bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep, int 
 // 3: square g_out + g without storing it.
 // partial_sum (one entry per workgroup) may be NULL in mode 2.
 bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum);
+bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
+                  uint32_t grid, hipStream_t stream);
 void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,
                         int has_max, int clip_mode, mxopt_norm_result* d_out);
 

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(os.path.dirname(HERE), "libmxopt.so")
 F32, I32, F16, BF16, U32 = 0, 1, 2, 3, 4
 OK, ERR_INVALID_ARG, ERR_FAILURE, ERR_HIP, ERR_OOM = 0, 1, 2, 3, 4
 TF_FIRST = 0x1
+SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM = 0, 1, 2
 CLIP_ALWAYS_MULTIPLY, CLIP_IF_ABOVE = 0, 1
 CHUNK_ELEMS = 4096
 
@@ -101,6 +102,9 @@ SIGNATURES = {
                                    C.c_void_p]),
     "mxopt_accumulate_norm_only": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
                                              C.c_void_p]),
+    "mxopt_fill_synthetic": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_uint64, C.c_uint64, C.c_int,
+                                       C.c_double, C.c_double]),
+    "mxopt_synthetic_key": (C.c_uint64, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64]),
     "mxopt_read_norm_result": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(NormResult)]),
     "mxopt_version": (C.c_char_p, []),
 }

@@ -199,6 +199,19 @@ def _sgd_plain_with_pending(self, table: "Table", learning_rate: float, weight_d
             self.handle)
 
 
+def _fill_synthetic(self, t: torch.Tensor, seed: int, distribution: int = L.SYNTH_NORMAL, a: float = 1.0,
+                    b: float = 0.0, first_index: int = 0) -> None:
+    """Deterministic synthetic data into `t` (see mxopt_fill_synthetic): reproducible on the host."""
+    if not t.is_contiguous():
+        raise L.InvalidArg(L.ERR_INVALID_ARG, "mxopt needs dense (contiguous) buffers")
+    L.check(self.lib.mxopt_fill_synthetic(self.handle, _dev_ptr(t), t.numel(), dtype_code(t), seed & (2 ** 64 - 1),
+                                          first_index, distribution, a, b), self.handle)
+
+
+def synthetic_key(seed: int, config: int = 0, step: int = 0, micro_batch: int = 0, tensor_index: int = 0) -> int:
+    return L.load().mxopt_synthetic_key(seed & (2 ** 64 - 1), config, step, micro_batch, tensor_index)
+
+
 def _accumulate_transformed(self, table: "Table", first: bool, prep: Optional[L.GradPrep] = None) -> None:
     L.check(self.lib.mxopt_accumulate_transformed(self.handle, table.handle, int(first),
                                                   C.byref(prep) if prep else None), self.handle)
@@ -212,6 +225,7 @@ def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Opt
 
 Context.accumulate_norm_only = _accumulate_norm_only
 Context.accumulate_transformed = _accumulate_transformed
+Context.fill_synthetic = _fill_synthetic
 Context.sgd_plain_with_pending = _sgd_plain_with_pending
 
 

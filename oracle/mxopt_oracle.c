@@ -67,6 +67,35 @@ void oracle_bf16_to_f32(const uint16_t* x, float* out, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = bf16_to_f32(x[i]);
 }
 
+/* Host twin of the library's synthetic-data generator (defined at mxopt_fill_synthetic in include/mxopt.h). */
+static inline uint64_t synth_hash(uint64_t seed, uint64_t idx) {
+  uint64_t z = seed + (idx + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+void oracle_fill_synthetic(void* out, int dtype, size_t n, uint64_t seed, uint64_t first_index, int dist, double a,
+                           double b) {
+  const float fa = dist == 2 ? (float)((b - a) / 16777216.0) : (float)(a / sqrt((65536.0 * 65536.0 - 1.0) / 3.0));
+  const float fb = dist == 2 ? (float)a : (float)b;
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t z = synth_hash(seed, first_index + i);
+    float x;
+    if (dist == 2) {
+      x = (float)(uint32_t)(z >> 40) * fa;
+      x = x + fb;
+    } else {
+      const int32_t sum = (int32_t)((z & 0xffffu) + ((z >> 16) & 0xffffu) + ((z >> 32) & 0xffffu) + (z >> 48)) - 131070;
+      x = (float)sum * fa;
+      if (dist == 1 && synth_hash(seed ^ 0xA5A5A5A5A5A5A5A5ull, first_index + i) % 100ull == 0ull) x = x * fb;
+    }
+    if (dtype == DT_BF16) ((uint16_t*)out)[i] = f32_to_bf16(x);
+    else ((float*)out)[i] = x;
+  }
+}
+
 /* Sum of squares in float64 (optimizers/mod.rs:43-55). */
 double oracle_sumsq(const void* g, int dt, size_t n) {
   double s = 0.0;

@@ -619,6 +619,58 @@ class SFTEngineOptimizerSide(_EngineBase):
 
 
 # --------------------------------------------------------------------------
+# Synthetic inputs: the host twin of the library's counter-based generator (its definition is in
+# include/mxopt.h at mxopt_fill_synthetic).  Not part of the reference; it lets a checker regenerate
+# any slice of any benchmark input without copying it.
+# --------------------------------------------------------------------------
+
+_M64 = (1 << 64) - 1
+SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM = 0, 1, 2
+
+
+def _splitmix_finish(z: np.ndarray) -> np.ndarray:
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def synthetic_hash(seed: int, index: np.ndarray) -> np.ndarray:
+    idx = np.asarray(index, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        return _splitmix_finish(np.uint64(seed & _M64) + (idx + np.uint64(1)) * np.uint64(0x9E3779B97F4A7C15))
+
+
+def synthetic_key(seed: int, config: int = 0, step: int = 0, micro_batch: int = 0, tensor_index: int = 0) -> int:
+    z = ((seed ^ config ^ (step << 32) ^ (micro_batch << 48) ^ tensor_index) + 0x9E3779B97F4A7C15) & _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def synthetic(n: int, dtype: str, seed: int, distribution: int = SYNTH_NORMAL, a: float = 1.0, b: float = 0.0,
+              first_index: int = 0) -> np.ndarray:
+    """Elements first_index .. first_index+n-1 of the stream `seed`; dtype "f32", "bf16" (uint16 bits) or "f16"."""
+    idx = np.arange(first_index, first_index + n, dtype=np.uint64)
+    z = synthetic_hash(seed, idx)
+    if distribution == SYNTH_UNIFORM:
+        x = (z >> np.uint64(40)).astype(F32) * _f32((b - a) / 16777216.0)
+        x = x + _f32(a)
+    else:
+        m = np.uint64(0xFFFF)
+        total = ((z & m) + ((z >> np.uint64(16)) & m) + ((z >> np.uint64(32)) & m) + (z >> np.uint64(48))).astype(np.int64)
+        x = (total - 131070).astype(F32) * _f32(a / math.sqrt((65536.0 * 65536.0 - 1.0) / 3.0))
+        if distribution == SYNTH_NORMAL_OUTLIERS:
+            hit = synthetic_hash(seed ^ 0xA5A5A5A5A5A5A5A5, idx) % np.uint64(100) == np.uint64(0)
+            x = np.where(hit, x * _f32(b), x).astype(F32)
+    if dtype == "bf16":
+        return f32_to_bf16(x)
+    if dtype == "f16":
+        with np.errstate(over="ignore"):
+            return x.astype(np.float16)
+    return x.astype(F32, copy=False)
+
+
+# --------------------------------------------------------------------------
 # Learning-rate schedules  (optimizers/mod.rs:239-292) -- host float64 closed forms
 # --------------------------------------------------------------------------
 

@@ -72,6 +72,9 @@ class OracleC:
         lib.oracle_accumulate_f32.restype = None
         lib.oracle_scale_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_float]
         lib.oracle_scale_f32.restype = None
+        lib.oracle_fill_synthetic.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_uint64, C.c_uint64, C.c_int,
+                                              C.c_double, C.c_double]
+        lib.oracle_fill_synthetic.restype = None
         lib.oracle_f32_to_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         lib.oracle_bf16_to_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
 
@@ -84,6 +87,13 @@ class OracleC:
     def f32_to_bf16(self, x: np.ndarray) -> np.ndarray:
         out = np.empty(x.shape, np.uint16)
         self.lib.oracle_f32_to_bf16(_ptr(x), _ptr(out), x.size)
+        return out
+
+    def fill_synthetic(self, n: int, dtype: str, seed: int, distribution: int = 0, a: float = 1.0, b: float = 0.0,
+                       first_index: int = 0) -> np.ndarray:
+        out = np.empty(n, np.uint16 if dtype == "bf16" else np.float32)
+        self.lib.oracle_fill_synthetic(_ptr(out), DT_BF16 if dtype == "bf16" else DT_F32, n, seed & (2 ** 64 - 1),
+                                       first_index, distribution, a, b)
         return out
 
     def adam(self, p, g, m, v, args: AdamArgs, fused: bool = True) -> np.ndarray:

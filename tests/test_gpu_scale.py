@@ -4,11 +4,12 @@
   bit for bit against the C twin of the oracle -- once with the reference's default (no bias
   correction) through the kernel-level table, once bias-corrected through the optimizer object, where
   tensor i of step s must see t = s*N + i + 1 (the reference counts update_single calls).
-* Qwen3-1.7B list, bf16 parameters and gradients with 1 % x100 outliers, clip 1.0 (config 2) and the
-  Qwen3-4B list, float32 SGD with momentum / RMSprop (config 3): every tensor of at most 1 Mi elements in
-  full plus seeded windows (head, tail, interior) of every larger one, two steps, bit for bit; the
-  global norm of every step against a float64 reduction done by torch on the device (a library routine
-  that is not the reference) at rel 1e-5.
+* Qwen3-1.7B list, bf16 parameters and gradients with 1 % x100 outliers, clip 1.0 (config 2): EVERY
+  element, two steps; the inputs are generated on the device by the library's counter-based generator
+  and regenerated on the host by the oracle's twin of it, the norm is checked against the exact
+  float64 sum.
+* Qwen3-4B list, float32 SGD with momentum / RMSprop (config 3): every tensor of at most 1 Mi elements in
+  full plus seeded windows (head, tail, interior) of every larger one, bit for bit.
 * 10,000 small bf16 tensors (config 4): EVERY element, three steps, packed back to back so that most
   tensors start at an address that is only 2-byte aligned, and separately allocated.
 * Qwen3-8B list, bf16 parameters / float32 moments, 4 micro-batches into a float32 buffer, clip 1.0,
@@ -163,45 +164,50 @@ def test_config1_bias_corrected_per_call_step_count(oracle_c):
 # config 2
 # ---------------------------------------------------------------------------------------
 
-def test_config2_full_size_outliers_clip_windows(oracle_c):
+def test_config2_full_size_every_element(oracle_c):
+    """Inputs come from the library's counter-based generator on the device and are regenerated on the
+    host by the oracle's twin of it: nothing is copied to the device, every one of 1.72 G elements of
+    p, m and v is compared after each of two steps."""
     import torch
     import mxopt as mx
     _, sizes = qwen_sizes("1.7B")
-    n = sum(sizes)
-    assert n == 1_720_574_976 and len(sizes) == 310
-    torch.manual_seed(0x5EED0002)
+    n, nt = sum(sizes), len(sizes)
+    assert n == 1_720_574_976 and nt == 310
     bf = torch.bfloat16
-    p_slab, offs, dp = carve(torch, sizes, bf)
-    g_slab, _, dg = carve(torch, sizes, bf)
-    m_slab, _, dm = carve(torch, sizes, torch.float32)
-    v_slab, _, dv = carve(torch, sizes, torch.float32)
-    p_slab.normal_(0, 0.02)
-    m_slab.zero_()
-    v_slab.zero_()
-    idx = window_index(torch, sizes, offs, seed=2)
-    win = lambda slab: to_host(slab[idx])
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    dp = [torch.empty(s, dtype=bf, device="cuda") for s in sizes]
+    dg = [torch.empty(s, dtype=bf, device="cuda") for s in sizes]
+    dm = [torch.zeros(s, device="cuda") for s in sizes]
+    dv = [torch.zeros(s, device="cuda") for s in sizes]
     ctx = mx.Context()
+    SEED, CFG = 0x5EED0001, 2
+    p_ref = np.empty(n, np.uint16)
+    for i in range(nt):
+        key = mx.synthetic_key(SEED, CFG, 0, 0, i)
+        ctx.fill_synthetic(dp[i], key, mx.SYNTH_NORMAL, 0.02)
+        p_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, O.SYNTH_NORMAL, 0.02)
     t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
     t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
     hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
     res = ctx.norm_result()
-    p_ref, m_ref, v_ref = win(p_slab), win(m_slab), win(v_slab)
+    m_ref, v_ref = np.zeros(n, F), np.zeros(n, F)
+    g_ref = np.empty(n, np.uint16)
     for step in range(2):
-        g_slab.normal_(0, 1e-3)
-        for lo in range(0, g_slab.numel(), 1 << 28):                # 1 % of the elements x100, in pieces
-            piece = g_slab[lo:lo + (1 << 28)]
-            piece.mul_(torch.where(torch.rand(piece.shape, device="cuda") < 0.01, 100.0, 1.0).to(bf))
+        for i in range(nt):                     # fresh gradients each step: 1 % of the elements x100
+            key = mx.synthetic_key(SEED, CFG, step + 1, 1, i)
+            ctx.fill_synthetic(dg[i], key, mx.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0)
+            g_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0)
         ctx.global_norm(t_g, res, max_norm=1.0)
         ctx.adam(t_upd, hp, mx.make_prep(scale=res))
         r = ctx.read_norm_result(res)
-        scale = check_norm(r, device_sumsq_f64(torch, dg))
-        expected = 1e-3 * math.sqrt(n * (0.99 + 0.01 * 1e4))         # ~417: the clip is active
+        scale = check_norm(r, oracle_c.sumsq(g_ref))                       # exact float64 sum on the host
+        expected = 1e-3 * math.sqrt(n * (0.99 + 0.01 * 1e4))               # ~417: the clip is active
         assert abs(r.norm - expected) < 0.02 * expected and scale < 0.01
         args = B.adam_args(5e-6, 0.9, 0.999, 1e-8, 0.01, scale=scale)
-        p_ref = oracle_c.f32_to_bf16(oracle_c.adam(p_ref, win(g_slab), m_ref, v_ref, args, fused=True))
-        same_bits(win(p_slab), p_ref, f"p step {step}")
-        same_bits(win(m_slab), m_ref, f"m step {step}")
-        same_bits(win(v_slab), v_ref, f"v step {step}")
+        p_ref = oracle_c.f32_to_bf16(oracle_c.adam(p_ref, g_ref, m_ref, v_ref, args, fused=True))
+        same_bits(to_host(torch.cat(dp)), p_ref, f"p step {step}")
+        same_bits(torch.cat(dm).cpu().numpy(), m_ref, f"m step {step}")
+        same_bits(torch.cat(dv).cpu().numpy(), v_ref, f"v step {step}")
     t_g.close()
     t_upd.close()
     ctx.close()

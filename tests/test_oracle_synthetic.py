@@ -1,0 +1,49 @@
+"""The counter-based synthetic-data generator: the oracle's NumPy statement, its C twin and the
+library's host-only key function agree; the distributions are what the benchmark configurations ask for."""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+import mxopt_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
+
+
+def test_numpy_and_c_twin_agree(oracle_c):
+    for dist, a, b in ((O.SYNTH_NORMAL, 1e-3, 0.0), (O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0), (O.SYNTH_UNIFORM, 0.9, 1.1)):
+        for dt in ("f32", "bf16"):
+            for first in (0, 7, 2 ** 40 + 3):
+                x = O.synthetic(50021, dt, 0xDEADBEEF12345678, dist, a, b, first_index=first)
+                y = oracle_c.fill_synthetic(50021, dt, 0xDEADBEEF12345678, dist, a, b, first_index=first)
+                assert np.array_equal(x, y), (dist, dt, first)
+
+
+def test_a_slice_is_the_same_as_the_middle_of_the_whole():
+    whole = O.synthetic(10000, "bf16", 42, O.SYNTH_NORMAL, 0.02)
+    assert np.array_equal(O.synthetic(100, "bf16", 42, O.SYNTH_NORMAL, 0.02, first_index=1234), whole[1234:1334])
+
+
+def test_distributions():
+    x = O.synthetic(4_000_000, "f32", 1, O.SYNTH_NORMAL, 1e-3).astype(np.float64)
+    assert abs(x.mean()) < 3e-6 and abs(x.std() - 1e-3) < 2e-6 and np.abs(x).max() <= 3.47e-3
+    assert abs(np.mean(np.abs(x) < 1e-3) - 0.669) < 0.005                    # bell shaped: 66.9 % within one sigma (a normal has 68.3 %)
+    y = O.synthetic(4_000_000, "f32", 2, O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0).astype(np.float64)
+    assert abs(np.mean(np.abs(y) > 3.5e-3) - 0.0097) < 0.001                 # 1 % x100, a few of them still small
+    assert abs(np.sqrt(np.mean(y * y)) - 1e-3 * np.sqrt(0.99 + 0.01 * 1e4)) < 2e-4
+    u = O.synthetic(1_000_000, "f32", 3, O.SYNTH_UNIFORM, 0.9, 1.1)
+    assert u.min() >= 0.9 and u.max() < 1.1 and abs(u.mean() - 1.0) < 2e-4
+    assert len(np.unique(O.synthetic(100000, "f32", 4, O.SYNTH_UNIFORM, 0.0, 1.0))) > 99000
+    # different streams are unrelated
+    a, b = O.synthetic(100000, "f32", 10, 0, 1.0), O.synthetic(100000, "f32", 11, 0, 1.0)
+    assert abs(np.corrcoef(a, b)[0, 1]) < 0.02
+
+
+def test_key_function_matches_the_library():
+    from mxopt import _lib
+    lib = _lib.load()
+    for args in ((0x5EED0001, 5, 0, 0, 0), (0x5EED0001, 5, 9, 3, 398), (2 ** 64 - 1, 0, 2 ** 31, 65535, 2 ** 32)):
+        assert lib.mxopt_synthetic_key(*[C.c_uint64(v & (2 ** 64 - 1)) for v in args]) == O.synthetic_key(*args), args
+    assert O.synthetic_key(1, 2, 3, 4, 5) != O.synthetic_key(1, 2, 3, 4, 6)
