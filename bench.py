@@ -41,7 +41,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
                     choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
-                             "cfg4", "cfg4-flat", "cfg5", "copy", "grpo-engine", "sft-engine"])
+                             "cfg4", "cfg4-flat", "cfg5", "cfg5-deferred", "copy", "grpo-engine", "sft-engine"])
     ap.add_argument("--cpu-sample", type=int, default=512 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -62,7 +62,7 @@ def parse_args():
 
 def tensor_sizes(args):
     from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B", "grpo-engine": "8B", "sft-engine": "8B"}.get(args.workload)
+    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B", "cfg5-deferred": "8B", "grpo-engine": "8B", "sft-engine": "8B"}.get(args.workload)
     if model:
         sizes = []
         for _, shape in param_list(QWEN3[model]):
@@ -99,7 +99,7 @@ class Workload:
     # -- helpers
     SEED = 0x5EED0001
     CONFIG_ID = {"cfg1": 1, "cfg1-update-single": 1, "cfg1-update-many": 1, "cfg2": 2, "cfg3-sgd": 3, "cfg3-rmsprop": 3,
-                 "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8}
+                 "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "cfg5-deferred": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8}
 
     def _fill(self, views, stream_id, dist, a, b=0.0):
         """Counter-based synthetic data (mxopt_fill_synthetic): every element is a function of
@@ -207,6 +207,33 @@ class Workload:
             self._timed("adamw", lambda: c.adam_with_pending(self.t_upd_pending, self.hp, self.prep))
         else:
             self._timed("adamw", lambda: c.adam(self.t_upd, self.hp, self.prep))
+
+    # -- cfg5 without its accumulation buffer: the four micro-batches stay resident and are summed in
+    #    registers, in arrival order, by the norm pass (8 B/elem) and by the update (18 + 10 B/elem)
+    def _setup_cfg5_deferred(self):
+        t, mx = self.torch, self.mx
+        bf = t.bfloat16
+        self.n_micro = 4
+        self.p = self._randn_list(bf, 0.02)
+        self.m = self._zeros_list()
+        self.v = self._zeros_list()
+        self.g = [self._randn_list(bf, 1e-3) for _ in range(self.n_micro)]
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
+                                     for p, g, m, v in zip(self.p, self.g[0], self.m, self.v)])
+        self.t_upd.set_pending(self.g[1:])
+        self.hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
+        self.prep = mx.make_prep(scale=self.res)
+        self.dtype = "f32"
+        self.storage = "bf16 parameters and gradients, float32 moments, no accumulation buffer"
+        self.bytes_per_elem = {"norm_of_sum": 2 * self.n_micro, "adamw": 2 * self.n_micro + 10 + 10}
+        self.step_bytes_per_elem = sum(self.bytes_per_elem.values())
+        self.dominant = "adamw"
+        self.note = "4 resident micro-batches summed in registers (float32, arrival order) by the norm pass and by AdamW"
+
+    def _step_cfg5_deferred(self):
+        c = self.ctx
+        self._timed("norm_of_sum", lambda: c.norm_with_pending_list(self.t_upd, self.res, max_norm=1.0))
+        self._timed("adamw", lambda: c.adam_with_pending_list(self.t_upd, self.hp, self.prep))
 
     # -- cfg1: fp32 AdamW
     def _setup_cfg1(self):
@@ -399,7 +426,7 @@ def cpu_baseline(args, n_total):
         return best
 
     fused_s = None
-    if w in ("cfg5", "cfg2", "cfg4", "cfg4-flat"):
+    if w in ("cfg5", "cfg5-deferred", "cfg2", "cfg4", "cfg4-flat"):
         p, g = oc.f32_to_bf16(p32), oc.f32_to_bf16(g32)
         del p32, g32
         acc = np.empty(S, f32)
@@ -407,7 +434,7 @@ def cpu_baseline(args, n_total):
 
         def step(fused):
             src = g
-            if w == "cfg5":
+            if w in ("cfg5", "cfg5-deferred"):
                 for k in range(4):
                     oc.accumulate_f32(acc, g, k == 0)
                 src = acc
@@ -417,7 +444,7 @@ def cpu_baseline(args, n_total):
             out = oc.adam(p, src, m, v, a, fused=fused)
             oc.f32_to_bf16(out)     # parameters are kept in bf16
         what = ("4x accumulate + sumsq + scale + AdamW as 13 separate float32 passes (adamw.rs:84-116) + bf16 cast"
-                if w == "cfg5" else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
+                if w in ("cfg5", "cfg5-deferred") else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
         t_unfused = timeit(lambda: step(False))
         fused_s = timeit(lambda: step(True))
     elif w.startswith("cfg1"):

@@ -229,6 +229,42 @@ int mxopt_sgd_plain(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, 
 int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate, double weight_decay,
                                  const mxopt_grad_prep* prep, int prep_covers_sum);
 
+/* ---- deferred accumulation ---------------------------------------------------------
+ * With HBM to spare the accumulation buffer need not exist.  The micro-batch gradients of one
+ * optimizer step stay where the backward passes left them; the norm pass and the update kernel add
+ * them in registers, left to right in float32:  ((g + x0) + x1) + x2.  These are the additions
+ * Qwen3Model::accumulate_gradients (models/qwen3/model.rs:2217-2243) / the engines
+ * (grpo/engine.rs:2632-2666, sft/engine.rs:282-290) would have made into a float32 buffer, in the
+ * same order, so parameters and moments come out bit-identical while the buffer is never written
+ * or read back: four bf16 micro-batches + AdamW move 36 B/elem instead of 58.
+ *
+ * tensor.g is the first addend: the first micro-batch, or a float32 buffer that already holds
+ * earlier ones (more micro-batches than MXOPT_MAX_PENDING + 1).  The pending streams x0.. all have
+ * one dtype; tensor.g has that dtype or float32.  The caller keeps every stream alive and unchanged
+ * until the update has run.  No counterpart in the reference (it materialises every sum). */
+#define MXOPT_MAX_PENDING 3
+
+/* Attach k (0..MXOPT_MAX_PENDING; 0 detaches) pending streams to every row of the table:
+ * streams[j * num_tensors + i] is pending stream j of row i, `dtype` their element type.  A
+ * stream of a row with n > 0 must not be NULL and must share the 16-byte phase of the row's other
+ * buffers (see mxopt_tensor_layout).  Stream-ordered like mxopt_table_retarget; call it again when
+ * the buffers of the next step differ. */
+int mxopt_table_set_pending(mxopt_table* t, int k, const void* const* streams, int dtype);
+
+/* Norm (and clip factor) of prep_pre(g + x0 + ...) over the whole table; nothing is stored.
+ * Arguments as mxopt_global_norm. */
+int mxopt_norm_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep, double max_norm,
+                                 int clip_mode, mxopt_norm_result* d_result);
+
+/* mxopt_adam on the gradient prep(g + x0 + ...).  p_out must have p's dtype (in place or not). */
+int mxopt_adam_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp,
+                                 const mxopt_grad_prep* prep);
+
+/* mxopt_sgd_plain on the gradient prep(g + x0 + ...), which is float32 (the sum promotes);
+ * the SFT engine's boundary (sft/engine.rs:293-371) without its accumulation buffer. */
+int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                      double weight_decay, const mxopt_grad_prep* prep);
+
 /* ---- global norm ------------------------------------------------------------------ */
 
 /* Sum of squares of the gradients (after prep's pre_mul / clamp_pre) over the whole

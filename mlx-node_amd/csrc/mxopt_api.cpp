@@ -445,16 +445,74 @@ int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n) 
   return upload_descriptors(t);
 }
 
+int mxopt_table_set_pending(mxopt_table* t, int k, const void* const* streams, int dtype) {
+  if (!t) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_set_pending: null table");
+  mxopt_ctx* ctx = t->ctx;
+  if (k < 0 || k > MXOPT_MAX_PENDING)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                "mxopt_table_set_pending: k must be in [0, " + std::to_string(MXOPT_MAX_PENDING) + "]");
+  if (k == 0) {
+    t->pending_k = 0;
+    return MXOPT_OK;
+  }
+  if (!streams) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_set_pending: streams is NULL");
+  if (!float_dtype(dtype)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_set_pending: unsupported dtype code");
+  const size_t n = t->host.size();
+  const size_t esize = (size_t)dtype_size(dtype);
+  for (int j = 0; j < k; ++j) {
+    for (size_t i = 0; i < n; ++i) {
+      if (t->host[i].n == 0) continue;
+      const void* ptr = streams[(size_t)j * n + i];
+      const std::string where = "mxopt_table_set_pending: stream " + std::to_string(j) + " of tensor " + std::to_string(i);
+      if (!ptr) return fail(ctx, MXOPT_ERR_INVALID_ARG, where + " is NULL");
+      const DevTensor& d = t->dev[i];
+      if (d.flags & kTfUnaligned) {
+        if (reinterpret_cast<uintptr_t>(ptr) % esize) return fail(ctx, MXOPT_ERR_INVALID_ARG, where + " is not element-aligned");
+      } else if ((reinterpret_cast<uintptr_t>(ptr) + (uintptr_t)d.head * esize) & 15u) {
+        return fail(ctx, MXOPT_ERR_INVALID_ARG, where + " does not share the 16-byte phase of the tensor's other buffers");
+      }
+    }
+  }
+  if (n == 0) {
+    t->pending_k = k;
+    t->pending_dtype = dtype;
+    return MXOPT_OK;
+  }
+  DeviceGuard guard(ctx->device);
+  const size_t bytes = (size_t)MXOPT_MAX_PENDING * n * sizeof(void*);
+  if (!t->d_pending) HIP_TRY(ctx, hipMalloc((void**)&t->d_pending, bytes));
+  // Same two-buffer staging as the descriptors: the call does not wait for the copy.
+  const int turn = t->turn_pending ^= 1;
+  if (!t->pinned_pending[turn]) {
+    HIP_TRY(ctx, hipHostMalloc((void**)&t->pinned_pending[turn], bytes, hipHostMallocDefault));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&t->copied_pending[turn], hipEventDisableTiming));
+  } else {
+    HIP_TRY(ctx, hipEventSynchronize(t->copied_pending[turn]));
+  }
+  std::memcpy(t->pinned_pending[turn], streams, (size_t)k * n * sizeof(void*));
+  HIP_TRY(ctx, hipMemcpyAsync(t->d_pending, t->pinned_pending[turn], (size_t)k * n * sizeof(void*),
+                              hipMemcpyHostToDevice, ctx->stream));
+  HIP_TRY(ctx, hipEventRecord(t->copied_pending[turn], ctx->stream));
+  t->pending_k = k;
+  t->pending_dtype = dtype;
+  return MXOPT_OK;
+}
+
 void mxopt_table_destroy(mxopt_table* t) {
   if (!t) return;
   DeviceGuard guard(t->ctx->device);
   (void)hipStreamSynchronize(t->ctx->stream);
   if (t->d_tensors) (void)hipFree(t->d_tensors);
   if (t->d_chunks) (void)hipFree(t->d_chunks);
+  if (t->d_pending) (void)hipFree(t->d_pending);
   for (int k = 0; k < 2; ++k) {
     if (t->pinned[k]) {
       (void)hipHostFree(t->pinned[k]);
       (void)hipEventDestroy(t->copied[k]);
+    }
+    if (t->pinned_pending[k]) {
+      (void)hipHostFree(t->pinned_pending[k]);
+      (void)hipEventDestroy(t->copied_pending[k]);
     }
   }
   delete t;
@@ -588,6 +646,39 @@ int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double le
   });
 }
 
+static void attach_pending(const mxopt_table* t, Launch& L) {
+  L.pending = t->d_pending;
+  L.ntensors = (uint32_t)t->host.size();
+  L.npending = t->pending_k;
+}
+
+int mxopt_adam_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp,
+                                 const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedM | kNeedV, "mxopt_adam_with_pending_list");
+  if (rc) return rc;
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_adam_with_pending_list: hp is NULL");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, "mxopt_adam_with_pending_list", [&](const Group& g, Launch& L) {
+    attach_pending(t, L);
+    return launch_adam_list(g.pd, g.gd, g.pod, t->pending_k ? t->pending_dtype : g.gd, L, *hp, dp);
+  });
+}
+
+int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                      double weight_decay, const mxopt_grad_prep* prep) {
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG, "mxopt_sgd_plain_with_pending_list");
+  if (rc) return rc;
+  const DevPrep dp = make_prep(prep);
+  const float lr32 = (float)learning_rate;
+  const float wd32 = (float)weight_decay;
+  const int has_wd = weight_decay > 0.0;  // sft/engine.rs:345
+  return run_update(ctx, t, "mxopt_sgd_plain_with_pending_list", [&](const Group& g, Launch& L) {
+    attach_pending(t, L);
+    return launch_sgd_plain_list(g.pd, g.gd, g.pod, t->pending_k ? t->pending_dtype : g.gd, L,
+                                 round_to_dtype(lr32, g.pd), wd32, has_wd, dp);
+  });
+}
+
 int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep) {
   int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_grad_transform");
   if (rc) return rc;
@@ -661,6 +752,34 @@ int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt
   if (rc) return rc;
   if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_accumulate_norm_only: d_result is NULL");
   return run_sumsq(ctx, t, 3, 0, prep, max_norm, clip_mode, d_result, "mxopt_accumulate_norm_only");
+}
+
+int mxopt_norm_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep, double max_norm,
+                                 int clip_mode, mxopt_norm_result* d_result) {
+  const char* op = "mxopt_norm_with_pending_list";
+  int rc = require(ctx, t, kNeedG, op);
+  if (rc) return rc;
+  if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": d_result is NULL");
+  if (clip_mode != MXOPT_CLIP_ALWAYS_MULTIPLY && clip_mode != MXOPT_CLIP_IF_ABOVE)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unknown clip mode");
+  DeviceGuard guard(ctx->device);
+  const DevPrep dp = make_prep(prep);
+  size_t total_grid = 0;
+  for (const Group& g : t->groups) total_grid += persistent_grid(ctx, g.nchunks);
+  rc = ensure_partials(ctx, std::max<size_t>(total_grid, 1));
+  if (rc) return rc;
+  size_t offset = 0;
+  for (const Group& g : t->groups) {
+    Launch L = make_launch(ctx, t, g, true);
+    L.nontemporal = ctx->nontemporal_reduce;
+    attach_pending(t, L);
+    if (!launch_sumsq_list(g.gd, t->pending_k ? t->pending_dtype : g.gd, L, dp, ctx->d_partial_sum + offset))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
+    rc = check_launch(ctx, op);
+    if (rc) return rc;
+    offset += L.grid;
+  }
+  return finish_norm(ctx, (uint32_t)offset, max_norm, clip_mode, d_result);
 }
 
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out) {

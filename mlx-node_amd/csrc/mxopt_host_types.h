@@ -92,4 +92,11 @@ struct mxopt_table {
   mxopt::DevTensor* pinned[2] = {nullptr, nullptr};  // staging for per-step scalar updates
   hipEvent_t copied[2] = {nullptr, nullptr};
   int turn = 0;
+  // Deferred accumulation: pending gradient streams, pending_k x tensors pointers (stream-major).
+  int pending_k = 0;
+  int pending_dtype = 0;
+  const void** d_pending = nullptr;                  // MXOPT_MAX_PENDING x tensors slots
+  const void** pinned_pending[2] = {nullptr, nullptr};
+  hipEvent_t copied_pending[2] = {nullptr, nullptr};
+  int turn_pending = 0;
 };

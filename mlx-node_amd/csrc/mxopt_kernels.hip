@@ -124,6 +124,7 @@ struct ChunkView {
   uint64_t start;  // first element of the chunk inside the tensor
   uint32_t len;    // elements in this chunk (kChunk except for the last one)
   uint32_t head;   // chunk 0 of a shifted tensor: elements [0, head) are this workgroup's too
+  uint32_t tensor; // row of the table (0 for a single tensor passed by value)
   bool fast;       // full chunk of a 16-byte aligned (after the head) tensor: 128-bit path, fully unrolled
 };
 
@@ -134,9 +135,11 @@ __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, con
   if (C != nullptr) {  // table walk
     const DevChunk ch = C[c];
     cv.t = T[ch.tensor];
+    cv.tensor = ch.tensor;
     index = ch.index;
   } else {             // a single tensor described in the kernel arguments: chunk c of `one`
     cv.t = one;
+    cv.tensor = 0;
     index = c;
   }
   cv.start = (uint64_t)cv.t.head + (uint64_t)index * kChunk;
@@ -477,6 +480,210 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
   }
 }
 
+// ------------------------------------------------------------------------------------
+// Deferred accumulation.  The gradient is g + x_0 + ... + x_{kx-1}, added left to right in float32:
+// the additions Qwen3Model::accumulate_gradients (models/qwen3/model.rs:2217-2243) would have made
+// into a float32 buffer, made in registers instead, so that the buffer is never written or re-read.
+// X[j * ntensors + row] is stream j of table row `row` (dtype XD); g is either the first micro-batch
+// or a float32 buffer that already holds earlier ones.
+// ------------------------------------------------------------------------------------
+
+constexpr int kMaxPending = MXOPT_MAX_PENDING;
+
+struct PendingStreams {
+  const void* x[kMaxPending];
+};
+
+__device__ __forceinline__ PendingStreams pending_of(const void* const* __restrict__ X, uint32_t ntensors, uint32_t row,
+                                                     int kx) {
+  PendingStreams ps;
+#pragma unroll
+  for (int j = 0; j < kMaxPending; ++j) ps.x[j] = j < kx ? X[(size_t)j * ntensors + row] : nullptr;
+  return ps;
+}
+
+template <int GD, int XD>
+__device__ __forceinline__ float pending_sum_element(const void* G, const PendingStreams& ps, int kx, uint64_t off) {
+  float s = Elem<GD>::load(G, off);
+#pragma unroll
+  for (int j = 0; j < kMaxPending; ++j)
+    if (j < kx) s = s + Elem<XD>::load(ps.x[j], off);
+  return s;
+}
+
+template <int PD, int GD, int XD, class Math>
+__global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* __restrict__ T,
+                                                               const DevChunk* __restrict__ C, DevTensor one,
+                                                               uint32_t nchunks, uint32_t ntensors,
+                                                               const void* const* __restrict__ X, int kx, Math math,
+                                                               DevPrep prep) {
+  constexpr int E = (PD != MXOPT_F32 || GD != MXOPT_F32 || XD != MXOPT_F32) ? 8 : 4;
+  constexpr int U = kElemsPerLane / E;
+  if (skip_requested(prep)) return;
+  const PrepRegs pr = load_prep(prep);
+  const uint32_t tid = threadIdx.x;
+
+  for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const ChunkView cv = locate(T, C, one, c);
+    const PendingStreams ps = pending_of(X, ntensors, cv.tensor, kx);
+    const uint64_t start = cv.start;
+    const uint32_t len = cv.len, flags = cv.t.flags;
+    const float bc1 = cv.t.bc1, bc2 = cv.t.bc2;
+    const void* P = cv.t.p;
+    void* PO = cv.t.p_out;
+    const void* G = cv.t.g;
+    float* M = cv.t.m;
+    float* V = cv.t.v;
+    const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
+    auto one_element = [&](uint64_t off) {
+      float p = Elem<PD>::load(P, off);
+      const float ge = prep_all(pr, pending_sum_element<GD, XD>(G, ps, kx, off));
+      float m = Math::kM ? M[off] : 0.0f;
+      float v = read_v ? V[off] : 0.0f;
+      math(p, ge, m, v, bc1, bc2, flags);
+      Elem<PD>::store(PO, off, p);
+      if (Math::kM) M[off] = m;
+      if (use_v) V[off] = v;
+    };
+
+    if (cv.fast) {
+      float p[U][E], g[U][E], x[kMaxPending][U][E], m[U][E], v[U][E];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
+        load_group<GD, E, false>(G, off, g[j]);
+#pragma unroll
+        for (int k = 0; k < kMaxPending; ++k)
+          if (k < kx) load_group<XD, E, false>(ps.x[k], off, x[k][j]);
+        load_group<PD, E, false>(P, off, p[j]);
+        if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m[j]);
+        if (read_v) load_group<MXOPT_F32, E, false>(V, off, v[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          float s = g[j][e];
+#pragma unroll
+          for (int k = 0; k < kMaxPending; ++k)
+            if (k < kx) s = s + x[k][j][e];
+          math(p[j][e], prep_all(pr, s), m[j][e], v[j][e], bc1, bc2, flags);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
+        store_group<PD, E, false>(PO, off, p[j]);
+        if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m[j]);
+        if (use_v) store_group<MXOPT_F32, E, false>(V, off, v[j]);
+      }
+    } else {
+      const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
+      for (uint32_t q = tid; q < ngroups; q += kThreads) {
+        const uint64_t off = start + (uint64_t)q * E;
+        float p[E], g[E], x[E], m[E], v[E];
+        load_group<PD, E, false>(P, off, p);
+        load_group<GD, E, false>(G, off, g);
+#pragma unroll
+        for (int k = 0; k < kMaxPending; ++k) {
+          if (k < kx) {
+            load_group<XD, E, false>(ps.x[k], off, x);
+#pragma unroll
+            for (int e = 0; e < E; ++e) g[e] = g[e] + x[e];
+          }
+        }
+        if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m);
+        if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) math(p[e], prep_all(pr, g[e]), m[e], v[e], bc1, bc2, flags);
+        store_group<PD, E, false>(PO, off, p);
+        if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
+        if (use_v) store_group<MXOPT_F32, E, false>(V, off, v);
+      }
+      for (uint32_t i = ngroups * E + tid; i < len; i += kThreads) one_element(start + i);
+    }
+    if (tid < cv.head) one_element(tid);
+  }
+}
+
+// Sum of squares of prep_pre(g + x_0 + ...), nothing stored: the norm the update above will clip by.
+template <int GD, int XD, bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* __restrict__ T,
+                                                              const DevChunk* __restrict__ C, DevTensor one,
+                                                              uint32_t nchunks, uint32_t ntensors,
+                                                              const void* const* __restrict__ X, int kx, DevPrep prep,
+                                                              double* __restrict__ partial_sum) {
+  constexpr int E = (GD != MXOPT_F32 || XD != MXOPT_F32) ? 8 : 4;
+  constexpr int U = kElemsPerLane / E;
+  const PrepRegs pr = load_prep(prep);
+  const bool clamped = (pr.flags & kPrepClampPre) != 0;
+  const uint32_t tid = threadIdx.x;
+  double acc_sum = 0.0;
+
+  for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+    const ChunkView cv = locate(T, C, one, c);
+    const PendingStreams ps = pending_of(X, ntensors, cv.tensor, kx);
+    const void* G = cv.t.g;
+    float s32 = 0.0f;
+    bool bad = false;
+    auto one_element = [&](uint64_t off) {
+      const float y = norm_value(pr, pending_sum_element<GD, XD>(G, ps, kx, off), clamped, bad);
+      s32 = fmaf(y, y, s32);
+    };
+    if (cv.fast) {
+      float g[U][E], x[kMaxPending][U][E];
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
+        load_group<GD, E, NT>(G, off, g[j]);
+#pragma unroll
+        for (int k = 0; k < kMaxPending; ++k)
+          if (k < kx) load_group<XD, E, NT>(ps.x[k], off, x[k][j]);
+      }
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          float s = g[j][e];
+#pragma unroll
+          for (int k = 0; k < kMaxPending; ++k)
+            if (k < kx) s = s + x[k][j][e];
+          const float y = norm_value(pr, s, clamped, bad);
+          s32 = fmaf(y, y, s32);
+        }
+      }
+    } else {
+      const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
+      for (uint32_t q = tid; q < ngroups; q += kThreads) {
+        const uint64_t off = cv.start + (uint64_t)q * E;
+        float g[E], x[E];
+        load_group<GD, E, false>(G, off, g);
+#pragma unroll
+        for (int k = 0; k < kMaxPending; ++k) {
+          if (k < kx) {
+            load_group<XD, E, false>(ps.x[k], off, x);
+#pragma unroll
+            for (int e = 0; e < E; ++e) g[e] = g[e] + x[e];
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const float y = norm_value(pr, g[e], clamped, bad);
+          s32 = fmaf(y, y, s32);
+        }
+      }
+      for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) one_element(cv.start + i);
+    }
+    if (tid < cv.head) one_element(tid);
+    // As in sumsq_kernel: float32 inside a chunk, float64 across chunks; a hidden NaN/Inf poisons the partial.
+    acc_sum += (double)(bad ? __builtin_nanf("") : s32);
+  }
+
+  unsigned long long unused = 0;
+  block_sum(acc_sum, unused);
+  if (tid == 0) partial_sum[blockIdx.x] = acc_sum;
+}
+
 // Pass 2: one workgroup folds the partials in a fixed order and derives norm and scale.
 __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __restrict__ partial_sum,
                                                                uint32_t npartials, double max_norm, int has_max,
@@ -695,6 +902,75 @@ bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep
     case 1: return sumsq_for_mode<1>(ad, gd, L, prep, first, partial_sum);
     case 2: return sumsq_for_mode<2>(ad, gd, L, prep, first, partial_sum);
     case 3: return sumsq_for_mode<3>(ad, gd, L, prep, first, partial_sum);
+  }
+  return false;
+}
+
+#define MXOPT_LAUNCH_LIST(kernel, L, ...)                                                                     \
+  hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).one, \
+                     (L).nchunks, (L).ntensors, (L).pending, (L).npending, __VA_ARGS__)
+
+// g is either of the pending streams' dtype (the first micro-batch) or float32 (a buffer of earlier ones).
+template <int PD, class Math>
+static bool update_list_for_pd(int gd, int xd, const Launch& L, const Math& math, const DevPrep& prep) {
+  if (gd != xd && gd != MXOPT_F32) return false;
+  const bool same = gd == xd;
+  switch (xd) {
+    case MXOPT_F32:
+      MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F32, Math>), L, math, prep);
+      return true;
+    case MXOPT_BF16:
+      if (same) MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_BF16, MXOPT_BF16, Math>), L, math, prep);
+      else MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_BF16, Math>), L, math, prep);
+      return true;
+    case MXOPT_F16:
+      if (same) MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F16, MXOPT_F16, Math>), L, math, prep);
+      else MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F16, Math>), L, math, prep);
+      return true;
+  }
+  return false;
+}
+
+bool launch_adam_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
+  if (od != pd) return false;
+  switch (pd) {
+    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, AdamMath{hp}, prep);
+    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, AdamMath{hp}, prep);
+    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, AdamMath{hp}, prep);
+  }
+  return false;
+}
+
+bool launch_sgd_plain_list(int pd, int gd, int od, int xd, const Launch& L, float lr_p, float wd, int has_wd,
+                           const DevPrep& prep) {
+  if (od != pd) return false;
+  switch (pd) {
+    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, PlainSgdMath<MXOPT_F32, false>{lr_p, wd, has_wd}, prep);
+    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, PlainSgdMath<MXOPT_BF16, false>{lr_p, wd, has_wd}, prep);
+    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, PlainSgdMath<MXOPT_F16, false>{lr_p, wd, has_wd}, prep);
+  }
+  return false;
+}
+
+template <int GD, int XD>
+static void launch_sumsq_list_t(const Launch& L, const DevPrep& prep, double* ps) {
+  if (L.nontemporal) MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, true>), L, prep, ps);
+  else MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, false>), L, prep, ps);
+}
+
+bool launch_sumsq_list(int gd, int xd, const Launch& L, const DevPrep& prep, double* partial_sum) {
+  if (gd != xd && gd != MXOPT_F32) return false;
+  const bool same = gd == xd;
+  switch (xd) {
+    case MXOPT_F32: launch_sumsq_list_t<MXOPT_F32, MXOPT_F32>(L, prep, partial_sum); return true;
+    case MXOPT_BF16:
+      if (same) launch_sumsq_list_t<MXOPT_BF16, MXOPT_BF16>(L, prep, partial_sum);
+      else launch_sumsq_list_t<MXOPT_F32, MXOPT_BF16>(L, prep, partial_sum);
+      return true;
+    case MXOPT_F16:
+      if (same) launch_sumsq_list_t<MXOPT_F16, MXOPT_F16>(L, prep, partial_sum);
+      else launch_sumsq_list_t<MXOPT_F32, MXOPT_F16>(L, prep, partial_sum);
+      return true;
   }
   return false;
 }

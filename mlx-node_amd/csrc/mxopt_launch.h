@@ -20,6 +20,10 @@ struct Launch {
   uint32_t grid = 0;                 // workgroups (<= nchunks)
   hipStream_t stream = nullptr;
   int nontemporal = 0;               // non-zero: streaming-hint loads and stores
+  // Deferred accumulation (the *_list launchers): stream j of table row r is pending[j * ntensors + r].
+  const void* const* pending = nullptr;
+  uint32_t ntensors = 0;
+  int npending = 0;
 };
 
 // Each returns false when the dtype combination has no kernel.
@@ -40,6 +44,12 @@ bool launch_transform(int gd, int od, const Launch& L, const DevPrep& prep, int 
 // 3: square g_out + g without storing it.
 // partial_sum (one entry per workgroup) may be NULL in mode 2.
 bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum);
+// Deferred accumulation: the gradient is g + pending_0 + ... (float32 adds, left to right); xd is the
+// pending streams' dtype, gd either xd or float32.  Parameters are updated in their own dtype.
+bool launch_adam_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep);
+bool launch_sgd_plain_list(int pd, int gd, int od, int xd, const Launch& L, float lr_p, float wd, int has_wd,
+                           const DevPrep& prep);
+bool launch_sumsq_list(int gd, int xd, const Launch& L, const DevPrep& prep, double* partial_sum);
 bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
                   uint32_t grid, hipStream_t stream);
 void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,

@@ -88,6 +88,12 @@ SIGNATURES = {
     "mxopt_sgd_hp_from_f64": (C.c_int, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_int, C.POINTER(SgdHp)]),
     "mxopt_rmsprop_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.POINTER(RmspropHp)]),
     "mxopt_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_table_set_pending": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.c_int]),
+    "mxopt_norm_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                               C.c_void_p]),
+    "mxopt_adam_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_sgd_plain_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
+                                                    C.POINTER(GradPrep)]),
     "mxopt_adam_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
     "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),

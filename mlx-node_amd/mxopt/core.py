@@ -223,7 +223,27 @@ def _accumulate_norm_only(self, table: "Table", out: NormResultBuffer, prep: Opt
                                                 max_norm, clip_mode, C.c_void_p(out.ptr)), self.handle)
 
 
+def _norm_with_pending_list(self, table: "Table", out: NormResultBuffer, prep: Optional[L.GradPrep] = None,
+                            max_norm: float = -1.0, clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
+    L.check(self.lib.mxopt_norm_with_pending_list(self.handle, table.handle, C.byref(prep) if prep else None,
+                                                  max_norm, clip_mode, C.c_void_p(out.ptr)), self.handle)
+
+
+def _adam_with_pending_list(self, table: "Table", hp: L.AdamHp, prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_adam_with_pending_list(self.handle, table.handle, C.byref(hp),
+                                                  C.byref(prep) if prep else None), self.handle)
+
+
+def _sgd_plain_with_pending_list(self, table: "Table", learning_rate: float, weight_decay: float = 0.0,
+                                 prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_sgd_plain_with_pending_list(self.handle, table.handle, learning_rate, weight_decay,
+                                                       C.byref(prep) if prep else None), self.handle)
+
+
 Context.accumulate_norm_only = _accumulate_norm_only
+Context.norm_with_pending_list = _norm_with_pending_list
+Context.adam_with_pending_list = _adam_with_pending_list
+Context.sgd_plain_with_pending_list = _sgd_plain_with_pending_list
 Context.accumulate_transformed = _accumulate_transformed
 Context.fill_synthetic = _fill_synthetic
 Context.sgd_plain_with_pending = _sgd_plain_with_pending
@@ -256,6 +276,26 @@ class Table:
             arr[i] = r.to_c()
         L.check(self.ctx.lib.mxopt_table_retarget(self.handle, arr, len(rows)), self.ctx.handle)
         self.rows = rows
+
+    def set_pending(self, streams: Sequence[Sequence[torch.Tensor]]) -> None:
+        """Deferred accumulation: streams[j][i] is pending gradient j of row i (all of one dtype)."""
+        streams = [list(s) for s in streams]
+        k, n = len(streams), len(self.rows)
+        if k == 0:
+            L.check(self.ctx.lib.mxopt_table_set_pending(self.handle, 0, None, 0), self.ctx.handle)
+            self.pending = []
+            return
+        if any(len(s) != n for s in streams):
+            raise L.InvalidArg(L.ERR_INVALID_ARG, "every pending stream needs one tensor per table row")
+        flat = [t for s in streams for t in s]
+        if any(not t.is_contiguous() for t in flat):
+            raise L.InvalidArg(L.ERR_INVALID_ARG, "mxopt needs dense (contiguous) buffers")
+        if any(t.dtype != flat[0].dtype for t in flat):
+            raise L.InvalidArg(L.ERR_INVALID_ARG, "pending streams must share one dtype")
+        arr = (C.c_void_p * max(len(flat), 1))(*[_dev_ptr(t) for t in flat])
+        code = dtype_code(flat[0]) if flat else 0
+        L.check(self.ctx.lib.mxopt_table_set_pending(self.handle, k, arr, code), self.ctx.handle)
+        self.pending = streams   # keeps the tensors alive
 
     @property
     def total_elems(self) -> int:
