@@ -75,6 +75,22 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
                                 const mxopt_array* params, const mxopt_array* grads, const mxopt_array* outs,
                                 const mxopt_grad_prep* prep);
 
+/* update_many over k micro-batches that were never summed (deferred accumulation, see mxopt.h):
+ * the gradient of parameter i is grads[i] + grads[n + i] + ... + grads[(k-1) n + i], added left to
+ * right in float32 -- the sum k-1 calls of Qwen3Model::accumulate_gradients (model.rs:2217-2243)
+ * would have left in a float32 buffer -- then `prep`, then, when max_norm >= 0, the clip factor of
+ * GradientUtils::clip_grad_norm (optimizers/mod.rs:67-107; clip_mode as in mxopt_global_norm) of
+ * that gradient's global norm, then the Adam/AdamW update with update_many's per-call step
+ * counting.  Two launches per dtype group, no accumulation buffer, no host synchronisation.
+ * 1 <= k <= MXOPT_MAX_PENDING + 1; micro-batches 2..k share one dtype, the first has it or is
+ * float32; outs[i] has params[i]'s dtype (it may be params[i] itself); Adam and AdamW only.
+ * d_norm (nullable, device memory) receives norm, clip factor and the non-finite flag; pass
+ * prep->d_skip_if_nonzero = &d_norm->nonfinite to leave everything untouched on a NaN/Inf gradient. */
+int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, const char* const* param_names,
+                                            const mxopt_array* params, size_t k, const mxopt_array* grads,
+                                            const mxopt_array* outs, const mxopt_grad_prep* prep, double max_norm,
+                                            int clip_mode, mxopt_norm_result* d_norm);
+
 /* reset(): drops all state; Adam/AdamW also zero the call counter (adam.rs:143-146,
  * adamw.rs:146-150, sgd.rs:157-159, rmsprop.rs:119-121). */
 int mxopt_optimizer_reset(mxopt_optimizer* opt);

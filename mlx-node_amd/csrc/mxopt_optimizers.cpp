@@ -336,14 +336,18 @@ int mxopt_optimizer_update_single(mxopt_optimizer* opt, const char* param_name, 
   return MXOPT_OK;
 }
 
-int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* const* param_names,
-                                const mxopt_array* params, const mxopt_array* grads, const mxopt_array* outs,
-                                const mxopt_grad_prep* prep) {
-  if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "update_many: optimizer is NULL");
+}  // extern "C"
+
+// Rows, per-call step scalars and the cached table of one batched update; shared by update_many and
+// update_many_accumulated.  On return opt->many_table describes `rows` and *hp holds the coefficients.
+static int prepare_many(mxopt_optimizer* opt, size_t n, const char* const* param_names, const mxopt_array* params,
+                        const mxopt_array* grads, const mxopt_array* outs, std::vector<StateEntry*>* states_out,
+                        Hp* hp_out) {
   mxopt_ctx* ctx = opt->ctx;
-  if (n && (!param_names || !params || !grads || !outs)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "update_many: null argument");
   std::vector<mxopt_tensor> rows(n);
-  std::vector<StateEntry*> states(n, nullptr);
+  std::vector<StateEntry*>& states = *states_out;
+  states.assign(n, nullptr);
+  Hp& hp = *hp_out;
   const int64_t step_before = opt->step;
   for (size_t i = 0; i < n; ++i) {
     int rc = fill_row(opt, param_names[i], &params[i], &grads[i], &outs[i], &rows[i], &states[i]);
@@ -352,7 +356,6 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
       return rc;
     }
   }
-  Hp hp;
   int rc = make_hp(opt, &hp);
   if (rc) return rc;
   // Same buffers as last time?  Then only the per-step scalars change.
@@ -388,6 +391,21 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
       if ((rc = mxopt_table_set_step_scalars(opt->many_table, b1.data(), b2.data(), fl.data()))) return rc;
     }
   }
+  return MXOPT_OK;
+}
+
+extern "C" {
+
+int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* const* param_names,
+                                const mxopt_array* params, const mxopt_array* grads, const mxopt_array* outs,
+                                const mxopt_grad_prep* prep) {
+  if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "update_many: optimizer is NULL");
+  mxopt_ctx* ctx = opt->ctx;
+  if (n && (!param_names || !params || !grads || !outs)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "update_many: null argument");
+  std::vector<StateEntry*> states;
+  Hp hp;
+  int rc = prepare_many(opt, n, param_names, params, grads, outs, &states, &hp);
+  if (rc) return rc;
   switch (opt->kind) {
     case Kind::Adam:
     case Kind::AdamW: rc = mxopt_adam(ctx, opt->many_table, &hp.adam, prep); break;
@@ -398,6 +416,57 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
   if (opt->kind == Kind::Sgd && opt->momentum != 0.0)
     for (StateEntry* st : states) st->has_velocity = true;
   return MXOPT_OK;
+}
+
+int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, const char* const* param_names,
+                                            const mxopt_array* params, size_t k, const mxopt_array* grads,
+                                            const mxopt_array* outs, const mxopt_grad_prep* prep, double max_norm,
+                                            int clip_mode, mxopt_norm_result* d_norm) {
+  const char* op = "update_many_accumulated";
+  if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": optimizer is NULL");
+  mxopt_ctx* ctx = opt->ctx;
+  if (!is_adam(opt)) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": Adam and AdamW only");
+  if (k < 1 || k > (size_t)MXOPT_MAX_PENDING + 1)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                std::string(op) + ": between 1 and " + std::to_string(MXOPT_MAX_PENDING + 1) + " micro-batches");
+  if (n && (!param_names || !params || !grads || !outs))
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
+  if (prep && prep->d_scale && max_norm >= 0.0)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": prep->d_scale and max_norm exclude each other");
+  // Every later micro-batch must look like the first: same sizes, one dtype.
+  int xd = n && k > 1 ? grads[n].dtype : MXOPT_F32;
+  for (size_t j = 1; j < k; ++j) {
+    for (size_t i = 0; i < n; ++i) {
+      const mxopt_array& g = grads[j * n + i];
+      int rc = check_array(ctx, &g, "update_many_accumulated: gradient");
+      if (rc) return rc;
+      if (g.n != grads[i].n || g.dtype != xd)
+        return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                    std::string(op) + ": micro-batch " + std::to_string(j) + " of '" + param_names[i] +
+                        "' differs from the first in size, or from the other pending ones in dtype");
+    }
+  }
+  const int64_t step_before = opt->step;
+  std::vector<StateEntry*> states;
+  Hp hp;
+  int rc = prepare_many(opt, n, param_names, params, grads, outs, &states, &hp);
+  if (rc) return rc;
+  std::vector<const void*> streams((k - 1) * n);
+  for (size_t j = 1; j < k; ++j)
+    for (size_t i = 0; i < n; ++i) streams[(j - 1) * n + i] = grads[j * n + i].data;
+  rc = mxopt_table_set_pending(opt->many_table, (int)(k - 1), streams.data(), xd);
+  mxopt_grad_prep local;
+  if (prep) local = *prep; else std::memset(&local, 0, sizeof local);
+  if (!rc && max_norm >= 0.0) {
+    mxopt_norm_result* slot = d_norm;
+    if (!slot) rc = norm_scratch(ctx, &slot);
+    if (!rc) rc = mxopt_norm_with_pending_list(ctx, opt->many_table, &local, max_norm, clip_mode, slot);
+    local.d_scale = &slot->scale;
+  }
+  if (!rc) rc = mxopt_adam_with_pending_list(ctx, opt->many_table, &hp.adam, &local);
+  (void)mxopt_table_set_pending(opt->many_table, 0, nullptr, 0);
+  if (rc) opt->step = step_before;  // the update was not launched
+  return rc;
 }
 
 int mxopt_optimizer_reset(mxopt_optimizer* opt) {

@@ -135,6 +135,9 @@ SIGNATURES.update({
     "mxopt_optimizer_update_single": (C.c_int, [C.c_void_p, C.c_char_p, _PA, _PA, _PA]),
     "mxopt_optimizer_update_many": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA, _PA, _PA,
                                               C.POINTER(GradPrep)]),
+    "mxopt_optimizer_update_many_accumulated": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA, C.c_size_t,
+                                                          _PA, _PA, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                                          C.c_void_p]),
     "mxopt_optimizer_reset": (C.c_int, [C.c_void_p]),
     "mxopt_optimizer_step_count": (C.c_int64, [C.c_void_p]),
     "mxopt_optimizer_state": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),

@@ -95,6 +95,25 @@ class _Optimizer:
                                                      C.byref(prep) if prep else None), self.ctx.handle)
         return list(outs)
 
+    def update_many_accumulated(self, names: Sequence[str], params: Sequence[torch.Tensor],
+                                micro_batches: Sequence[Sequence[torch.Tensor]],
+                                outs: Optional[Sequence[torch.Tensor]] = None, prep: Optional[L.GradPrep] = None,
+                                max_norm: float = -1.0, clip_mode: int = L.CLIP_ALWAYS_MULTIPLY,
+                                norm_out=None) -> List[torch.Tensor]:
+        """One Adam/AdamW step on the sum of `micro_batches` (added in registers, in order, in float32),
+        clipped to `max_norm` by its global norm when max_norm >= 0.  In place unless `outs` is given."""
+        if outs is None:
+            outs = list(params)
+        n, k = len(names), len(micro_batches)
+        if any(len(mb) != n for mb in micro_batches):
+            raise L.InvalidArg(L.ERR_INVALID_ARG, "every micro-batch needs one gradient per name")
+        cnames = (C.c_char_p * max(n, 1))(*[s.encode() for s in names])
+        flat = [g for mb in micro_batches for g in mb]
+        L.check(self.lib.mxopt_optimizer_update_many_accumulated(
+            self.handle, n, cnames, _arrs(params), k, _arrs(flat), _arrs(outs), C.byref(prep) if prep else None,
+            max_norm, clip_mode, C.c_void_p(norm_out.ptr) if norm_out is not None else None), self.ctx.handle)
+        return list(outs)
+
     def reset(self) -> None:
         L.check(self.lib.mxopt_optimizer_reset(self.handle), self.ctx.handle)
 

@@ -248,3 +248,40 @@ def test_set_pending_rejects_what_the_kernels_cannot_walk(mx, ctx):
     ctx.adam_with_pending_list(t, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01))
     ctx.synchronize()
     t.close()
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f32"])
+def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind):
+    """update_many_accumulated == accumulate_gradients (float32 buffer) k-1 times, clip_grad_norm,
+    then update_single tensor by tensor, including the per-call step count under bias correction;
+    two optimizer steps, the second with fresh buffers (table retargeted) and fewer micro-batches."""
+    sizes = [3, 4096, 5000, 70001]
+    names = [f"layers.{i}.w" for i in range(len(sizes))]
+    ps = lists(41, sizes, kind, 0.02)
+    opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True, ctx=ctx)
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+    dp = [to_dev(p) for p in ps]
+    res = ctx.norm_result()
+    cur = ps
+    for step, k in enumerate((4, 2)):
+        micro = [lists(50 + 10 * step + j, sizes, kind, 1e-3) for j in range(k)]
+        dmicro = [[to_dev(g) for g in mb] for mb in micro]
+        opt.update_many_accumulated(names, dp, dmicro, max_norm=1e-2, norm_out=res)
+        acc = oracle_sum(micro[0], micro[1:])
+        scale = device_scale(ctx, res, acc, 1e-2)
+        nxt = []
+        for i, name in enumerate(names):
+            want = cast(ref.update_single(name, cur[i], acc[i] * scale), kind)
+            assert_bit_equal(to_host(dp[i]), want, f"step {step} {name}")
+            m, v = opt.state(name)
+            assert_bit_equal(to_host(m), ref.state[name][0], f"m {name}")
+            assert_bit_equal(to_host(v), ref.state[name][1], f"v {name}")
+            nxt.append(want)
+        cur = nxt
+        assert opt.step == ref.step == (step + 1) * len(names)
+    # a refused call leaves the counter alone
+    with pytest.raises(mx.InvalidArg, match="between 1 and 4"):
+        opt.update_many_accumulated(names, dp, [dmicro[0]] * 5)
+    with pytest.raises(mx.InvalidArg, match="Adam and AdamW only"):
+        mx.SGD(0.1, ctx=ctx).update_many_accumulated(names, dp, dmicro)
+    assert opt.step == 2 * len(names)

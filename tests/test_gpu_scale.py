@@ -16,6 +16,9 @@
   last micro-batch folded into the update (config 5, ~131 GB resident): seeded windows of every stream
   are read back before and after the step and pushed through the NumPy oracle (bit-exact given the
   device's clip factor); norm as above.
+* The same configuration without its accumulation buffer (deferred accumulation: the four resident
+  micro-batches are summed in registers): the same sum of squares and a position-weighted checksum of
+  EVERY parameter and moment bit equal to those of the buffered run from identical generated inputs.
 """
 import math
 
@@ -409,4 +412,83 @@ def test_config5_full_size_windows_and_norm():
     assert np.array_equal(win(v_slab).view(np.uint32), ref.state["w"][1].view(np.uint32)), "second moment"
     t_acc.close()
     t_upd.close()
+    ctx.close()
+
+
+def bit_checksums(torch, slab, piece=1 << 26):
+    """(sum of the bit patterns, sum of bit pattern x (1 + position mod 65521)) over a whole slab, in
+    wrapping int64: a single flipped bit, or two equal values changing places, changes one of them."""
+    bits = slab.view(torch.int16 if slab.element_size() == 2 else torch.int32)
+    plain = weighted = 0
+    for start in range(0, bits.numel(), piece):
+        b = bits[start:start + piece].to(torch.int64)
+        w = torch.arange(start, start + b.numel(), device=slab.device, dtype=torch.int64).remainder_(65521).add_(1)
+        plain = (plain + int(b.sum())) & (2 ** 64 - 1)
+        weighted = (weighted + int((b * w).sum())) & (2 ** 64 - 1)
+    return plain, weighted
+
+
+def test_config5_deferred_accumulation_equals_buffered_every_element():
+    import torch
+    import mxopt as mx
+    _, sizes = qwen_sizes("8B")
+    n = sum(sizes)
+    free, _ = torch.cuda.mem_get_info()
+    if free < n * 22 + (12 << 30):
+        pytest.skip("needs ~190 GB of free device memory")
+    bf = torch.bfloat16
+    p_slab, offs, dp = carve(torch, sizes, bf)
+    m_slab, _, dm = carve(torch, sizes, torch.float32)
+    v_slab, _, dv = carve(torch, sizes, torch.float32)
+    micro = [carve(torch, sizes, bf) for _ in range(4)]
+    ctx = mx.Context()
+    seed = 0x5EED0055
+
+    def generate():
+        for i in range(len(sizes)):
+            ctx.fill_synthetic(dp[i], mx.synthetic_key(seed, 5, 0, 0, i), mx.SYNTH_NORMAL, 0.02)
+            ctx.fill_synthetic(dm[i], mx.synthetic_key(seed, 5, 0, 1, i), mx.SYNTH_NORMAL, 1e-4)
+            ctx.fill_synthetic(dv[i], mx.synthetic_key(seed, 5, 0, 2, i), mx.SYNTH_UNIFORM, 0.0, 1e-8)
+
+    for k, (_, _, dg) in enumerate(micro):
+        for i in range(len(sizes)):
+            ctx.fill_synthetic(dg[i], mx.synthetic_key(seed, 5, 0, 3 + k, i), mx.SYNTH_NORMAL, 1e-3)
+    hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
+    res = ctx.norm_result()
+
+    # buffered: three accumulation passes, the fourth micro-batch measured and folded into the update
+    generate()
+    a_slab, _, da = carve(torch, sizes, torch.float32)
+    for k in range(4):
+        t_acc = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(micro[k][2], da)])
+        if k < 3:
+            ctx.accumulate(t_acc, first=(k == 0))
+        else:
+            ctx.accumulate_norm_only(t_acc, res, max_norm=1.0)
+        ctx.synchronize()
+        t_acc.close()
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=g, m=m, v=v)
+                       for p, a, g, m, v in zip(dp, da, micro[3][2], dm, dv)])
+    ctx.adam_with_pending(t_upd, hp, mx.make_prep(scale=res))
+    r_buf = ctx.read_norm_result(res)
+    t_upd.close()
+    del a_slab, da
+    sums_buf = [bit_checksums(torch, s) for s in (p_slab, m_slab, v_slab)]
+
+    # deferred: no buffer; the inputs are regenerated, the micro-batches are still where they were
+    generate()
+    sums_before = [bit_checksums(torch, s) for s in (p_slab, m_slab, v_slab)]
+    assert sums_before != sums_buf                       # the update did change every stream
+    t_def = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, micro[0][2], dm, dv)])
+    t_def.set_pending([mb[2] for mb in micro[1:]])
+    ctx.norm_with_pending_list(t_def, res, max_norm=1.0)
+    ctx.adam_with_pending_list(t_def, hp, mx.make_prep(scale=res))
+    r_def = ctx.read_norm_result(res)
+    sums_def = [bit_checksums(torch, s) for s in (p_slab, m_slab, v_slab)]
+
+    assert r_def.sumsq == r_buf.sumsq and r_def.scale == r_buf.scale and r_def.nonfinite == 0
+    expected_norm = 1e-3 * math.sqrt(4 * n)
+    assert abs(r_def.norm - expected_norm) < 0.01 * expected_norm
+    assert sums_def == sums_buf
+    t_def.close()
     ctx.close()
