@@ -23,11 +23,11 @@
  * may be used from different threads.  Kernels are enqueued on the context's stream;
  * no call synchronises with the host except mxopt_synchronize / mxopt_read_*.
  *
- * HIP graphs: the kernel entry points (mxopt_adam ... mxopt_accumulate_norm_only) only launch
+ * HIP graphs: the kernel entry points (mxopt_adam ... mxopt_norm_with_pending_list) only launch
  * kernels -- no allocation, copy or memset -- once the first reduction call on a context has
  * allocated its per-workgroup partials buffer, so a step may be recorded into a graph after
- * one eager warm-up call.  mxopt_table_build and mxopt_table_set_step_scalars copy from host
- * memory and stay outside a capture.
+ * one eager warm-up call.  mxopt_table_build, mxopt_table_set_step_scalars, mxopt_table_retarget
+ * and mxopt_table_set_pending copy from host memory and stay outside a capture.
  */
 #ifndef MXOPT_H
 #define MXOPT_H

@@ -287,7 +287,7 @@ int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
   if (!ctx || !name) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: null argument");
   std::string n(name);
   if (n == "grid_blocks_per_cu") {
-    if (value < 1 || value > 64) return fail(ctx, MXOPT_ERR_INVALID_ARG, "grid_blocks_per_cu must be in [1, 64]");
+    if (value < 1 || value > 1024) return fail(ctx, MXOPT_ERR_INVALID_ARG, "grid_blocks_per_cu must be in [1, 1024]");
     ctx->grid_blocks_per_cu = (int)value;
   } else if (n == "persistent") {
     ctx->persistent = value != 0;
@@ -764,13 +764,20 @@ int mxopt_norm_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxo
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unknown clip mode");
   DeviceGuard guard(ctx->device);
   const DevPrep dp = make_prep(prep);
+  // Several read-only streams at once: measured 10 % faster with four times the workgroups of the
+  // one- and two-stream reductions (11.2 -> 10.2 ms on the 8B list with four bf16 micro-batches).
+  auto list_grid = [&](uint32_t nchunks) {
+    const uint64_t cap = (uint64_t)ctx->num_cus * (uint64_t)ctx->grid_blocks_per_cu * 4u;
+    return (uint32_t)std::min<uint64_t>(nchunks, std::max<uint64_t>(cap, 1));
+  };
   size_t total_grid = 0;
-  for (const Group& g : t->groups) total_grid += persistent_grid(ctx, g.nchunks);
+  for (const Group& g : t->groups) total_grid += list_grid(g.nchunks);
   rc = ensure_partials(ctx, std::max<size_t>(total_grid, 1));
   if (rc) return rc;
   size_t offset = 0;
   for (const Group& g : t->groups) {
     Launch L = make_launch(ctx, t, g, true);
+    L.grid = list_grid(g.nchunks);
     L.nontemporal = ctx->nontemporal_reduce;
     attach_pending(t, L);
     if (!launch_sumsq_list(g.gd, t->pending_k ? t->pending_dtype : g.gd, L, dp, ctx->d_partial_sum + offset))

@@ -128,8 +128,8 @@ def test_adamw_over_deferred_micro_batches(mx, ctx, combo, k, layout):
 
 def test_deferred_equals_buffered_path_bit_for_bit(mx, ctx):
     """Four bf16 micro-batches: accumulate x3 + accumulate_norm_only + adam_with_pending (float32 buffer)
-    against norm_with_pending_list + adam_with_pending_list (no buffer): same sum of squares, same clip
-    factor, same parameters and moments."""
+    against norm_with_pending_list + adam_with_pending_list (no buffer): same sum of squares (to float64
+    rounding), same clip factor, same parameters and moments."""
     import torch
     sizes = [4096 * 5 + 3, 17, 4096, 250001]
     ps = lists(7, sizes, "bf16", 0.02)
@@ -161,7 +161,8 @@ def test_deferred_equals_buffered_path_bit_for_bit(mx, ctx):
         r = ctx.read_norm_result(res)
         out.append((r.sumsq, r.scale, [to_host(x) for x in dp], [to_host(x) for x in dm], [to_host(x) for x in dv]))
     a, b = out
-    assert a[0] == b[0] and a[1] == b[1]
+    # the two norm passes fold their per-workgroup float64 partials over different grids
+    assert abs(a[0] - b[0]) <= 1e-12 * a[0] and a[1] == b[1]
     for i in range(len(sizes)):
         assert_bit_equal(b[2][i], a[2][i], f"p{i}")
         assert_bit_equal(b[3][i], a[3][i], f"m{i}")
