@@ -50,6 +50,9 @@ def parse_args():
     ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab", "packed"],
                     help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
                          "tensors are 512-byte aligned views into it")
+    ap.add_argument("--defer", type=int, default=0,
+                    help="engine workloads: 1 = defer_accumulation (four resident micro-batches, no accumulation "
+                         "buffer, summed in registers by the applying call)")
     ap.add_argument("--fold-last", type=int, default=1,
                     help="cfg5: 1 = the last micro-batch is measured (norm) but folded into the update instead of "
                          "being written to the accumulation buffer; 0 = four plain accumulation passes")
@@ -350,23 +353,40 @@ class Workload:
         self.p = self._randn_list(bf, 0.02)
         self.g = self._randn_list(bf, 1e-3)
         params = dict(zip(self.names, self.p))
-        self.grads = dict(zip(self.names, self.g))
         self.n_micro = 4
+        defer = bool(self.args.defer)
+        # deferred accumulation reads every micro-batch of the cycle at the end: they must all be resident
+        self.micro = [dict(zip(self.names, self.g))]
+        for _ in range(self.n_micro - 1 if defer else 0):
+            self.micro.append(dict(zip(self.names, self._randn_list(bf, 1e-3))))
         if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
             self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=4,
-                                                     ctx=self.ctx)
-            self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10}
-            self.note = "per micro-batch: validity+norm of clamp(g) (2 B), acc += clip(clamp(g)) (6/10 B), 32-byte read-back"
+                                                     defer_accumulation=defer, ctx=self.ctx)
+            if defer:
+                self.bytes_per_elem = {"micro_batch_first": 2, "micro_batch": 2, "micro_batch_apply": 2 + 4 * 2 + 4}
+                self.note = ("per micro-batch: validity+norm of clamp(g) (2 B), 32-byte read-back; the last call adds "
+                             "sum_j clip_j(clamp(g_j)) in registers and applies lr/N (12 B)")
+            else:
+                self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10}
+                self.note = "per micro-batch: validity+norm of clamp(g) (2 B), acc += clip(clamp(g)) (6/10 B), 32-byte read-back"
         else:                # acc += g in float32, last pass carries the norm of acc/N; p -= lr*(clip(acc/N) + wd*p)
             self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=4,
-                                                    weight_decay=0.01, accumulate_in_f32=True, ctx=self.ctx)
-            self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 6 + 10}
-            self.note = "float32 accumulation buffer; last micro-batch: norm of (acc+g)/N read-only, then folded into the update"
-        self.step_bytes_per_elem = (self.bytes_per_elem["micro_batch_first"] + 2 * self.bytes_per_elem["micro_batch"] +
+                                                    weight_decay=0.01, accumulate_in_f32=True,
+                                                    defer_accumulation=defer, ctx=self.ctx)
+            if defer:
+                self.bytes_per_elem = {"micro_batch_apply": 4 * 2 + 4 * 2 + 4}
+                self.note = ("micro-batches 1-3 only leave their addresses; the last call takes the norm of sum/N "
+                             "(8 B, read only) and updates from the same four streams (12 B)")
+            else:
+                self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 6 + 10}
+                self.note = "float32 accumulation buffer; last micro-batch: norm of (acc+g)/N read-only, then folded into the update"
+        self.step_bytes_per_elem = (self.bytes_per_elem.get("micro_batch_first", 0) +
+                                    2 * self.bytes_per_elem.get("micro_batch", 0) +
                                     self.bytes_per_elem["micro_batch_apply"])
         self.dominant = "micro_batch_apply"
         self.dtype = "f32"
-        self.storage = "bf16 parameters and gradients, float32 accumulation buffer"
+        self.storage = ("bf16 parameters and gradients, no accumulation buffer" if defer
+                        else "bf16 parameters and gradients, float32 accumulation buffer")
 
     def _setup_grpo_engine(self):
         self._setup_engine("grpo")
@@ -377,7 +397,7 @@ class Workload:
     def _step_grpo_engine(self):
         for k in range(self.n_micro):
             name = "micro_batch_first" if k == 0 else ("micro_batch_apply" if k == self.n_micro - 1 else "micro_batch")
-            self._timed(name, lambda: self.engine.micro_batch(self.grads))
+            self._timed(name, lambda: self.engine.micro_batch(self.micro[k % len(self.micro)]))
 
     _step_sft_engine = _step_grpo_engine
 

@@ -265,6 +265,15 @@ int mxopt_adam_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxo
 int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
                                       double weight_decay, const mxopt_grad_prep* prep);
 
+/* The same update with every micro-batch pre-processed on its own before it is added:
+ * gradient = prep_0(g) + prep_1(x0) + ..., where prep_j is `prep` (d_scale ignored) with the clip factor
+ * read from d_scales[j] (k + 1 device pointers, or all NULL for no factor) -- the GRPO engine's
+ * "clamp, clip by this micro-batch's own norm, accumulate" (grpo/engine.rs:636-661) followed by its
+ * apply_gradients (:666-692), without the accumulation buffer. */
+int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                           double weight_decay, const mxopt_grad_prep* prep,
+                                           const float* const* d_scales);
+
 /* ---- global norm ------------------------------------------------------------------ */
 
 /* Sum of squares of the gradients (after prep's pre_mul / clamp_pre) over the whole

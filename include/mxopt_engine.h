@@ -52,6 +52,16 @@ typedef struct mxopt_engine_config {
   int32_t accumulate_in_f32;           /* SFT: 0 = the reference's accumulator dtype (that of the
                                           gradients: bf16 + bf16 -> bf16), 1 = float32 buffer.
                                           GRPO accumulates clipped (float32) gradients either way */
+  int32_t defer_accumulation;          /* 1 = no accumulation buffer: the engine only remembers where
+                                          each micro-batch's gradients lie and the update adds them in
+                                          registers (float32, arrival order: the numbers of the float32
+                                          buffer, bit for bit).  The caller keeps every gradient buffer of
+                                          a cycle alive and unchanged until the call that applies them
+                                          (or flush_gradients / reset) has returned.  Needs
+                                          gradient_accumulation_steps <= MXOPT_MAX_PENDING + 1, the same
+                                          gradient names in every micro-batch of a cycle, SFT:
+                                          accumulate_in_f32 = 1, GRPO: apply = SGD.  No counterpart in
+                                          the reference. */
 } mxopt_engine_config;
 
 /* The reference's defaults for `kind` (GRPOEngineConfig::default, SftEngineConfig::default). */

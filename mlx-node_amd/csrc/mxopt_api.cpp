@@ -679,6 +679,35 @@ int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, doub
   });
 }
 
+int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
+                                           double weight_decay, const mxopt_grad_prep* prep,
+                                           const float* const* d_scales) {
+  const char* op = "mxopt_sgd_plain_with_pending_list_each";
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG, op);
+  if (rc) return rc;
+  if (!d_scales) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": d_scales is NULL");
+  DevPrep dp = make_prep(prep);
+  dp.d_scale = nullptr;
+  dp.flags |= kPrepEachStream;
+  StreamScales sc{};
+  int with = 0;
+  for (int j = 0; j <= t->pending_k; ++j) {
+    sc.s[j] = d_scales[j];
+    with += d_scales[j] != nullptr;
+  }
+  if (with != 0 && with != t->pending_k + 1)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": either every stream has a clip factor or none");
+  const float lr32 = (float)learning_rate;
+  const float wd32 = (float)weight_decay;
+  const int has_wd = weight_decay > 0.0;
+  return run_update(ctx, t, op, [&](const Group& g, Launch& L) {
+    attach_pending(t, L);
+    L.scales = sc;
+    return launch_sgd_plain_list(g.pd, g.gd, g.pod, t->pending_k ? t->pending_dtype : g.gd, L,
+                                 round_to_dtype(lr32, g.pd), wd32, has_wd, dp);
+  });
+}
+
 int mxopt_grad_transform(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_grad_prep* prep) {
   int rc = require(ctx, t, kNeedG | kNeedGOut, "mxopt_grad_transform");
   if (rc) return rc;

@@ -44,6 +44,10 @@ struct mxopt_engine {
   uint64_t nan_gradient_count = 0;
   uint32_t consecutive_nan_count = 0;
   bool needs_emergency_save = false;
+  // defer_accumulation: where the accepted micro-batches of the current cycle lie.  Column c of every
+  // entry belongs to slot held_slots[c] (the order of the cycle's first micro-batch).
+  std::vector<size_t> held_slots;
+  std::vector<std::vector<mxopt_array>> held;
 };
 
 namespace {
@@ -156,6 +160,77 @@ void end_cycle(mxopt_engine* e) {
   for (Slot& s : e->slots) s.in_acc = false;
   e->have_acc = false;
   e->micro_step = 0;
+  e->held.clear();
+  e->held_slots.clear();
+}
+
+// ---- deferred accumulation ---------------------------------------------------------------
+
+// Remembers where this micro-batch's gradients lie.  The first micro-batch of a cycle fixes the set of
+// names (a name given twice keeps its first gradient, as the maps of the reference would); later ones
+// must bring exactly that set.
+int defer_record(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_array* grads) {
+  mxopt_ctx* ctx = e->ctx;
+  const size_t n = idx.size();
+  if (e->held.empty()) {
+    std::vector<char> seen(e->slots.size(), 0);
+    e->held_slots.clear();
+    std::vector<mxopt_array> first;
+    for (size_t i = 0; i < n; ++i) {
+      if (seen[idx[i]]) continue;
+      seen[idx[i]] = 1;
+      e->held_slots.push_back(idx[i]);
+      first.push_back(grads[i]);
+    }
+    e->held.push_back(std::move(first));
+    return MXOPT_OK;
+  }
+  std::vector<const mxopt_array*> by_slot(e->slots.size(), nullptr);
+  size_t distinct = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (by_slot[idx[i]]) continue;
+    by_slot[idx[i]] = &grads[i];
+    ++distinct;
+  }
+  const char* same_names = "engine: deferred accumulation needs the same gradient names in every micro-batch of a cycle";
+  if (distinct != e->held_slots.size()) return fail(ctx, MXOPT_ERR_INVALID_ARG, same_names);
+  std::vector<mxopt_array> row;
+  const int pending_dtype = e->held.size() > 1 && !e->held[1].empty() ? e->held[1][0].dtype : -1;
+  for (size_t slot : e->held_slots) {
+    if (!by_slot[slot]) return fail(ctx, MXOPT_ERR_INVALID_ARG, same_names);
+    const mxopt_array& g = *by_slot[slot];
+    const int want = pending_dtype >= 0 ? pending_dtype : (row.empty() ? g.dtype : row[0].dtype);
+    const int first_dtype = e->held[0][row.size()].dtype;
+    if (g.dtype != want || (first_dtype != g.dtype && first_dtype != MXOPT_F32))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  "engine: deferred accumulation needs one gradient dtype ('" + e->slots[slot].name + "' differs)");
+    row.push_back(g);
+  }
+  e->held.push_back(std::move(row));
+  return MXOPT_OK;
+}
+
+// Table over the held columns: parameters updated in place, g = the first micro-batch, the later ones
+// attached as pending streams.
+int defer_table(mxopt_engine* e, mxopt_table** out) {
+  mxopt_ctx* ctx = e->ctx;
+  const size_t n = e->held_slots.size();
+  std::vector<mxopt_tensor> rows(n, blank_tensor());
+  for (size_t c = 0; c < n; ++c) {
+    const Slot& s = e->slots[e->held_slots[c]];
+    mxopt_tensor& r = rows[c];
+    r.p = s.param.data; r.p_out = s.param.data;
+    r.p_dtype = r.p_out_dtype = (uint8_t)s.param.dtype;
+    r.g = e->held[0][c].data; r.g_dtype = (uint8_t)e->held[0][c].dtype;
+    r.n = s.param.n;
+  }
+  int rc = cached_table(ctx, rows, out);
+  if (rc) return rc;
+  const size_t k = e->held.size() - 1;
+  std::vector<const void*> streams(k * n);
+  for (size_t j = 0; j < k; ++j)
+    for (size_t c = 0; c < n; ++c) streams[j * n + c] = e->held[j + 1][c].data;
+  return mxopt_table_set_pending(*out, (int)k, streams.data(), k && n ? e->held[1][0].dtype : MXOPT_F32);
 }
 
 // ---- GRPO: grpo/engine.rs:561-704 ------------------------------------------------------
@@ -172,6 +247,7 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
   mxopt_norm_result h;
   std::memset(&h, 0, sizeof h);
   h.scale = 1.0f;
+  mxopt_norm_result* d_result = e->d_result;
   int rc;
   if (n) {
     // One read of the gradients: validity of the raw values and the norm of the clamped ones.
@@ -182,8 +258,10 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     mxopt_table* t = nullptr;
     if ((rc = cached_table(ctx, rows, &t))) return rc;
     const double max_norm = e->cfg.has_gradient_clip_norm ? e->cfg.gradient_clip_norm : -1.0;
-    if ((rc = mxopt_global_norm(ctx, t, 0, &prep, max_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, e->d_result))) return rc;
-    if ((rc = mxopt_read_norm_result(ctx, e->d_result, &h))) return rc;
+    // deferred: every accepted micro-batch of the cycle keeps its own clip factor on the device
+    if (e->cfg.defer_accumulation) d_result += e->held.size();
+    if ((rc = mxopt_global_norm(ctx, t, 0, &prep, max_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, d_result))) return rc;
+    if ((rc = mxopt_read_norm_result(ctx, d_result, &h))) return rc;
   }
   if (h.nonfinite) {  // engine.rs:571-633: skip the whole micro-batch, touch nothing
     e->nan_gradient_count += 1;
@@ -204,6 +282,34 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
   if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result->scale;
   const int32_t N = acc_steps(e);
+
+  if (e->cfg.defer_accumulation) {
+    // Nothing is accumulated: the micro-batch is only remembered.  At the end of the cycle one pass
+    // over p and the held gradients forms sum_j clip_j(clamp(g_j)) in registers and applies lr/N.
+    if ((rc = defer_record(e, idx, grads))) return rc;
+    e->have_acc = true;
+    e->micro_step += 1;
+    int applied = 0;
+    if (e->micro_step >= N) {
+      if (!e->held_slots.empty()) {
+        mxopt_table* t = nullptr;
+        if ((rc = defer_table(e, &t))) return rc;
+        const float* scales[MXOPT_MAX_PENDING + 1] = {nullptr, nullptr, nullptr, nullptr};
+        if (e->cfg.has_gradient_clip_norm)
+          for (size_t j = 0; j < e->held.size(); ++j) scales[j] = &e->d_result[j].scale;
+        prep.d_scale = nullptr;
+        rc = mxopt_sgd_plain_with_pending_list_each(ctx, t, e->cfg.learning_rate / (double)N, 0.0, &prep, scales);
+        (void)mxopt_table_set_pending(t, 0, nullptr, 0);
+        if (rc) return rc;
+      }
+      end_cycle(e);
+      applied = 1;
+    }
+    e->step += 1;
+    fill_metrics(e, out, applied, 0);
+    if (n) add_norm(out, h);
+    return MXOPT_OK;
+  }
 
   if (e->micro_step + 1 >= N && e->cfg.apply == MXOPT_ENGINE_APPLY_SGD) {
     // Last micro-batch of the cycle: p -= (lr/N) * (acc + clip(clamp(g))) in one pass over p, acc and
@@ -341,11 +447,79 @@ int sft_apply(mxopt_engine* e, int32_t count, bool norm_ready, mxopt_engine_metr
   return MXOPT_OK;
 }
 
+// The boundary of sft_apply over held micro-batches: average by `count`, clip by the norm of the
+// averaged sum, clamp, decay, update -- the sum itself is formed in registers by both passes.
+int sft_apply_deferred(mxopt_engine* e, int32_t count, mxopt_engine_metrics* out, mxopt_norm_result* h_out,
+                       bool* measured) {
+  mxopt_ctx* ctx = e->ctx;
+  *measured = false;
+  int rc = MXOPT_OK;
+  if (!e->held_slots.empty()) {
+    mxopt_grad_prep prep = no_prep();
+    prep.has_pre_mul = 1;
+    prep.pre_mul = (float)(1.0 / (double)count);  // mul_scalar(scale): float64, then one cast
+    if (e->cfg.has_gradient_clip_value) {
+      prep.has_clamp_post = 1;
+      prep.post_lo = (float)(-e->cfg.gradient_clip_value);
+      prep.post_hi = (float)e->cfg.gradient_clip_value;
+    }
+    const bool clip = e->cfg.has_gradient_clip_norm != 0;
+    if (e->cfg.apply == MXOPT_ENGINE_APPLY_ADAMW) {
+      const size_t n = e->held_slots.size(), k = e->held.size();
+      std::vector<const char*> names(n);
+      std::vector<mxopt_array> params(n), grads(k * n);
+      for (size_t c = 0; c < n; ++c) {
+        const Slot& s = e->slots[e->held_slots[c]];
+        names[c] = s.name.c_str();
+        params[c] = s.param;
+        for (size_t j = 0; j < k; ++j) grads[j * n + c] = e->held[j][c];
+      }
+      rc = mxopt_optimizer_update_many_accumulated(e->adamw, n, names.data(), params.data(), k, grads.data(),
+                                                   params.data(), &prep, clip ? e->cfg.gradient_clip_norm : -1.0,
+                                                   MXOPT_CLIP_ALWAYS_MULTIPLY, e->d_result);
+    } else {
+      mxopt_table* t = nullptr;
+      if ((rc = defer_table(e, &t))) return rc;
+      if (clip) {
+        rc = mxopt_norm_with_pending_list(ctx, t, &prep, e->cfg.gradient_clip_norm, MXOPT_CLIP_ALWAYS_MULTIPLY,
+                                          e->d_result);
+        prep.d_scale = &e->d_result->scale;
+      }
+      if (!rc) rc = mxopt_sgd_plain_with_pending_list(ctx, t, e->cfg.learning_rate, e->cfg.weight_decay, &prep);
+      (void)mxopt_table_set_pending(t, 0, nullptr, 0);
+    }
+    if (rc) return rc;
+    if (clip && out) {
+      if ((rc = mxopt_read_norm_result(ctx, e->d_result, h_out))) return rc;
+      *measured = true;
+    }
+  }
+  end_cycle(e);
+  e->step += 1;
+  return MXOPT_OK;
+}
+
 int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_array* grads,
                     mxopt_engine_metrics* out) {
   mxopt_ctx* ctx = e->ctx;
   const size_t n = idx.size();
   e->consecutive_nan_count = 0;  // sft/engine.rs:261-267
+  if (e->cfg.defer_accumulation) {
+    int rc = defer_record(e, idx, grads);
+    if (rc) return rc;
+    e->have_acc = true;
+    e->micro_step += 1;
+    int applied = 0;
+    mxopt_norm_result h;
+    bool measured = false;
+    if (e->micro_step >= acc_steps(e)) {
+      if ((rc = sft_apply_deferred(e, acc_steps(e), out, &h, &measured))) return rc;
+      applied = 1;
+    }
+    fill_metrics(e, out, applied, 0);
+    if (measured) add_norm(out, h);
+    return MXOPT_OK;
+  }
   const bool first_cycle_step = !e->have_acc;
   if (first_cycle_step)
     for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
@@ -506,6 +680,16 @@ int mxopt_engine_new(mxopt_ctx* ctx, const mxopt_engine_config* config, size_t n
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: unknown engine kind");
   if (config->apply != MXOPT_ENGINE_APPLY_SGD && config->apply != MXOPT_ENGINE_APPLY_ADAMW)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: unknown apply mode");
+  if (config->defer_accumulation) {
+    if (config->gradient_accumulation_steps > MXOPT_MAX_PENDING + 1)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  "mxopt_engine_new: defer_accumulation holds at most " + std::to_string(MXOPT_MAX_PENDING + 1) +
+                      " micro-batches");
+    if (config->kind == MXOPT_ENGINE_SFT && !config->accumulate_in_f32)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: defer_accumulation adds in float32 (set accumulate_in_f32)");
+    if (config->kind == MXOPT_ENGINE_GRPO && config->apply != MXOPT_ENGINE_APPLY_SGD)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: defer_accumulation in the GRPO engine applies plain SGD only");
+  }
   mxopt_engine* e = new (std::nothrow) mxopt_engine();
   if (!e) return fail(ctx, MXOPT_ERR_OOM, "mxopt_engine_new: out of host memory");
   e->ctx = ctx;
@@ -526,7 +710,8 @@ int mxopt_engine_new(mxopt_ctx* ctx, const mxopt_engine_config* config, size_t n
   int rc = MXOPT_OK;
   {
     DeviceGuard guard(ctx->device);
-    hipError_t err = hipMalloc((void**)&e->d_result, sizeof(mxopt_norm_result));
+    // one slot per micro-batch a deferred cycle can hold; slot 0 serves everything else
+    hipError_t err = hipMalloc((void**)&e->d_result, (MXOPT_MAX_PENDING + 1) * sizeof(mxopt_norm_result));
     if (err != hipSuccess) rc = hip_fail(ctx, err, "mxopt_engine_new: hipMalloc");
   }
   if (!rc && config->apply == MXOPT_ENGINE_APPLY_ADAMW) {
@@ -573,7 +758,8 @@ int mxopt_engine_flush_gradients(mxopt_engine* e, int* flushed, mxopt_engine_met
   }
   mxopt_norm_result h;
   bool measured = false;
-  int rc = sft_apply(e, e->micro_step, false, out, &h, &measured);
+  int rc = e->cfg.defer_accumulation ? sft_apply_deferred(e, e->micro_step, out, &h, &measured)
+                                     : sft_apply(e, e->micro_step, false, out, &h, &measured);
   if (rc) return rc;
   if (flushed) *flushed = 1;
   fill_metrics(e, out, 1, 0);
@@ -609,6 +795,8 @@ int mxopt_engine_reset(mxopt_engine* e) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_reset: null engine");
   for (Slot& s : e->slots) s.in_acc = false;
   e->have_acc = false;
+  e->held.clear();
+  e->held_slots.clear();
   e->micro_step = 0;
   e->step = 0;
   e->nan_gradient_count = 0;

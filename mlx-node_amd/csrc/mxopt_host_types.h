@@ -43,11 +43,18 @@ struct DevChunk {
 
 constexpr uint32_t kPrepPreMul = 1u, kPrepClampPre = 2u, kPrepClampPost = 4u;
 constexpr uint32_t kPrepPendingOnly = 8u;  // update kernels with a pending gradient: g + prep(g2), not prep(g + g2)
+constexpr uint32_t kPrepEachStream = 16u;  // list kernels: prep every stream (own clip factor), then add
 struct DevPrep {  // kernel argument
   const float* d_scale;
   const unsigned long long* d_skip_if_nonzero;
   float pre_mul, pre_lo, pre_hi, post_lo, post_hi;
   uint32_t flags;
+};
+
+// Deferred accumulation with kPrepEachStream: the clip factor of tensor.g and of each pending stream
+// (device scalars; all NULL = no factor).
+struct StreamScales {
+  const float* s[MXOPT_MAX_PENDING + 1];
 };
 
 // Tensors of one dtype combination: a contiguous run of chunk entries, one launch.

@@ -515,13 +515,38 @@ template <int PD, int GD, int XD, class Math>
 __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* __restrict__ T,
                                                                const DevChunk* __restrict__ C, DevTensor one,
                                                                uint32_t nchunks, uint32_t ntensors,
-                                                               const void* const* __restrict__ X, int kx, Math math,
-                                                               DevPrep prep) {
+                                                               const void* const* __restrict__ X, int kx,
+                                                               StreamScales scales, Math math, DevPrep prep) {
   constexpr int E = (PD != MXOPT_F32 || GD != MXOPT_F32 || XD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
   if (skip_requested(prep)) return;
   const PrepRegs pr = load_prep(prep);
   const uint32_t tid = threadIdx.x;
+  // Either prep(g + x0 + ...) or, with kPrepEachStream, prep_0(g) + prep_1(x0) + ...: every micro-batch
+  // clamped and scaled by its own clip factor before it is added (grpo/engine.rs:636-661).
+  const bool each = (pr.flags & kPrepEachStream) != 0;
+  PrepRegs ps_regs[kMaxPending + 1];
+#pragma unroll
+  for (int j = 0; j <= kMaxPending; ++j) {
+    ps_regs[j] = pr;
+    const bool has = each && j <= kx && scales.s[j] != nullptr;
+    ps_regs[j].has_scale = has;
+    ps_regs[j].scale = has ? *scales.s[j] : 1.0f;
+  }
+  auto gradient = [&](float g, const float (&x)[kMaxPending]) {
+    if (!each) {
+      float s = g;
+#pragma unroll
+      for (int k = 0; k < kMaxPending; ++k)
+        if (k < kx) s = s + x[k];
+      return prep_all(pr, s);
+    }
+    float s = prep_all(ps_regs[0], g);
+#pragma unroll
+    for (int k = 0; k < kMaxPending; ++k)
+      if (k < kx) s = s + prep_all(ps_regs[k + 1], x[k]);
+    return s;
+  };
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
     const ChunkView cv = locate(T, C, one, c);
@@ -537,7 +562,10 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
     const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
     auto one_element = [&](uint64_t off) {
       float p = Elem<PD>::load(P, off);
-      const float ge = prep_all(pr, pending_sum_element<GD, XD>(G, ps, kx, off));
+      float xs[kMaxPending];
+#pragma unroll
+      for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? Elem<XD>::load(ps.x[k], off) : 0.0f;
+      const float ge = gradient(Elem<GD>::load(G, off), xs);
       float m = Math::kM ? M[off] : 0.0f;
       float v = read_v ? V[off] : 0.0f;
       math(p, ge, m, v, bc1, bc2, flags);
@@ -563,11 +591,10 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float s = g[j][e];
+          float xs[kMaxPending];
 #pragma unroll
-          for (int k = 0; k < kMaxPending; ++k)
-            if (k < kx) s = s + x[k][j][e];
-          math(p[j][e], prep_all(pr, s), m[j][e], v[j][e], bc1, bc2, flags);
+          for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? x[k][j][e] : 0.0f;
+          math(p[j][e], gradient(g[j][e], xs), m[j][e], v[j][e], bc1, bc2, flags);
         }
       }
 #pragma unroll
@@ -581,21 +608,21 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
       const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
       for (uint32_t q = tid; q < ngroups; q += kThreads) {
         const uint64_t off = start + (uint64_t)q * E;
-        float p[E], g[E], x[E], m[E], v[E];
+        float p[E], g[E], x[kMaxPending][E], m[E], v[E];
         load_group<PD, E, false>(P, off, p);
         load_group<GD, E, false>(G, off, g);
 #pragma unroll
-        for (int k = 0; k < kMaxPending; ++k) {
-          if (k < kx) {
-            load_group<XD, E, false>(ps.x[k], off, x);
-#pragma unroll
-            for (int e = 0; e < E; ++e) g[e] = g[e] + x[e];
-          }
-        }
+        for (int k = 0; k < kMaxPending; ++k)
+          if (k < kx) load_group<XD, E, false>(ps.x[k], off, x[k]);
         if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m);
         if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
 #pragma unroll
-        for (int e = 0; e < E; ++e) math(p[e], prep_all(pr, g[e]), m[e], v[e], bc1, bc2, flags);
+        for (int e = 0; e < E; ++e) {
+          float xs[kMaxPending];
+#pragma unroll
+          for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? x[k][e] : 0.0f;
+          math(p[e], gradient(g[e], xs), m[e], v[e], bc1, bc2, flags);
+        }
         store_group<PD, E, false>(PO, off, p);
         if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
         if (use_v) store_group<MXOPT_F32, E, false>(V, off, v);
@@ -909,6 +936,7 @@ bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep
 #define MXOPT_LAUNCH_LIST(kernel, L, ...)                                                                     \
   hipLaunchKernelGGL(kernel, dim3((L).grid), dim3(kThreads), 0, (L).stream, (L).tensors, (L).chunks, (L).one, \
                      (L).nchunks, (L).ntensors, (L).pending, (L).npending, __VA_ARGS__)
+#define MXOPT_LAUNCH_UPDATE_LIST(kernel, L, ...) MXOPT_LAUNCH_LIST(kernel, L, (L).scales, __VA_ARGS__)
 
 // g is either of the pending streams' dtype (the first micro-batch) or float32 (a buffer of earlier ones).
 template <int PD, class Math>
@@ -917,15 +945,15 @@ static bool update_list_for_pd(int gd, int xd, const Launch& L, const Math& math
   const bool same = gd == xd;
   switch (xd) {
     case MXOPT_F32:
-      MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F32, Math>), L, math, prep);
+      MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F32, Math>), L, math, prep);
       return true;
     case MXOPT_BF16:
-      if (same) MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_BF16, MXOPT_BF16, Math>), L, math, prep);
-      else MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_BF16, Math>), L, math, prep);
+      if (same) MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_BF16, MXOPT_BF16, Math>), L, math, prep);
+      else MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_BF16, Math>), L, math, prep);
       return true;
     case MXOPT_F16:
-      if (same) MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F16, MXOPT_F16, Math>), L, math, prep);
-      else MXOPT_LAUNCH_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F16, Math>), L, math, prep);
+      if (same) MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F16, MXOPT_F16, Math>), L, math, prep);
+      else MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F16, Math>), L, math, prep);
       return true;
   }
   return false;

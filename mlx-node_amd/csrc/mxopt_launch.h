@@ -24,6 +24,7 @@ struct Launch {
   const void* const* pending = nullptr;
   uint32_t ntensors = 0;
   int npending = 0;
+  StreamScales scales{};             // used when the prep carries kPrepEachStream
 };
 
 // Each returns false when the dtype combination has no kernel.

@@ -94,6 +94,8 @@ SIGNATURES = {
     "mxopt_adam_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_sgd_plain_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
                                                     C.POINTER(GradPrep)]),
+    "mxopt_sgd_plain_with_pending_list_each": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
+                                                         C.POINTER(GradPrep), C.POINTER(C.c_void_p)]),
     "mxopt_adam_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
     "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),
@@ -175,7 +177,7 @@ class EngineConfig(C.Structure):
                 ("weight_decay", C.c_double), ("max_nan_gradients", C.c_int64),
                 ("emergency_save_threshold", C.c_int32), ("apply", C.c_int32),
                 ("beta1", C.c_double), ("beta2", C.c_double), ("eps", C.c_double),
-                ("accumulate_in_f32", C.c_int32)]
+                ("accumulate_in_f32", C.c_int32), ("defer_accumulation", C.c_int32)]
 
 
 class EngineMetrics(C.Structure):

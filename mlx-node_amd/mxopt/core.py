@@ -240,6 +240,15 @@ def _sgd_plain_with_pending_list(self, table: "Table", learning_rate: float, wei
                                                        C.byref(prep) if prep else None), self.handle)
 
 
+def _sgd_plain_with_pending_list_each(self, table: "Table", learning_rate: float, scales: Sequence[Optional[int]],
+                                      weight_decay: float = 0.0, prep: Optional[L.GradPrep] = None) -> None:
+    """scales: one device address of a float per stream (tensor.g first), or None for all of them."""
+    arr = (C.c_void_p * max(len(scales), 1))(*scales)
+    L.check(self.lib.mxopt_sgd_plain_with_pending_list_each(self.handle, table.handle, learning_rate, weight_decay,
+                                                            C.byref(prep) if prep else None, arr), self.handle)
+
+
+Context.sgd_plain_with_pending_list_each = _sgd_plain_with_pending_list_each
 Context.accumulate_norm_only = _accumulate_norm_only
 Context.norm_with_pending_list = _norm_with_pending_list
 Context.adam_with_pending_list = _adam_with_pending_list

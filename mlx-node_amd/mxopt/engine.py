@@ -5,6 +5,8 @@ crates/mlx-core/src/grpo/engine.rs:561-704; SftTrainingEngine, crates/mlx-core/s
 Config keyword names and defaults are those of GRPOEngineConfig / SftEngineConfig (None = the
 reference's Option::None); getters are those of the engines (step, micro_step, nan_gradient_count,
 needs_emergency_save, clear_emergency_save_flag, reset).  Parameters are updated in place.
+With defer_accumulation=True the engine keeps no accumulation buffer: it remembers the gradient tensors
+of a cycle (this shim keeps them alive) and the applying call adds them in registers.
 """
 from __future__ import annotations
 
@@ -61,7 +63,10 @@ class _EngineOptimizerSide:
         for i, nm in enumerate(names):
             arrs[i] = _arr(gradients[nm])
         m = L.EngineMetrics()
+        held = getattr(self, "_held", [])
+        held.append(list(gradients.values()))    # deferred accumulation reads them when the cycle is applied
         self._check(self.lib.mxopt_engine_micro_batch(self.handle, len(names), cnames, arrs, C.byref(m)))
+        self._held = [] if m.gradients_applied or m.micro_step == 0 else held
         return m
 
     def metrics(self) -> L.EngineMetrics:
@@ -99,7 +104,8 @@ class _EngineOptimizerSide:
 
 
 def _config(kind, learning_rate, gradient_accumulation_steps, gradient_clip_norm, gradient_clip_value, weight_decay,
-            max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps, accumulate_in_f32) -> L.EngineConfig:
+            max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps, accumulate_in_f32,
+            defer_accumulation=False) -> L.EngineConfig:
     cfg = L.EngineConfig()
     L.load().mxopt_engine_config_default(kind, C.byref(cfg))
     if learning_rate is not None:
@@ -119,6 +125,7 @@ def _config(kind, learning_rate, gradient_accumulation_steps, gradient_clip_norm
     cfg.apply = {"sgd": L.ENGINE_APPLY_SGD, "adamw": L.ENGINE_APPLY_ADAMW}[apply]
     cfg.beta1, cfg.beta2, cfg.eps = beta1, beta2, eps
     cfg.accumulate_in_f32 = int(accumulate_in_f32)
+    cfg.defer_accumulation = int(defer_accumulation)
     return cfg
 
 
@@ -130,10 +137,11 @@ class GRPOEngineOptimizerSide(_EngineOptimizerSide):
                  gradient_clip_norm: Optional[float] = 1.0, gradient_clip_value: Optional[float] = None,
                  max_nan_gradients: Optional[int] = None, emergency_save_threshold: Optional[int] = None,
                  apply: str = "sgd", weight_decay: float = 0.01, beta1: float = 0.9, beta2: float = 0.999,
-                 eps: float = 1e-8, ctx: Optional[Context] = None):
+                 eps: float = 1e-8, defer_accumulation: bool = False, ctx: Optional[Context] = None):
         super().__init__(params, _config(L.ENGINE_GRPO, learning_rate, gradient_accumulation_steps, gradient_clip_norm,
                                          gradient_clip_value, weight_decay, max_nan_gradients,
-                                         emergency_save_threshold, apply, beta1, beta2, eps, True), ctx)
+                                         emergency_save_threshold, apply, beta1, beta2, eps, True,
+                                         defer_accumulation), ctx)
 
 
 class SFTEngineOptimizerSide(_EngineOptimizerSide):
@@ -144,11 +152,11 @@ class SFTEngineOptimizerSide(_EngineOptimizerSide):
                  weight_decay: Optional[float] = None, max_nan_gradients: Optional[int] = None,
                  emergency_save_threshold: Optional[int] = None, apply: str = "sgd", beta1: float = 0.9,
                  beta2: float = 0.999, eps: float = 1e-8, accumulate_in_f32: bool = False,
-                 ctx: Optional[Context] = None):
+                 defer_accumulation: bool = False, ctx: Optional[Context] = None):
         super().__init__(params, _config(L.ENGINE_SFT, learning_rate, gradient_accumulation_steps, gradient_clip_norm,
                                          gradient_clip_value, 0.0 if weight_decay is None else weight_decay,
                                          max_nan_gradients, emergency_save_threshold, apply, beta1, beta2, eps,
-                                         accumulate_in_f32), ctx)
+                                         accumulate_in_f32, defer_accumulation), ctx)
 
     def flush_gradients(self) -> bool:
         flushed = C.c_int()

@@ -61,7 +61,7 @@ int main(void) {
   S(mxopt_rmsprop_hp); F(mxopt_rmsprop_hp, has_weight_decay);
   S(mxopt_array); F(mxopt_array, dtype);
   S(mxopt_engine_config); F(mxopt_engine_config, gradient_clip_norm); F(mxopt_engine_config, max_nan_gradients);
-  F(mxopt_engine_config, apply); F(mxopt_engine_config, eps); F(mxopt_engine_config, accumulate_in_f32);
+  F(mxopt_engine_config, apply); F(mxopt_engine_config, eps); F(mxopt_engine_config, accumulate_in_f32); F(mxopt_engine_config, defer_accumulation);
   S(mxopt_engine_metrics); F(mxopt_engine_metrics, nan_gradient_count); F(mxopt_engine_metrics, clip_scale);
   F(mxopt_engine_metrics, grad_norm);
   return 0;

@@ -205,3 +205,92 @@ def test_one_micro_batch_per_step(mx, kind, apply, bf16):
         assert m.gradients_applied and m.norm_measured and m.clip_scale < 1.0
         ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
         check_state(dev, ref, dparams, f"{kind} step {it}")
+
+
+# ---------------------------------------------------------------------------------------
+# defer_accumulation: no accumulation buffer, the micro-batches of a cycle are added in registers by
+# the applying call.  The oracle is the unchanged (buffered) engine: every number must be the same.
+# ---------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("n_acc", [1, 3, 4])
+def test_grpo_deferred_sequence(mx, bf16, n_acc):
+    rng = np.random.default_rng(107 + n_acc)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=2.0, gradient_clip_value=0.02,
+              max_nan_gradients=50, emergency_save_threshold=2)
+    dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
+    ref = O.GRPOEngineOptimizerSide(params, **kw)
+    script = ["ok", "ok", "nan", "inf", "ok", "ok", "-inf", "ok", "ok", "ok", "ok", "ok", "ok"]
+    for it, kind in enumerate(script):
+        grads = make_grads(rng, bf16, 0.01 * (1 + it % 3))
+        if kind != "ok":
+            v = O.as_f32(grads["w1"]).copy()
+            v[4096 + 5] = {"nan": np.nan, "inf": np.inf, "-inf": -np.inf}[kind]
+            grads["w1"] = O.f32_to_bf16(v) if bf16 else v
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        if kind == "ok":
+            exact = exact_clamped_sumsq(grads, 0.02)
+            assert m.norm_measured and abs(m.grad_norm - math.sqrt(exact)) <= 1e-5 * math.sqrt(exact)
+            r = ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
+        else:
+            r = ref.micro_batch(grads)
+        assert (bool(m.skipped), bool(m.gradients_applied), m.step) == (r["skipped"], r["gradients_applied"], r["step"])
+        if m.gradients_applied or n_acc == 1:
+            check_state(dev, ref, dparams, f"micro-batch {it} ({kind})")
+        else:   # inside a cycle the parameters have not moved on either side; the counters must agree
+            st, mm = ref.state, dev.metrics()
+            assert (mm.step, mm.micro_step, mm.nan_gradient_count) == (st.step, st.micro_step, st.nan_gradient_count)
+    dev.reset()
+    ref.reset()
+    check_state(dev, ref, dparams, "after reset")
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("apply", ["sgd", "adamw"])
+def test_sft_deferred_sequence(mx, bf16, apply):
+    rng = np.random.default_rng(123)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.02, gradient_accumulation_steps=3, gradient_clip_norm=0.5, gradient_clip_value=0.002,
+              weight_decay=0.01, apply=apply)
+    dev = mx.SFTEngineOptimizerSide(dparams, accumulate_in_f32=True, defer_accumulation=True, **kw)
+    ref = O.SFTEngineOptimizerSide(params, **kw)
+    for it in range(8):                                     # two full cycles + two leftover micro-batches
+        grads = make_grads(rng, bf16, 0.01)
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        wide = {k: O.as_f32(g) for k, g in grads.items()}    # a float32 sum = float32 gradients to the oracle
+        boundary = ref.state.micro_step + 1 >= 3
+        r = ref.micro_batch(wide, norm_sumsq=m.grad_sumsq) if boundary else ref.micro_batch(wide)
+        assert bool(m.norm_measured) == boundary
+        assert (bool(m.gradients_applied), m.step) == (r["gradients_applied"], r["step"])
+        check_state(dev, ref, dparams, f"micro-batch {it}")
+    assert ref.state.micro_step == 2
+    assert dev.flush_gradients() is True
+    assert ref.flush_gradients(norm_sumsq=dev.last_metrics.grad_sumsq) is True
+    check_state(dev, ref, dparams, "after flush")
+    assert dev.flush_gradients() is False and ref.flush_gradients() is False
+
+
+def test_deferred_mode_refuses_what_it_cannot_hold(mx):
+    rng = np.random.default_rng(5)
+    params = make_params(rng, False)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    with pytest.raises(ValueError, match="at most 4 micro-batches"):
+        mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=5, accumulate_in_f32=True, defer_accumulation=True)
+    with pytest.raises(ValueError, match="adds in float32"):
+        mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=2, defer_accumulation=True)
+    with pytest.raises(ValueError, match="plain SGD only"):
+        mx.GRPOEngineOptimizerSide(dparams, gradient_accumulation_steps=2, apply="adamw", defer_accumulation=True)
+    dev = mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=2, accumulate_in_f32=True, defer_accumulation=True)
+    dev.micro_batch({k: to_dev(g) for k, g in make_grads(rng, False, 0.01).items()})
+    before = {k: to_host(v) for k, v in dparams.items()}
+    with pytest.raises(ValueError, match="same gradient names"):
+        dev.micro_batch({k: to_dev(g) for k, g in make_grads(rng, False, 0.01, ["embed", "w1"]).items()})
+    assert dev.micro_step == 1
+    for k in dparams:
+        assert_bit_equal(to_host(dparams[k]), before[k], k)
+    # the cycle is still open: the complete micro-batch finishes it
+    m = dev.micro_batch({k: to_dev(g) for k, g in make_grads(rng, False, 0.01).items()})
+    assert m.gradients_applied and dev.micro_step == 0
