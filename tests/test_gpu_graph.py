@@ -72,3 +72,59 @@ def test_clip_and_adamw_step_replays_from_a_graph():
     for t in (t_g, t_upd):
         t.close()
     ctx.close()
+
+
+def test_deferred_accumulation_step_replays_from_a_graph():
+    """norm over three un-summed micro-batches + AdamW on their sum, captured once; the pending pointers
+    were uploaded before the capture (mxopt_table_set_pending copies from host memory)."""
+    import torch
+    import mxopt as mx
+    rng = np.random.default_rng(321)
+    ps = [O.f32_to_bf16(rng.normal(0, 0.02, n).astype(F)) for n in SIZES]
+    stream = torch.cuda.Stream()
+    ctx = mx.Context(stream=stream)
+    dp = [to_dev(p) for p in ps]
+    dmicro = [[torch.zeros(n, dtype=torch.bfloat16, device="cuda") for n in SIZES] for _ in range(3)]
+    dm = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in SIZES]
+    dv = [torch.zeros(n, dtype=torch.float32, device="cuda") for n in SIZES]
+    res = ctx.norm_result()
+    table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dmicro[0], dm, dv)])
+    table.set_pending(dmicro[1:])
+    hp = mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    prep = mx.make_prep(scale=res, skip_if_nonfinite=res)
+    ctx.norm_with_pending_list(table, res, max_norm=1e-2)     # warm-up: sizes the partials buffer
+    ctx.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        ctx.norm_with_pending_list(table, res, max_norm=1e-2)
+        ctx.adam_with_pending_list(table, hp, prep)
+    torch.cuda.synchronize()
+
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    cur = list(ps)
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for it in range(4):
+        micro = [[O.f32_to_bf16(rng.normal(0, 1e-3 * (it + 1), n).astype(F)) for n in SIZES] for _ in range(3)]
+        if it == 1:
+            micro[2][4][1234] = 0x7F80                # +Inf in the last micro-batch: nothing may change
+        for dst, src in zip(dmicro, micro):
+            for d, g in zip(dst, src):
+                d.copy_(to_dev(g))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        r = ctx.read_norm_result(res)
+        if it == 1:
+            assert r.nonfinite == 1
+        else:
+            acc = [O.accumulate_fp32(O.accumulate_fp32(O.accumulate_fp32(None, a), b), c) for a, b, c in zip(*micro)]
+            n32, _ = O.norm_scale_c1(O.exact_sumsq(acc), 1e-2)
+            assert r.nonfinite == 0 and abs(r.norm - float(n32)) <= 1e-5 * float(n32)
+            for i in range(len(SIZES)):
+                cur[i] = O.f32_to_bf16(ref.update_single(str(i), cur[i], acc[i] * F(r.scale)))
+        for i in range(len(SIZES)):
+            assert_bit_equal(to_host(dp[i]), cur[i], f"p{i} replay {it}")
+        scratch.add_(1.0)
+        torch.cuda.synchronize()
+    table.close()
+    ctx.close()
