@@ -17,6 +17,7 @@ bounded sample of the same workload and scales it to the full parameter list.
 from __future__ import annotations
 
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -50,6 +51,9 @@ def parse_args():
     ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab", "packed"],
                     help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
                          "tensors are 512-byte aligned views into it")
+    ap.add_argument("--placement", default="spread", choices=["spread", "plain"],
+                    help="spread: the buffers are allocated inside mxopt_hbm_spread_begin/end (their physical pages "
+                         "interleaved with released memory); plain: wherever the driver puts them")
     ap.add_argument("--defer", type=int, default=0,
                     help="engine workloads: 1 = defer_accumulation (four resident micro-batches, no accumulation "
                          "buffer, summed in registers by the applying call)")
@@ -96,8 +100,9 @@ class Workload:
         self.n = int(sum(self.sizes))
         self.kernel_events = {}     # kernel name -> list of (start, end) events
         self.res = self.ctx.norm_result()
-        getattr(self, "_setup_" + args.workload.replace("-", "_"))()
-        torch.cuda.synchronize()
+        with (self.ctx.hbm_spread() if args.placement == "spread" else contextlib.nullcontext()):
+            getattr(self, "_setup_" + args.workload.replace("-", "_"))()
+            torch.cuda.synchronize()
 
     # -- helpers
     SEED = 0x5EED0001
@@ -585,7 +590,9 @@ def main():
         "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
                    "bytes_per_elem_per_step": wl.step_bytes_per_elem,
                    "storage": getattr(wl, "storage", "float32 everywhere"), "note": wl.note, "scale": args.scale,
-                   "alloc": args.alloc},
+                   "alloc": args.alloc,
+                   "placement": ("buffers allocated between mxopt_hbm_spread_begin and _end (64 MiB blocks, every "
+                                 "third kept meanwhile)" if args.placement == "spread" else "plain")},
         "elements_per_s": round(n * steps_per_s, 1),
         "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "kernels": kernels,

@@ -313,6 +313,58 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
   return MXOPT_OK;
 }
 
+// ---- HBM placement --------------------------------------------------------------------
+
+struct mxopt_hbm_spread {
+  mxopt_ctx* ctx = nullptr;
+  std::vector<void*> kept;
+};
+
+int mxopt_hbm_spread_begin(mxopt_ctx* ctx, size_t block_bytes, int keep_one_in, mxopt_hbm_spread** out) {
+  if (!ctx || !out) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_spread_begin: null argument");
+  *out = nullptr;
+  if (block_bytes == 0) block_bytes = (size_t)64 << 20;
+  if (keep_one_in == 0) keep_one_in = 3;
+  if (block_bytes < ((size_t)2 << 20) || keep_one_in < 2)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_spread_begin: blocks of at least 2 MiB, keep_one_in >= 2");
+  DeviceGuard guard(ctx->device);
+  size_t free_b = 0, total_b = 0;
+  HIP_TRY(ctx, hipMemGetInfo(&free_b, &total_b));
+  const size_t margin = (size_t)1 << 30;  // left to the runtime's own needs
+  const size_t count = free_b > margin ? (free_b - margin) / block_bytes : 0;
+  if (count > 60000)  // the driver limits the number of live allocations of a process
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_spread_begin: block size too small for this much free memory");
+  mxopt_hbm_spread* s = new (std::nothrow) mxopt_hbm_spread();
+  if (!s) return fail(ctx, MXOPT_ERR_OOM, "mxopt_hbm_spread_begin: out of host memory");
+  s->ctx = ctx;
+  std::vector<void*> all;
+  all.reserve(count);
+  for (size_t i = 0; i < count; ++i) {
+    void* p = nullptr;
+    if (hipMalloc(&p, block_bytes) != hipSuccess) {
+      (void)hipGetLastError();  // running out early is fine: what was obtained is spread
+      break;
+    }
+    all.push_back(p);
+  }
+  for (size_t i = 0; i < all.size(); ++i) {
+    if (i % (size_t)keep_one_in == 0) s->kept.push_back(all[i]);
+    else (void)hipFree(all[i]);
+  }
+  *out = s;
+  return MXOPT_OK;
+}
+
+int mxopt_hbm_spread_end(mxopt_hbm_spread* s) {
+  if (!s) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_spread_end: null argument");
+  {
+    DeviceGuard guard(s->ctx->device);
+    for (void* p : s->kept) (void)hipFree(p);
+  }
+  delete s;
+  return MXOPT_OK;
+}
+
 // ---- tables ---------------------------------------------------------------------------
 
 int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxopt_table** out) {

@@ -88,6 +88,8 @@ SIGNATURES = {
     "mxopt_sgd_hp_from_f64": (C.c_int, [C.c_double, C.c_double, C.c_double, C.c_double, C.c_int, C.POINTER(SgdHp)]),
     "mxopt_rmsprop_hp_from_f64": (None, [C.c_double, C.c_double, C.c_double, C.c_double, C.POINTER(RmspropHp)]),
     "mxopt_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_hbm_spread_begin": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
+    "mxopt_hbm_spread_end": (C.c_int, [C.c_void_p]),
     "mxopt_table_set_pending": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.c_int]),
     "mxopt_norm_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
                                                C.c_void_p]),

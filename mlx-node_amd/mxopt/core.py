@@ -249,6 +249,31 @@ def _sgd_plain_with_pending_list_each(self, table: "Table", learning_rate: float
 
 
 Context.sgd_plain_with_pending_list_each = _sgd_plain_with_pending_list_each
+class _HbmSpread:
+    """with ctx.hbm_spread(): allocate the long-lived buffers here (see mxopt_hbm_spread_begin)."""
+
+    def __init__(self, ctx: "Context", block_bytes: int, keep_one_in: int):
+        self.ctx, self.block_bytes, self.keep_one_in = ctx, block_bytes, keep_one_in
+        self.handle = C.c_void_p()
+
+    def __enter__(self):
+        torch.cuda.empty_cache()     # what torch caches is not free memory to the driver
+        L.check(self.ctx.lib.mxopt_hbm_spread_begin(self.ctx.handle, self.block_bytes, self.keep_one_in,
+                                                    C.byref(self.handle)), self.ctx.handle)
+        return self
+
+    def __exit__(self, *exc):
+        if self.handle:
+            L.check(self.ctx.lib.mxopt_hbm_spread_end(self.handle), self.ctx.handle)
+            self.handle = C.c_void_p()
+        return False
+
+
+def _hbm_spread(self, block_bytes: int = 0, keep_one_in: int = 0) -> _HbmSpread:
+    return _HbmSpread(self, block_bytes, keep_one_in)
+
+
+Context.hbm_spread = _hbm_spread
 Context.accumulate_norm_only = _accumulate_norm_only
 Context.norm_with_pending_list = _norm_with_pending_list
 Context.adam_with_pending_list = _adam_with_pending_list
