@@ -172,7 +172,7 @@ class Workload:
         need = self.n * (2 + 8 + 4)
         free, _ = t.cuda.mem_get_info()
         self.n_micro = 4
-        n_gbuf = 4 if free > need + 4 * self.n * 2 + (8 << 30) else 1
+        n_gbuf = 4 if free > need + 4 * self.n * 2 + (3 << 30) else 1
         self.p = self._randn_list(bf, 0.02)
         self.m = self._zeros_list()
         self.v = self._zeros_list()
