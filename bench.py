@@ -54,6 +54,8 @@ def parse_args():
     ap.add_argument("--placement", default="spread", choices=["spread", "plain"],
                     help="spread: the buffers are allocated inside mxopt_hbm_spread_begin/end (their physical pages "
                          "interleaved with released memory); plain: wherever the driver puts them")
+    ap.add_argument("--spread-block-mb", type=int, default=0, help="--placement spread: block size (0 = the library's 64)")
+    ap.add_argument("--spread-keep", type=int, default=0, help="--placement spread: every n-th block is kept (0 = 3)")
     ap.add_argument("--defer", type=int, default=0,
                     help="engine workloads: 1 = defer_accumulation (four resident micro-batches, no accumulation "
                          "buffer, summed in registers by the applying call)")
@@ -100,7 +102,8 @@ class Workload:
         self.n = int(sum(self.sizes))
         self.kernel_events = {}     # kernel name -> list of (start, end) events
         self.res = self.ctx.norm_result()
-        with (self.ctx.hbm_spread() if args.placement == "spread" else contextlib.nullcontext()):
+        with (self.ctx.hbm_spread(args.spread_block_mb << 20, args.spread_keep) if args.placement == "spread"
+              else contextlib.nullcontext()):
             getattr(self, "_setup_" + args.workload.replace("-", "_"))()
             torch.cuda.synchronize()
 
@@ -591,8 +594,9 @@ def main():
                    "bytes_per_elem_per_step": wl.step_bytes_per_elem,
                    "storage": getattr(wl, "storage", "float32 everywhere"), "note": wl.note, "scale": args.scale,
                    "alloc": args.alloc,
-                   "placement": ("buffers allocated between mxopt_hbm_spread_begin and _end (64 MiB blocks, every "
-                                 "third kept meanwhile)" if args.placement == "spread" else "plain")},
+                   "placement": (f"buffers allocated between mxopt_hbm_spread_begin and _end "
+                                 f"({args.spread_block_mb or 64} MiB blocks, one in {args.spread_keep or 3} kept meanwhile)"
+                                 if args.placement == "spread" else "plain")},
         "elements_per_s": round(n * steps_per_s, 1),
         "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
         "kernels": kernels,

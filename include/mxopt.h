@@ -83,6 +83,8 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
  *   mxopt_hbm_spread_end(s);                   fills those gaps; end() releases the rest
  *
  * block_bytes = 0: 64 MiB; keep_one_in = 0: every third block is kept (>= 2: every keep_one_in-th).
+ * The defaults suit buffer sets of tens of GB (Qwen3-1.7B ... 8B lists); the 0.6B list wanted 256 MiB
+ * blocks, so a host with unusual sizes should time one step per candidate.
  * Between the two calls about (1 - 1/keep_one_in) of the free memory can be allocated.  Both calls
  * synchronise with the device and are meant for start-up, not for the training loop.  No counterpart
  * in the reference. */
