@@ -43,7 +43,7 @@ def assert_bit_equal(got: np.ndarray, want: np.ndarray, what: str = "") -> None:
     if np.array_equal(gb, wb):
         return
     # NaNs may differ in payload only
-    if got.dtype == np.float32:
+    if got.dtype in (np.float32, np.float16):
         both_nan = np.isnan(got) & np.isnan(want)
     else:
         both_nan = ((gb & 0x7FFF) > 0x7F80) & ((wb & 0x7FFF) > 0x7F80)

@@ -269,3 +269,124 @@ def test_host_layer_utilities_match_the_oracle(mx, sizes, bf16, max_norm, clip_v
     want_p = O.apply_gradients(ps, acc_o, lr)
     for k in names:
         assert_bit_equal(to_host(dp[k]), want_p[k], f"applied {k}")
+
+
+@settings(max_examples=150, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@given(sizes=st.lists(SIZES, min_size=1, max_size=4), k=st.integers(0, 3), head=st.sampled_from([0, 1, 2, 3, "mixed"]),
+       pd=st.sampled_from(DTYPES), xd=st.sampled_from(DTYPES), first_f32=st.booleans(),
+       kind=st.sampled_from(["adamw", "sgd_plain", "sgd_plain_each"]), pre_mul=st.sampled_from([None, 0.5]),
+       clamp_pre=st.sampled_from([None, 1.5e-3]), clip=st.booleans(), clamp_post=st.sampled_from([None, 4e-4]),
+       poison=st.sampled_from([None, "nan", "inf"]), seed=st.integers(0, 2 ** 31))
+def test_deferred_accumulation_kernels_match_the_oracle(mx, sizes, k, head, pd, xd, first_f32, kind, pre_mul, clamp_pre,
+                                                        clip, clamp_post, poison, seed):
+    """g + x0 + ... summed in registers.  "adamw" / "sgd_plain": prep(sum) with the clip factor of the
+    sum's norm; "sgd_plain_each": every stream clamped and clipped by its own norm before the add (the
+    GRPO order).  The oracle accumulates into a float32 buffer, micro-batch by micro-batch.  head = h:
+    every buffer becomes 16-byte aligned after h elements (vector path behind a peeled head); "mixed":
+    every buffer starts one element in, so 16-bit and float32 streams disagree (element-wise path)."""
+    import torch
+    rng = np.random.default_rng(seed)
+    ctx = mx.default_context()
+    gd = "f32" if first_f32 else xd
+    if head == "mixed":
+        shift = {"f32": 1, "bf16": 1, "f16": 1}
+    else:
+        shift = {"f32": (4 - head) % 4, "bf16": (8 - head) % 8, "f16": (8 - head) % 8}
+    ps = [cast(rng.normal(0, 0.05, n).astype(F), pd) for n in sizes]
+    streams = [[cast(rng.normal(0, 1e-3, n).astype(F), gd if j == 0 else xd) for n in sizes] for j in range(k + 1)]
+    if poison and sum(sizes):
+        j = int(rng.integers(0, k + 1))
+        i = int(rng.choice([t for t, n in enumerate(sizes) if n]))
+        a = O.as_f32(streams[j][i]).copy()
+        a[int(rng.integers(0, sizes[i]))] = np.nan if poison == "nan" else np.inf
+        with np.errstate(over="ignore"):
+            streams[j][i] = cast(a, gd if j == 0 else xd)
+    dp = [to_dev(p, shift[pd]) for p in ps]
+    dstreams = [[to_dev(g, shift[gd if j == 0 else xd]) for g in s] for j, s in enumerate(streams)]
+    dm = [to_dev(np.zeros(n, F), shift["f32"]) for n in sizes]
+    dv = [to_dev(np.zeros(n, F), shift["f32"]) for n in sizes]
+    adam = kind == "adamw"
+    rows = [mx.TensorSpec(p=p, p_out=p, g=g, m=m if adam else None, v=v if adam else None)
+            for p, g, m, v in zip(dp, dstreams[0], dm, dv)]
+    table = ctx.table(rows)
+    if head == "mixed" and pd == gd == "f32" and xd != "f32" and k and sum(sizes):
+        # the row's own buffers agree (all float32, head 3), a 16-bit pending stream one element in does not
+        with pytest.raises(mx.InvalidArg, match="16-byte phase"):
+            table.set_pending(dstreams[1:])
+        table.close()
+        return
+    table.set_pending(dstreams[1:])
+    max_norm = 1e-2
+    lr, wd = 0.05, 0.01
+
+    if kind == "sgd_plain_each":
+        # one norm per stream, of the clamped values (grpo/engine.rs:636-653)
+        results, scales, bad = [], [], False
+        for j in range(k + 1):
+            res = ctx.norm_result()
+            tj = ctx.table([mx.TensorSpec(g=g) for g in dstreams[j]])
+            ctx.global_norm(tj, res, prep=mx.make_prep(clamp_pre=(-clamp_pre, clamp_pre)) if clamp_pre else None,
+                            max_norm=max_norm)
+            r = ctx.read_norm_result(res)
+            bad = bad or bool(r.nonfinite)
+            results.append(res)
+            scales.append(F(r.scale))
+            tj.close()
+        if bad:
+            table.close()
+            return          # the engine drops such a micro-batch before anything is added
+        prep = mx.make_prep(clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None)
+        ptrs = [r.scale_ptr for r in results] if clip else [None] * (k + 1)
+        ctx.sgd_plain_with_pending_list_each(table, lr, ptrs, prep=prep)
+        want_g = []
+        for i in range(len(sizes)):
+            total = None
+            for j in range(k + 1):
+                t = prep_oracle(streams[j][i], None, clamp_pre, scales[j] if clip else None, None)[1]
+                total = t if total is None else total + t
+            want_g.append(total)
+    else:
+        res = ctx.norm_result()
+        pre = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None)
+        if clip:
+            ctx.norm_with_pending_list(table, res, prep=pre, max_norm=max_norm)
+        r = ctx.read_norm_result(res)
+        acc = [O.accumulate_fp32(None, g) for g in streams[0]]
+        for s in streams[1:]:
+            acc = [O.accumulate_fp32(a, g) for a, g in zip(acc, s)]
+        if clip:
+            with np.errstate(invalid="ignore", over="ignore"):
+                pre_vals = [prep_oracle(a, pre_mul, clamp_pre, None, None)[0] for a in acc]
+                finite = all(np.isfinite(a).all() for a in acc)
+            assert bool(r.nonfinite) == (not finite)
+            if not finite:
+                table.close()
+                return      # the caller skips the step; what a NaN clip factor does to p is not specified
+            exact = O.exact_sumsq(pre_vals)
+            assert abs(r.sumsq - exact) <= 1e-5 * max(exact, 1e-300)
+        scale = F(r.scale) if clip else None
+        prep = mx.make_prep(pre_mul=pre_mul, clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None,
+                            scale=res if clip else None, clamp_post=(-clamp_post, clamp_post) if clamp_post else None)
+        if adam:
+            ctx.adam_with_pending_list(table, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.02), prep)
+        else:
+            ctx.sgd_plain_with_pending_list(table, lr, wd, prep)
+        with np.errstate(invalid="ignore", over="ignore"):
+            want_g = [prep_oracle(a, pre_mul, clamp_pre, scale, clamp_post)[1] for a in acc]
+
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.02)
+    for i, n in enumerate(sizes):
+        p32 = O.as_f32(ps[i])
+        with np.errstate(invalid="ignore", over="ignore"):
+            if adam:
+                want = ref.update_single(str(i), ps[i], want_g[i])
+            else:
+                g = want_g[i] + (F(wd) * p32 if kind == "sgd_plain" else 0)
+                lr_eff = lr
+                lr_p = O.as_f32(cast(np.array([lr_eff], F), pd))[0]
+                want = p32 - lr_p * g
+            assert_bit_equal(to_host(dp[i]), round_out(want, pd), f"p {i} (n={n})")
+        if adam:
+            assert_bit_equal(to_host(dm[i]), ref.state[str(i)][0], f"m {i}")
+            assert_bit_equal(to_host(dv[i]), ref.state[str(i)][1], f"v {i}")
+    table.close()
