@@ -56,6 +56,8 @@ def parse_args():
                          "interleaved with released memory); plain: wherever the driver puts them")
     ap.add_argument("--spread-block-mb", type=int, default=0, help="--placement spread: block size (0 = the library's 64)")
     ap.add_argument("--spread-keep", type=int, default=0, help="--placement spread: every n-th block is kept (0 = 3)")
+    ap.add_argument("--micro", type=int, default=4,
+                    help="cfg5-deferred and the engine workloads: micro-batches per optimizer step (deferred: up to 8)")
     ap.add_argument("--defer", type=int, default=0,
                     help="engine workloads: 1 = defer_accumulation (four resident micro-batches, no accumulation "
                          "buffer, summed in registers by the applying call)")
@@ -250,7 +252,7 @@ class Workload:
     def _setup_cfg5_deferred(self):
         t, mx = self.torch, self.mx
         bf = t.bfloat16
-        self.n_micro = 4
+        self.n_micro = self.args.micro
         self.p = self._randn_list(bf, 0.02)
         self.m = self._zeros_list()
         self.v = self._zeros_list()
@@ -265,7 +267,8 @@ class Workload:
         self.bytes_per_elem = {"norm_of_sum": 2 * self.n_micro, "adamw": 2 * self.n_micro + 10 + 10}
         self.step_bytes_per_elem = sum(self.bytes_per_elem.values())
         self.dominant = "adamw"
-        self.note = "4 resident micro-batches summed in registers (float32, arrival order) by the norm pass and by AdamW"
+        self.note = (f"{self.n_micro} resident micro-batches summed in registers (float32, arrival order) by the norm "
+                     "pass and by AdamW")
 
     def _step_cfg5_deferred(self):
         c = self.ctx
@@ -387,35 +390,35 @@ class Workload:
         self.p = self._randn_list(bf, 0.02)
         self.g = self._randn_list(bf, 1e-3)
         params = dict(zip(self.names, self.p))
-        self.n_micro = 4
+        self.n_micro = N = self.args.micro
         defer = bool(self.args.defer)
         # deferred accumulation reads every micro-batch of the cycle at the end: they must all be resident
         self.micro = [dict(zip(self.names, self.g))]
         for _ in range(self.n_micro - 1 if defer else 0):
             self.micro.append(dict(zip(self.names, self._randn_list(bf, 1e-3))))
         if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
-            self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=4,
+            self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=N,
                                                      defer_accumulation=defer, ctx=self.ctx)
             if defer:
-                self.bytes_per_elem = {"micro_batch_first": 2, "micro_batch": 2, "micro_batch_apply": 2 + 4 * 2 + 4}
+                self.bytes_per_elem = {"micro_batch_first": 2, "micro_batch": 2, "micro_batch_apply": 2 + N * 2 + 4}
                 self.note = ("per micro-batch: validity+norm of clamp(g) (2 B), 32-byte read-back; the last call adds "
                              "sum_j clip_j(clamp(g_j)) in registers and applies lr/N (12 B)")
             else:
                 self.bytes_per_elem = {"micro_batch_first": 2 + 6, "micro_batch": 2 + 10, "micro_batch_apply": 2 + 10}
                 self.note = "per micro-batch: validity+norm of clamp(g) (2 B), acc += clip(clamp(g)) (6/10 B), 32-byte read-back"
         else:                # acc += g in float32, last pass carries the norm of acc/N; p -= lr*(clip(acc/N) + wd*p)
-            self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=4,
+            self.engine = mx.SFTEngineOptimizerSide(params, learning_rate=2e-5, gradient_accumulation_steps=N,
                                                     weight_decay=0.01, accumulate_in_f32=True,
                                                     defer_accumulation=defer, ctx=self.ctx)
             if defer:
-                self.bytes_per_elem = {"micro_batch_apply": 4 * 2 + 4 * 2 + 4}
+                self.bytes_per_elem = {"micro_batch_apply": N * 2 + N * 2 + 4}
                 self.note = ("micro-batches 1-3 only leave their addresses; the last call takes the norm of sum/N "
                              "(8 B, read only) and updates from the same four streams (12 B)")
             else:
                 self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 6 + 10}
                 self.note = "float32 accumulation buffer; last micro-batch: norm of (acc+g)/N read-only, then folded into the update"
         self.step_bytes_per_elem = (self.bytes_per_elem.get("micro_batch_first", 0) +
-                                    2 * self.bytes_per_elem.get("micro_batch", 0) +
+                                    (N - 2) * self.bytes_per_elem.get("micro_batch", 0) +
                                     self.bytes_per_elem["micro_batch_apply"])
         self.dominant = "micro_batch_apply"
         self.dtype = "f32"

@@ -256,13 +256,15 @@ int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double le
  * Qwen3Model::accumulate_gradients (models/qwen3/model.rs:2217-2243) / the engines
  * (grpo/engine.rs:2632-2666, sft/engine.rs:282-290) would have made into a float32 buffer, in the
  * same order, so parameters and moments come out bit-identical while the buffer is never written
- * or read back: four bf16 micro-batches + AdamW move 36 B/elem instead of 58.
+ * or read back: four bf16 micro-batches + AdamW move 36 B/elem instead of 58.  Up to
+ * MXOPT_MAX_PENDING + 1 = 8 micro-batches can be held (with more than four the kernels walk a chunk
+ * in smaller pieces and reach somewhat less bandwidth: ten or more concurrent streams).
  *
  * tensor.g is the first addend: the first micro-batch, or a float32 buffer that already holds
  * earlier ones (more micro-batches than MXOPT_MAX_PENDING + 1).  The pending streams x0.. all have
  * one dtype; tensor.g has that dtype or float32.  The caller keeps every stream alive and unchanged
  * until the update has run.  No counterpart in the reference (it materialises every sum). */
-#define MXOPT_MAX_PENDING 3
+#define MXOPT_MAX_PENDING 7
 
 /* Attach k (0..MXOPT_MAX_PENDING; 0 detaches) pending streams to every row of the table:
  * streams[j * num_tensors + i] is pending stream j of row i, `dtype` their element type.  A

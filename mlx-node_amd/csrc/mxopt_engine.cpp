@@ -294,7 +294,7 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
       if (!e->held_slots.empty()) {
         mxopt_table* t = nullptr;
         if ((rc = defer_table(e, &t))) return rc;
-        const float* scales[MXOPT_MAX_PENDING + 1] = {nullptr, nullptr, nullptr, nullptr};
+        const float* scales[MXOPT_MAX_PENDING + 1] = {};
         if (e->cfg.has_gradient_clip_norm)
           for (size_t j = 0; j < e->held.size(); ++j) scales[j] = &e->d_result[j].scale;
         prep.d_scale = nullptr;

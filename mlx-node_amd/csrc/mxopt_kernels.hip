@@ -488,30 +488,32 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
 // or a float32 buffer that already holds earlier ones.
 // ------------------------------------------------------------------------------------
 
-constexpr int kMaxPending = MXOPT_MAX_PENDING;
+// KMAX: how many pending streams the instance has registers for (3 for up to four micro-batches, else 7).
 
+template <int KMAX>
 struct PendingStreams {
-  const void* x[kMaxPending];
+  const void* x[KMAX];
 };
 
-__device__ __forceinline__ PendingStreams pending_of(const void* const* __restrict__ X, uint32_t ntensors, uint32_t row,
+template <int KMAX>
+__device__ __forceinline__ PendingStreams<KMAX> pending_of(const void* const* __restrict__ X, uint32_t ntensors, uint32_t row,
                                                      int kx) {
-  PendingStreams ps;
+  PendingStreams<KMAX> ps;
 #pragma unroll
-  for (int j = 0; j < kMaxPending; ++j) ps.x[j] = j < kx ? X[(size_t)j * ntensors + row] : nullptr;
+  for (int j = 0; j < KMAX; ++j) ps.x[j] = j < kx ? X[(size_t)j * ntensors + row] : nullptr;
   return ps;
 }
 
-template <int GD, int XD>
-__device__ __forceinline__ float pending_sum_element(const void* G, const PendingStreams& ps, int kx, uint64_t off) {
+template <int GD, int XD, int KMAX>
+__device__ __forceinline__ float pending_sum_element(const void* G, const PendingStreams<KMAX>& ps, int kx, uint64_t off) {
   float s = Elem<GD>::load(G, off);
 #pragma unroll
-  for (int j = 0; j < kMaxPending; ++j)
+  for (int j = 0; j < KMAX; ++j)
     if (j < kx) s = s + Elem<XD>::load(ps.x[j], off);
   return s;
 }
 
-template <int PD, int GD, int XD, class Math>
+template <int PD, int GD, int XD, int KMAX, class Math>
 __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* __restrict__ T,
                                                                const DevChunk* __restrict__ C, DevTensor one,
                                                                uint32_t nchunks, uint32_t ntensors,
@@ -525,32 +527,32 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
   // Either prep(g + x0 + ...) or, with kPrepEachStream, prep_0(g) + prep_1(x0) + ...: every micro-batch
   // clamped and scaled by its own clip factor before it is added (grpo/engine.rs:636-661).
   const bool each = (pr.flags & kPrepEachStream) != 0;
-  PrepRegs ps_regs[kMaxPending + 1];
+  PrepRegs ps_regs[KMAX + 1];
 #pragma unroll
-  for (int j = 0; j <= kMaxPending; ++j) {
+  for (int j = 0; j <= KMAX; ++j) {
     ps_regs[j] = pr;
     const bool has = each && j <= kx && scales.s[j] != nullptr;
     ps_regs[j].has_scale = has;
     ps_regs[j].scale = has ? *scales.s[j] : 1.0f;
   }
-  auto gradient = [&](float g, const float (&x)[kMaxPending]) {
+  auto gradient = [&](float g, const float (&x)[KMAX]) {
     if (!each) {
       float s = g;
 #pragma unroll
-      for (int k = 0; k < kMaxPending; ++k)
+      for (int k = 0; k < KMAX; ++k)
         if (k < kx) s = s + x[k];
       return prep_all(pr, s);
     }
     float s = prep_all(ps_regs[0], g);
 #pragma unroll
-    for (int k = 0; k < kMaxPending; ++k)
+    for (int k = 0; k < KMAX; ++k)
       if (k < kx) s = s + prep_all(ps_regs[k + 1], x[k]);
     return s;
   };
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
     const ChunkView cv = locate(T, C, one, c);
-    const PendingStreams ps = pending_of(X, ntensors, cv.tensor, kx);
+    const PendingStreams<KMAX> ps = pending_of<KMAX>(X, ntensors, cv.tensor, kx);
     const uint64_t start = cv.start;
     const uint32_t len = cv.len, flags = cv.t.flags;
     const float bc1 = cv.t.bc1, bc2 = cv.t.bc2;
@@ -562,9 +564,9 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
     const bool use_v = math.uses_v(flags), read_v = math.reads_v(flags);
     auto one_element = [&](uint64_t off) {
       float p = Elem<PD>::load(P, off);
-      float xs[kMaxPending];
+      float xs[KMAX];
 #pragma unroll
-      for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? Elem<XD>::load(ps.x[k], off) : 0.0f;
+      for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? Elem<XD>::load(ps.x[k], off) : 0.0f;
       const float ge = gradient(Elem<GD>::load(G, off), xs);
       float m = Math::kM ? M[off] : 0.0f;
       float v = read_v ? V[off] : 0.0f;
@@ -574,14 +576,39 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
       if (use_v) V[off] = v;
     };
 
-    if (cv.fast) {
-      float p[U][E], g[U][E], x[kMaxPending][U][E], m[U][E], v[U][E];
+    if (cv.fast && KMAX > 3) {
+      // Many streams: one group per lane at a time (the same bytes in flight as four streams with the
+      // whole chunk loaded up front, and half the registers).
+#pragma unroll 1
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
+        float p[E], g[E], x[KMAX][E], m[E], v[E];
+        load_group<GD, E, false>(G, off, g);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+          if (k < kx) load_group<XD, E, false>(ps.x[k], off, x[k]);
+        load_group<PD, E, false>(P, off, p);
+        if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m);
+        if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          float xs[KMAX];
+#pragma unroll
+          for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? x[k][e] : 0.0f;
+          math(p[e], gradient(g[e], xs), m[e], v[e], bc1, bc2, flags);
+        }
+        store_group<PD, E, false>(PO, off, p);
+        if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m);
+        if (use_v) store_group<MXOPT_F32, E, false>(V, off, v);
+      }
+    } else if (cv.fast) {
+      float p[U][E], g[U][E], x[KMAX][U][E], m[U][E], v[U][E];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
         load_group<GD, E, false>(G, off, g[j]);
 #pragma unroll
-        for (int k = 0; k < kMaxPending; ++k)
+        for (int k = 0; k < KMAX; ++k)
           if (k < kx) load_group<XD, E, false>(ps.x[k], off, x[k][j]);
         load_group<PD, E, false>(P, off, p[j]);
         if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m[j]);
@@ -591,9 +618,9 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float xs[kMaxPending];
+          float xs[KMAX];
 #pragma unroll
-          for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? x[k][j][e] : 0.0f;
+          for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? x[k][j][e] : 0.0f;
           math(p[j][e], gradient(g[j][e], xs), m[j][e], v[j][e], bc1, bc2, flags);
         }
       }
@@ -608,19 +635,19 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
       const uint32_t ngroups = (flags & kTfUnaligned) ? 0u : len / E;
       for (uint32_t q = tid; q < ngroups; q += kThreads) {
         const uint64_t off = start + (uint64_t)q * E;
-        float p[E], g[E], x[kMaxPending][E], m[E], v[E];
+        float p[E], g[E], x[KMAX][E], m[E], v[E];
         load_group<PD, E, false>(P, off, p);
         load_group<GD, E, false>(G, off, g);
 #pragma unroll
-        for (int k = 0; k < kMaxPending; ++k)
+        for (int k = 0; k < KMAX; ++k)
           if (k < kx) load_group<XD, E, false>(ps.x[k], off, x[k]);
         if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m);
         if (read_v) load_group<MXOPT_F32, E, false>(V, off, v);
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float xs[kMaxPending];
+          float xs[KMAX];
 #pragma unroll
-          for (int k = 0; k < kMaxPending; ++k) xs[k] = k < kx ? x[k][e] : 0.0f;
+          for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? x[k][e] : 0.0f;
           math(p[e], gradient(g[e], xs), m[e], v[e], bc1, bc2, flags);
         }
         store_group<PD, E, false>(PO, off, p);
@@ -634,7 +661,7 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
 }
 
 // Sum of squares of prep_pre(g + x_0 + ...), nothing stored: the norm the update above will clip by.
-template <int GD, int XD, bool NT>
+template <int GD, int XD, int KMAX, bool NT>
 __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* __restrict__ T,
                                                               const DevChunk* __restrict__ C, DevTensor one,
                                                               uint32_t nchunks, uint32_t ntensors,
@@ -649,22 +676,41 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
 
   for (uint32_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
     const ChunkView cv = locate(T, C, one, c);
-    const PendingStreams ps = pending_of(X, ntensors, cv.tensor, kx);
+    const PendingStreams<KMAX> ps = pending_of<KMAX>(X, ntensors, cv.tensor, kx);
     const void* G = cv.t.g;
     float s32 = 0.0f;
     bool bad = false;
     auto one_element = [&](uint64_t off) {
-      const float y = norm_value(pr, pending_sum_element<GD, XD>(G, ps, kx, off), clamped, bad);
+      const float y = norm_value(pr, pending_sum_element<GD, XD, KMAX>(G, ps, kx, off), clamped, bad);
       s32 = fmaf(y, y, s32);
     };
-    if (cv.fast) {
-      float g[U][E], x[kMaxPending][U][E];
+    if (cv.fast && KMAX > 3) {
+#pragma unroll 1
+      for (int j = 0; j < U; ++j) {
+        const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
+        float g[E], x[KMAX][E];
+        load_group<GD, E, NT>(G, off, g);
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+          if (k < kx) load_group<XD, E, NT>(ps.x[k], off, x[k]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          float s = g[e];
+#pragma unroll
+          for (int k = 0; k < KMAX; ++k)
+            if (k < kx) s = s + x[k][e];
+          const float y = norm_value(pr, s, clamped, bad);
+          s32 = fmaf(y, y, s32);
+        }
+      }
+    } else if (cv.fast) {
+      float g[U][E], x[KMAX][U][E];
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
         load_group<GD, E, NT>(G, off, g[j]);
 #pragma unroll
-        for (int k = 0; k < kMaxPending; ++k)
+        for (int k = 0; k < KMAX; ++k)
           if (k < kx) load_group<XD, E, NT>(ps.x[k], off, x[k][j]);
       }
 #pragma unroll
@@ -673,7 +719,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
         for (int e = 0; e < E; ++e) {
           float s = g[j][e];
 #pragma unroll
-          for (int k = 0; k < kMaxPending; ++k)
+          for (int k = 0; k < KMAX; ++k)
             if (k < kx) s = s + x[k][j][e];
           const float y = norm_value(pr, s, clamped, bad);
           s32 = fmaf(y, y, s32);
@@ -686,7 +732,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
         float g[E], x[E];
         load_group<GD, E, false>(G, off, g);
 #pragma unroll
-        for (int k = 0; k < kMaxPending; ++k) {
+        for (int k = 0; k < KMAX; ++k) {
           if (k < kx) {
             load_group<XD, E, false>(ps.x[k], off, x);
 #pragma unroll
@@ -938,6 +984,16 @@ bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep
                      (L).nchunks, (L).ntensors, (L).pending, (L).npending, __VA_ARGS__)
 #define MXOPT_LAUNCH_UPDATE_LIST(kernel, L, ...) MXOPT_LAUNCH_LIST(kernel, L, (L).scales, __VA_ARGS__)
 
+constexpr int kFewPending = 3;  // up to four micro-batches take the instance with fewer registers
+
+template <int PD, int GD, int XD, class Math>
+static void launch_update_list_t(const Launch& L, const Math& math, const DevPrep& prep) {
+  if (L.npending <= kFewPending)
+    MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, GD, XD, kFewPending, Math>), L, math, prep);
+  else
+    MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, GD, XD, MXOPT_MAX_PENDING, Math>), L, math, prep);
+}
+
 // g is either of the pending streams' dtype (the first micro-batch) or float32 (a buffer of earlier ones).
 template <int PD, class Math>
 static bool update_list_for_pd(int gd, int xd, const Launch& L, const Math& math, const DevPrep& prep) {
@@ -945,15 +1001,15 @@ static bool update_list_for_pd(int gd, int xd, const Launch& L, const Math& math
   const bool same = gd == xd;
   switch (xd) {
     case MXOPT_F32:
-      MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F32, Math>), L, math, prep);
+      launch_update_list_t<PD, MXOPT_F32, MXOPT_F32>(L, math, prep);
       return true;
     case MXOPT_BF16:
-      if (same) MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_BF16, MXOPT_BF16, Math>), L, math, prep);
-      else MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_BF16, Math>), L, math, prep);
+      if (same) launch_update_list_t<PD, MXOPT_BF16, MXOPT_BF16>(L, math, prep);
+      else launch_update_list_t<PD, MXOPT_F32, MXOPT_BF16>(L, math, prep);
       return true;
     case MXOPT_F16:
-      if (same) MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F16, MXOPT_F16, Math>), L, math, prep);
-      else MXOPT_LAUNCH_UPDATE_LIST((update_list_kernel<PD, MXOPT_F32, MXOPT_F16, Math>), L, math, prep);
+      if (same) launch_update_list_t<PD, MXOPT_F16, MXOPT_F16>(L, math, prep);
+      else launch_update_list_t<PD, MXOPT_F32, MXOPT_F16>(L, math, prep);
       return true;
   }
   return false;
@@ -982,8 +1038,13 @@ bool launch_sgd_plain_list(int pd, int gd, int od, int xd, const Launch& L, floa
 
 template <int GD, int XD>
 static void launch_sumsq_list_t(const Launch& L, const DevPrep& prep, double* ps) {
-  if (L.nontemporal) MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, true>), L, prep, ps);
-  else MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, false>), L, prep, ps);
+  if (L.npending <= kFewPending) {
+    if (L.nontemporal) MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, kFewPending, true>), L, prep, ps);
+    else MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, kFewPending, false>), L, prep, ps);
+  } else {
+    if (L.nontemporal) MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, MXOPT_MAX_PENDING, true>), L, prep, ps);
+    else MXOPT_LAUNCH_LIST((sumsq_list_kernel<GD, XD, MXOPT_MAX_PENDING, false>), L, prep, ps);
+  }
 }
 
 bool launch_sumsq_list(int gd, int xd, const Launch& L, const DevPrep& prep, double* partial_sum) {

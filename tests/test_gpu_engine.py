@@ -213,7 +213,7 @@ def test_one_micro_batch_per_step(mx, kind, apply, bf16):
 # ---------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("n_acc", [1, 3, 4])
+@pytest.mark.parametrize("n_acc", [1, 3, 4, 6])
 def test_grpo_deferred_sequence(mx, bf16, n_acc):
     rng = np.random.default_rng(107 + n_acc)
     params = make_params(rng, bf16)
@@ -222,7 +222,7 @@ def test_grpo_deferred_sequence(mx, bf16, n_acc):
               max_nan_gradients=50, emergency_save_threshold=2)
     dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
     ref = O.GRPOEngineOptimizerSide(params, **kw)
-    script = ["ok", "ok", "nan", "inf", "ok", "ok", "-inf", "ok", "ok", "ok", "ok", "ok", "ok"]
+    script = ["ok", "ok", "nan", "inf", "ok", "ok", "-inf", "ok", "ok", "ok", "ok", "ok", "ok", "ok", "ok"]
     for it, kind in enumerate(script):
         grads = make_grads(rng, bf16, 0.01 * (1 + it % 3))
         if kind != "ok":
@@ -249,19 +249,20 @@ def test_grpo_deferred_sequence(mx, bf16, n_acc):
 
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("apply", ["sgd", "adamw"])
-def test_sft_deferred_sequence(mx, bf16, apply):
+@pytest.mark.parametrize("n_acc", [3, 6])
+def test_sft_deferred_sequence(mx, bf16, apply, n_acc):
     rng = np.random.default_rng(123)
     params = make_params(rng, bf16)
     dparams = {k: to_dev(v) for k, v in params.items()}
-    kw = dict(learning_rate=0.02, gradient_accumulation_steps=3, gradient_clip_norm=0.5, gradient_clip_value=0.002,
+    kw = dict(learning_rate=0.02, gradient_accumulation_steps=n_acc, gradient_clip_norm=0.5, gradient_clip_value=0.002,
               weight_decay=0.01, apply=apply)
     dev = mx.SFTEngineOptimizerSide(dparams, accumulate_in_f32=True, defer_accumulation=True, **kw)
     ref = O.SFTEngineOptimizerSide(params, **kw)
-    for it in range(8):                                     # two full cycles + two leftover micro-batches
+    for it in range(2 * n_acc + 2):                         # two full cycles + two leftover micro-batches
         grads = make_grads(rng, bf16, 0.01)
         m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
         wide = {k: O.as_f32(g) for k, g in grads.items()}    # a float32 sum = float32 gradients to the oracle
-        boundary = ref.state.micro_step + 1 >= 3
+        boundary = ref.state.micro_step + 1 >= n_acc
         r = ref.micro_batch(wide, norm_sumsq=m.grad_sumsq) if boundary else ref.micro_batch(wide)
         assert bool(m.norm_measured) == boundary
         assert (bool(m.gradients_applied), m.step) == (r["gradients_applied"], r["step"])
@@ -277,8 +278,8 @@ def test_deferred_mode_refuses_what_it_cannot_hold(mx):
     rng = np.random.default_rng(5)
     params = make_params(rng, False)
     dparams = {k: to_dev(v) for k, v in params.items()}
-    with pytest.raises(ValueError, match="at most 4 micro-batches"):
-        mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=5, accumulate_in_f32=True, defer_accumulation=True)
+    with pytest.raises(ValueError, match="at most 8 micro-batches"):
+        mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=9, accumulate_in_f32=True, defer_accumulation=True)
     with pytest.raises(ValueError, match="adds in float32"):
         mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=2, defer_accumulation=True)
     with pytest.raises(ValueError, match="plain SGD only"):

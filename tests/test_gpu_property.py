@@ -272,7 +272,7 @@ def test_host_layer_utilities_match_the_oracle(mx, sizes, bf16, max_norm, clip_v
 
 
 @settings(max_examples=150, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
-@given(sizes=st.lists(SIZES, min_size=1, max_size=4), k=st.integers(0, 3), head=st.sampled_from([0, 1, 2, 3, "mixed"]),
+@given(sizes=st.lists(SIZES, min_size=1, max_size=4), k=st.integers(0, 7), head=st.sampled_from([0, 1, 2, 3, "mixed"]),
        pd=st.sampled_from(DTYPES), xd=st.sampled_from(DTYPES), first_f32=st.booleans(),
        kind=st.sampled_from(["adamw", "sgd_plain", "sgd_plain_each"]), pre_mul=st.sampled_from([None, 0.5]),
        clamp_pre=st.sampled_from([None, 1.5e-3]), clip=st.booleans(), clamp_post=st.sampled_from([None, 4e-4]),
