@@ -417,6 +417,10 @@ class Workload:
             else:
                 self.bytes_per_elem = {"micro_batch_first": 6, "micro_batch": 10, "micro_batch_apply": 6 + 10}
                 self.note = "float32 accumulation buffer; last micro-batch: norm of (acc+g)/N read-only, then folded into the update"
+        if N == 1:   # one micro-batch per step: norm of g (2 B), update straight from g (6 B), either engine
+            self.bytes_per_elem = {"micro_batch_apply": 2 + 6}
+        elif N == 2:
+            self.bytes_per_elem.pop("micro_batch", None)
         self.step_bytes_per_elem = (self.bytes_per_elem.get("micro_batch_first", 0) +
                                     (N - 2) * self.bytes_per_elem.get("micro_batch", 0) +
                                     self.bytes_per_elem["micro_batch_apply"])
@@ -433,7 +437,7 @@ class Workload:
 
     def _step_grpo_engine(self):
         for k in range(self.n_micro):
-            name = "micro_batch_first" if k == 0 else ("micro_batch_apply" if k == self.n_micro - 1 else "micro_batch")
+            name = "micro_batch_apply" if k == self.n_micro - 1 else ("micro_batch_first" if k == 0 else "micro_batch")
             self._timed(name, lambda: self.engine.micro_batch(self.micro[k % len(self.micro)]))
 
     _step_sft_engine = _step_grpo_engine
