@@ -14,6 +14,7 @@ TF_FIRST = 0x1
 SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM = 0, 1, 2
 CLIP_ALWAYS_MULTIPLY, CLIP_IF_ABOVE = 0, 1
 CHUNK_ELEMS = 4096
+MAX_PENDING = 7
 
 
 class MxoptError(RuntimeError):

@@ -52,6 +52,7 @@ def test_ctypes_structs_match_c_layout(L, tmp_path):
 #include "mxopt_engine.h"
 #define S(T) printf(#T " %zu\n", sizeof(T))
 #define F(T, f) printf(#T "." #f " %zu\n", offsetof(T, f))
+#define V(name) printf("=" #name " %ld\n", (long)(name))
 int main(void) {
   S(mxopt_tensor); F(mxopt_tensor, n); F(mxopt_tensor, p_dtype); F(mxopt_tensor, flags); F(mxopt_tensor, bc2);
   S(mxopt_norm_result); F(mxopt_norm_result, norm_f32); F(mxopt_norm_result, scale); F(mxopt_norm_result, nonfinite);
@@ -64,6 +65,11 @@ int main(void) {
   F(mxopt_engine_config, apply); F(mxopt_engine_config, eps); F(mxopt_engine_config, accumulate_in_f32); F(mxopt_engine_config, defer_accumulation);
   S(mxopt_engine_metrics); F(mxopt_engine_metrics, nan_gradient_count); F(mxopt_engine_metrics, clip_scale);
   F(mxopt_engine_metrics, grad_norm);
+  V(MXOPT_OK); V(MXOPT_ERR_INVALID_ARG); V(MXOPT_ERR_FAILURE); V(MXOPT_ERR_HIP); V(MXOPT_ERR_OOM);
+  V(MXOPT_TF_FIRST); V(MXOPT_CHUNK_ELEMS); V(MXOPT_MAX_PENDING); V(MXOPT_CLIP_ALWAYS_MULTIPLY); V(MXOPT_CLIP_IF_ABOVE);
+  V(MXOPT_SYNTH_NORMAL); V(MXOPT_SYNTH_NORMAL_OUTLIERS); V(MXOPT_SYNTH_UNIFORM);
+  V(MXOPT_ENGINE_GRPO); V(MXOPT_ENGINE_SFT); V(MXOPT_ENGINE_APPLY_SGD); V(MXOPT_ENGINE_APPLY_ADAMW);
+  V(MXOPT_F32); V(MXOPT_F16); V(MXOPT_BF16);
   return 0;
 }''')
     exe = tmp_path / "layout"
@@ -73,7 +79,9 @@ int main(void) {
           "mxopt_adam_hp": L.AdamHp, "mxopt_sgd_hp": L.SgdHp, "mxopt_rmsprop_hp": L.RmspropHp, "mxopt_array": L.Array,
           "mxopt_engine_config": L.EngineConfig, "mxopt_engine_metrics": L.EngineMetrics}
     for key, val in want.items():
-        if "." in key:
+        if key.startswith("="):     # a constant: the ctypes module carries it without the MXOPT_ prefix
+            assert getattr(L, key[len("=MXOPT_"):]) == int(val), key
+        elif "." in key:
             t, f = key.split(".")
             assert getattr(py[t], f).offset == int(val), key
         else:
