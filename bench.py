@@ -13,6 +13,10 @@ before it starts).  `roofline` describes the dominant kernel (the AdamW update):
 bytes per launch / its average duration measured with events on the launch stream.
 `cpu_baseline` times the CPU restatement of the reference's un-fused op chain (oracle/) on a
 bounded sample of the same workload and scales it to the full parameter list.
+`deferred_accumulation` (default workload only, when four micro-batch buffers fit) is the same step on
+the same buffers with the micro-batches added in registers instead of into the float32 buffer.
+The buffers are allocated inside mxopt_hbm_spread_begin/_end unless --placement plain is given
+(`config.placement` says which).
 """
 from __future__ import annotations
 
