@@ -30,6 +30,8 @@ class _EngineOptimizerSide:
     def __init__(self, params: Dict[str, torch.Tensor], cfg: L.EngineConfig, ctx: Optional[Context]):
         self.ctx = ctx or default_context()
         self.lib = self.ctx.lib
+        self.defers = bool(cfg.defer_accumulation)
+        self._held = []
         self.params = dict(params)
         names = list(self.params)
         cnames = (C.c_char_p * max(len(names), 1))(*[s.encode() for s in names])
@@ -63,10 +65,11 @@ class _EngineOptimizerSide:
         for i, nm in enumerate(names):
             arrs[i] = _arr(gradients[nm])
         m = L.EngineMetrics()
-        held = getattr(self, "_held", [])
-        held.append(list(gradients.values()))    # deferred accumulation reads them when the cycle is applied
+        if self.defers:   # deferred accumulation reads the cycle's gradients when it is applied: keep them alive
+            self._held.append(list(gradients.values()))
         self._check(self.lib.mxopt_engine_micro_batch(self.handle, len(names), cnames, arrs, C.byref(m)))
-        self._held = [] if m.gradients_applied or m.micro_step == 0 else held
+        if m.gradients_applied or m.micro_step == 0:
+            self._held = []
         return m
 
     def metrics(self) -> L.EngineMetrics:
@@ -95,6 +98,7 @@ class _EngineOptimizerSide:
 
     def reset(self) -> None:
         self._check(self.lib.mxopt_engine_reset(self.handle))
+        self._held = []
 
     def save_optimizer_state(self, path) -> None:
         self._check(self.lib.mxopt_engine_save_optimizer_state(self.handle, str(path).encode()))
@@ -162,6 +166,7 @@ class SFTEngineOptimizerSide(_EngineOptimizerSide):
         flushed = C.c_int()
         m = L.EngineMetrics()
         self._check(self.lib.mxopt_engine_flush_gradients(self.handle, C.byref(flushed), C.byref(m)))
+        self._held = []
         self.last_metrics = m
         return bool(flushed.value)
 
