@@ -2,7 +2,7 @@
  *
  *   cabi_demo            known-answer checks through the optimizer objects (the reference's own
  *                        closed forms: __test__/core/optimizers.test.ts:151-203, 324-351) and the
- *                        engine entry points, then a timing of updateSingle-per-tensor against
+ *                        engine entry points (with and without an accumulation buffer), then a timing of updateSingle-per-tensor against
  *                        one update_many call over the Qwen3-0.6B parameter list.
  * Prints "PASS" lines and one "TIMING" line; exits non-zero on the first mismatch.
  */
@@ -113,6 +113,27 @@ static void known_answers(void) {
   const double want_w[2] = {9.975, 19.965};
   expect_close("GRPO engine: 4 micro-batches, lr/N", w, want_w, 2, 5e-6);
   mxopt_engine_free(eng);
+
+  /* The same known answer with no accumulation buffer: the engine only remembers where the four
+   * micro-batches lie (the host keeps them alive) and the last call adds them in registers.  The
+   * parameter and the gradients are allocated inside a placement window, as a host would at start-up. */
+  mxopt_hbm_spread* window = NULL;
+  CHECK_MX(mxopt_hbm_spread_begin(ctx, (size_t)512 << 20, 2, &window));
+  float* w2 = to_device(w0, 2);
+  float* held[4];
+  for (int k = 0; k < 4; ++k) held[k] = to_device(gs[k], 2);
+  CHECK_MX(mxopt_hbm_spread_end(window));
+  cfg.defer_accumulation = 1;
+  mxopt_array aw2 = {w2, 2, MXOPT_F32};
+  CHECK_MX(mxopt_engine_new(ctx, &cfg, 1, names, &aw2, &eng));
+  for (int k = 0; k < 4; ++k) {
+    mxopt_array a = {held[k], 2, MXOPT_F32};
+    CHECK_MX(mxopt_engine_micro_batch(eng, 1, names, &a, &m));
+    if (m.gradients_applied != (k == 3) || m.step != k + 1) { fprintf(stderr, "FAIL deferred engine bookkeeping at %d\n", k); exit(1); }
+  }
+  expect_close("GRPO engine, deferred accumulation: same answer", w2, want_w, 2, 5e-6);
+  mxopt_engine_free(eng);
+  for (int k = 0; k < 4; ++k) CHECK_HIP(hipFree(held[k]));
 }
 
 /* Qwen3-0.6B: vocab 151936, hidden 1024, 28 layers, q 2048x1024, k/v 1024x1024, o 1024x2048,
