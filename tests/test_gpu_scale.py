@@ -15,7 +15,9 @@
 * Qwen3-8B list, bf16 parameters / float32 moments, 4 micro-batches into a float32 buffer, clip 1.0,
   last micro-batch folded into the update (config 5, ~131 GB resident): seeded windows of every stream
   are read back before and after the step and pushed through the NumPy oracle (bit-exact given the
-  device's clip factor); norm as above.
+  device's clip factor); norm as above.  With generated inputs, EVERY element of every sixth tensor
+  (1.5 G elements, the embedding among them) of parameters, moments and accumulation buffer against
+  the C twin of the oracle.
 * The same configuration without its accumulation buffer (deferred accumulation: the four resident
   micro-batches are summed in registers): the same sum of squares and a position-weighted checksum of
   EVERY parameter and moment bit equal to those of the buffered run from identical generated inputs.
@@ -411,6 +413,84 @@ def test_config5_full_size_windows_and_norm():
     assert np.array_equal(win(p_slab), want_p), "parameters"
     assert np.array_equal(win(m_slab).view(np.uint32), ref.state["w"][0].view(np.uint32)), "first moment"
     assert np.array_equal(win(v_slab).view(np.uint32), ref.state["w"][1].view(np.uint32)), "second moment"
+    t_acc.close()
+    t_upd.close()
+    ctx.close()
+
+
+def test_config5_every_element_of_every_sixth_tensor(oracle_c):
+    """The benchmark's default step on the whole 8B list from generated inputs (one gradient buffer,
+    refilled for each micro-batch); every element of parameters, moments and accumulation buffer of every
+    sixth tensor -- the embedding and 66 others, 1.5 G elements -- is recomputed on the host by the C
+    twin of the oracle from regenerated inputs and compared bit for bit."""
+    import torch
+    import mxopt as mx
+    _, sizes = qwen_sizes("8B")
+    n, nt = sum(sizes), len(sizes)
+    torch.cuda.empty_cache()
+    free, _ = torch.cuda.mem_get_info()
+    if free < n * 16 + (8 << 30):
+        pytest.skip("needs ~131 GB of free device memory")
+    bf = torch.bfloat16
+    dp = [torch.empty(s, dtype=bf, device="cuda") for s in sizes]
+    dg = [torch.empty(s, dtype=bf, device="cuda") for s in sizes]
+    da = [torch.empty(s, device="cuda") for s in sizes]
+    dm = [torch.empty(s, device="cuda") for s in sizes]
+    dv = [torch.empty(s, device="cuda") for s in sizes]
+    ctx = mx.Context()
+    SEED, CFG = 0x5EED0001, 5
+    P, M, V, G = 0, 1, 2, 3          # stream ids inside the key; micro-batch k uses stream G + k
+
+    def spec(stream):
+        if stream == P:
+            return mx.SYNTH_NORMAL, 0.02, 0.0
+        if stream == M:
+            return mx.SYNTH_NORMAL, 1e-4, 0.0
+        if stream == V:
+            return mx.SYNTH_UNIFORM, 0.0, 1e-8
+        return mx.SYNTH_NORMAL, 1e-3, 0.0
+
+    def fill(tensors, stream):
+        dist, a, b = spec(stream)
+        for i, t in enumerate(tensors):
+            ctx.fill_synthetic(t, mx.synthetic_key(SEED, CFG, 0, stream, i), dist, a, b)
+
+    def host(i, stream, dtype):
+        dist, a, b = spec(stream)
+        return oracle_c.fill_synthetic(sizes[i], dtype, mx.synthetic_key(SEED, CFG, 0, stream, i), dist, a, b)
+
+    fill(dp, P); fill(dm, M); fill(dv, V)
+    t_acc = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(dg, da)])
+    t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=g, m=m, v=v) for p, a, g, m, v in zip(dp, da, dg, dm, dv)])
+    res = ctx.norm_result()
+    for k in range(4):
+        fill(dg, G + k)
+        if k < 3:
+            ctx.accumulate(t_acc, first=(k == 0))
+        else:
+            ctx.accumulate_norm_only(t_acc, res, max_norm=1.0)
+    ctx.adam_with_pending(t_upd, mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01), mx.make_prep(scale=res))
+    r = ctx.read_norm_result(res)
+    expected_norm = 1e-3 * math.sqrt(4 * n)
+    assert abs(r.norm - expected_norm) < 0.01 * expected_norm
+    n32, scale = O.norm_scale_c1(r.sumsq, 1.0)
+    assert F(r.scale) == scale and F(r.norm_f32) == n32 and r.nonfinite == 0
+
+    args = B.adam_args(5e-6, 0.9, 0.999, 1e-8, 0.01, scale=float(scale))
+    checked = 0
+    for i in range(0, nt, 6):
+        p_ref, m_ref, v_ref = host(i, P, "bf16"), host(i, M, "f32"), host(i, V, "f32")
+        acc = np.empty(sizes[i], F)
+        for k in range(3):
+            oracle_c.accumulate_f32(acc, host(i, G + k, "bf16"), k == 0)
+        same_bits(da[i].cpu().numpy(), acc, f"accumulation buffer of tensor {i} (three micro-batches)")
+        oracle_c.accumulate_f32(acc, host(i, G + 3, "bf16"), False)
+        p_new = oracle_c.f32_to_bf16(oracle_c.adam(p_ref, acc, m_ref, v_ref, args, fused=True))
+        same_bits(to_host(dp[i]), p_new, f"p of tensor {i}")
+        same_bits(dm[i].cpu().numpy(), m_ref, f"m of tensor {i}")
+        same_bits(dv[i].cpu().numpy(), v_ref, f"v of tensor {i}")
+        checked += sizes[i]
+    assert checked > 1_400_000_000
     t_acc.close()
     t_upd.close()
     ctx.close()
