@@ -9,7 +9,8 @@
   and regenerated on the host by the oracle's twin of it, the norm is checked against the exact
   float64 sum.
 * Qwen3-4B list, float32 SGD with momentum / RMSprop (config 3): every tensor of at most 1 Mi elements in
-  full plus seeded windows (head, tail, interior) of every larger one, bit for bit.
+  full plus seeded windows (head, tail, interior) of every larger one, bit for bit; with generated inputs,
+  EVERY element of every third tensor (1.5 G elements) over two steps of each optimizer.
 * 10,000 small bf16 tensors (config 4): EVERY element, three steps, packed back to back so that most
   tensors start at an address that is only 2-byte aligned, and separately allocated.
 * Qwen3-8B list, bf16 parameters / float32 moments, 4 micro-batches into a float32 buffer, clip 1.0,
@@ -268,6 +269,71 @@ def test_config3_full_size_sgd_and_rmsprop_windows(oracle_c):
         same_bits(win(p_slab), p_ref, f"rmsprop p step {step}")
         same_bits(win(v_slab), v_ref, f"rmsprop v step {step}")
     table.close()
+    ctx.close()
+
+
+def test_config3_every_element_of_every_third_tensor(oracle_c):
+    """SGD with momentum and RMSprop on the whole 4B list from generated inputs, two steps each (the
+    first SGD step takes the velocity-less branch); every element of every third tensor -- 1.5 G
+    elements, the embedding among them -- is recomputed on the host by the C twin from regenerated
+    inputs."""
+    import torch
+    import mxopt as mx
+    _, sizes = qwen_sizes("4B")
+    nt = len(sizes)
+    torch.cuda.empty_cache()
+    dp = [torch.empty(s, device="cuda") for s in sizes]
+    dg = [torch.empty(s, device="cuda") for s in sizes]
+    dv = [torch.empty(s, device="cuda") for s in sizes]
+    ctx = mx.Context()
+    SEED, CFG = 0x5EED0001, 3
+    picked = list(range(0, nt, 3))
+
+    def key(stream, step, i):
+        return mx.synthetic_key(SEED, CFG, step, stream, i)
+
+    def fill(tensors, stream, step, std):
+        for i, t in enumerate(tensors):
+            ctx.fill_synthetic(t, key(stream, step, i), mx.SYNTH_NORMAL, std)
+
+    def host(i, stream, step, std):
+        return oracle_c.fill_synthetic(sizes[i], "f32", key(stream, step, i), O.SYNTH_NORMAL, std)
+
+    for opt in ("sgd", "rmsprop"):
+        fill(dp, 0, 0, 0.02)
+        p_ref = {i: host(i, 0, 0, 0.02) for i in picked}
+        v_ref = {i: np.zeros(sizes[i], F) for i in picked}
+        if opt == "sgd":
+            for v in dv:
+                v.fill_(float("nan"))                      # must not be read on the first step
+            table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v, flags=mx.TF_FIRST) for p, g, v in zip(dp, dg, dv)])
+            hp = mx.sgd_hp(1e-4, 0.9, 1e-4, 0.0, False)
+        else:
+            for v in dv:
+                v.zero_()
+            table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v) for p, g, v in zip(dp, dg, dv)])
+            hp = mx.rmsprop_hp(1e-4, 0.99, 1e-8, 0.0)
+        for step in range(2):
+            stream = 1 if opt == "sgd" else 2
+            fill(dg, stream, step + 1, 1e-3)
+            if opt == "sgd":
+                if step == 1:
+                    table.set_step_scalars(flags=[0] * nt)
+                ctx.sgd(table, hp)
+                args = B.SgdArgs(lr=f32(1e-4), momentum=f32(0.9), one_minus_damp=f32(1.0), wd=f32(1e-4), has_wd=1,
+                                 has_momentum=1, nesterov=0, first=int(step == 0))
+            else:
+                ctx.rmsprop(table, hp)
+                args = B.RmspropArgs(lr=f32(1e-4), alpha=f32(0.99), one_minus_alpha=f32(1.0 - 0.99), eps=f32(1e-8),
+                                     wd=0.0, has_wd=0)
+            for i in picked:
+                g = host(i, stream, step + 1, 1e-3)
+                fn = oracle_c.sgd if opt == "sgd" else oracle_c.rmsprop
+                p_ref[i] = fn(p_ref[i], g, v_ref[i], args, fused=True)
+                same_bits(dp[i].cpu().numpy(), p_ref[i], f"{opt} p of tensor {i}, step {step}")
+                same_bits(dv[i].cpu().numpy(), v_ref[i], f"{opt} v of tensor {i}, step {step}")
+        table.close()
+    assert sum(sizes[i] for i in picked) > 1_300_000_000
     ctx.close()
 
 
