@@ -2,8 +2,10 @@
 and the 4096-element chunk, empty tensors), element shifts that are common to all streams or not,
 every dtype combination the kernels accept, every optimizer, every stage of the gradient
 pre-processing -- always bit for bit against the oracle.  Examples are derandomised: the same cases
-run every time."""
+run every time.  MXOPT_PROPERTY_EXAMPLES=<n> in the environment turns the file into a soak: n fresh random
+cases per test instead of the fixed ones."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -16,6 +18,14 @@ import mxopt_oracle as O
 from gpu_util import assert_bit_equal, to_dev, to_host
 
 F = np.float32
+SOAK = int(os.environ.get("MXOPT_PROPERTY_EXAMPLES", "0"))
+
+
+def cases(n):
+    return settings(max_examples=SOAK or n, deadline=None, derandomize=not SOAK, database=None,
+                    suppress_health_check=list(HealthCheck))
+
+
 SIZES = st.one_of(st.integers(0, 20), st.integers(4088, 4104), st.integers(8185, 8200), st.integers(21, 30000))
 DTYPES = ["f32", "bf16", "f16"]
 
@@ -53,7 +63,7 @@ def mx():
     return mxopt
 
 
-@settings(max_examples=200, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@cases(200)
 @given(sizes=st.lists(SIZES, min_size=1, max_size=5), shift=st.integers(0, 9), common_shift=st.booleans(),
        kind=st.sampled_from(["adam", "adamw", "adamw_bias", "sgd", "sgd_nesterov", "sgd_no_momentum", "rmsprop"]),
        pd=st.sampled_from(DTYPES), gd=st.sampled_from(DTYPES), out_f32=st.booleans(), in_place=st.booleans(),
@@ -136,7 +146,7 @@ def test_update_kernels_match_the_oracle(mx, sizes, shift, common_shift, kind, p
     t_g.close()
 
 
-@settings(max_examples=150, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@cases(150)
 @given(sizes=st.lists(SIZES, min_size=1, max_size=5), shift=st.integers(0, 9), gd=st.sampled_from(DTYPES),
        acc_f32=st.booleans(), pre_mul=st.sampled_from([None, 0.5]), clamp=st.sampled_from([None, 1.2e-3]),
        poison=st.sampled_from([None, "nan", "inf", "-inf"]), seed=st.integers(0, 2 ** 31))
@@ -223,7 +233,7 @@ def test_accumulation_and_transform_kernels_match_the_oracle(mx, sizes, shift, g
         t.close()
 
 
-@settings(max_examples=120, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@cases(120)
 @given(sizes=st.lists(SIZES, min_size=1, max_size=4), bf16=st.booleans(), max_norm=st.sampled_from([1e-3, 3e-2, 10.0]),
        clip_val=st.sampled_from([2e-4, 1.0]), lr=st.sampled_from([1e-6, 2e-5, 0.3]), seed=st.integers(0, 2 ** 31))
 def test_host_layer_utilities_match_the_oracle(mx, sizes, bf16, max_norm, clip_val, lr, seed):
@@ -271,7 +281,7 @@ def test_host_layer_utilities_match_the_oracle(mx, sizes, bf16, max_norm, clip_v
         assert_bit_equal(to_host(dp[k]), want_p[k], f"applied {k}")
 
 
-@settings(max_examples=150, deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+@cases(150)
 @given(sizes=st.lists(SIZES, min_size=1, max_size=4), k=st.integers(0, 7), head=st.sampled_from([0, 1, 2, 3, "mixed"]),
        pd=st.sampled_from(DTYPES), xd=st.sampled_from(DTYPES), first_f32=st.booleans(),
        kind=st.sampled_from(["adamw", "sgd_plain", "sgd_plain_each"]), pre_mul=st.sampled_from([None, 0.5]),
