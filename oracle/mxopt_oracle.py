@@ -479,8 +479,11 @@ class _EngineBase:
         self.state.needs_emergency_save = False
 
     def reset(self) -> None:
-        """grpo/engine.rs:2533-2546, sft/engine.rs:671-: *state = EngineState::default()."""
+        """grpo/engine.rs:2533-2546, sft/engine.rs:671-: *state = EngineState::default().  With this
+        build's AdamW apply the moments go too, as after the optimizers' own reset() (adamw.rs:146-150)."""
         self.state = _EngineState()
+        if self.adamw is not None:
+            self.adamw.reset()
 
     def _adamw_apply(self, grads: Dict[str, np.ndarray]) -> None:
         """This build's replacement for apply_gradients: AdamW on the prepared gradient, parameter
