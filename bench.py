@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0
 # WRITE_SIZE (each scaled by what the same counter reads for this library's plain copy kernel:
 # 1.98445 and 1.00000); the runs and raw values are in profiles/hbm_traffic_pmc_cfg5_and_copy.txt.
 # (workload, fold_last) -> bytes per element
-MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.97, ("cfg5", 0): 23.93}
+MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.97, ("cfg5", 0): 23.93, ("cfg5-deferred", 1): 27.89}
 
 
 def parse_args():
