@@ -586,7 +586,8 @@ def main():
     roofline = {"bound": "hbm", "achieved": dom["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(dom["gbps"] / HBM_PEAK_GBPS, 4),
                 "traffic": (round(MEASURED_TRAFFIC_B_PER_ELEM[(args.workload, int(args.fold_last))] * n)
-                            if (args.workload, int(args.fold_last)) in MEASURED_TRAFFIC_B_PER_ELEM else None),
+                            if (args.workload, int(args.fold_last)) in MEASURED_TRAFFIC_B_PER_ELEM and args.micro == 4
+                            else None),
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
