@@ -74,8 +74,8 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
 
 /* ---- HBM placement -------------------------------------------------------------------
  * Kernels that walk several streams at once (every update kernel here) run 5 - 12 % faster on this
- * part when the buffers' physical pages are interleaved with unrelated memory instead of lying in one
- * compact run -- what a process gets by default when it is the first to use the GPU.  The library
+ * part in most runs when the buffers' physical pages are interleaved with unrelated memory instead of
+ * lying in one compact run -- what a process gets by default when it is the first to use the GPU.  The library
  * never owns the caller's buffers, so it cannot place them; this pair lets a host do it at start-up:
  *
  *   mxopt_hbm_spread_begin(ctx, 0, 0, &s);    all free device memory is taken in blocks, then two of
