@@ -17,21 +17,20 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxopt.so")
 
-SOURCES = ["mxopt_kernels.hip", "mxopt_api.cpp", "mxopt_optimizers.cpp", "mxopt_engine.cpp", "mxopt_checkpoint.cpp"]
+SOURCES = ["mxopt_kernels.hip", "mxopt_reduce_kernels.hip", "mxopt_list_kernels.hip", "mxopt_api.cpp",
+           "mxopt_optimizers.cpp", "mxopt_engine.cpp", "mxopt_checkpoint.cpp"]
 
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fno-fast-math", "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
     "-I", os.path.join(ROOT, "include"), "-I", CSRC,
 ]
+OBJ_DIR = os.path.join(HERE, "bin", "obj")
 
 
-def build(verbose: bool = False) -> str:
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc] + FLAGS + ["-x", "hip"] + srcs + ["-o", LIB + ".tmp"]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -39,9 +38,24 @@ def build(verbose: bool = False) -> str:
     err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
         sys.stderr.write(err + "\n")
-        raise RuntimeError("hipcc failed")
+        raise RuntimeError("hipcc failed: " + os.path.basename(cmd[-1]))
     if verbose and err.strip():
         print(err)
+
+
+def build(verbose: bool = False) -> str:
+    """Every translation unit is compiled by its own hipcc process (they are independent and the three
+    kernel files take about as long as each other), then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = []
+    for s in SOURCES:
+        obj = os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o")
+        jobs.append(([hipcc] + FLAGS + ["-x", "hip", "-c", os.path.join(CSRC, s), "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+        list(pool.map(lambda j: _run(j[0], verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + [obj for _, obj in jobs] + ["-o", LIB + ".tmp"], verbose)
     os.replace(LIB + ".tmp", LIB)
     build_demo(verbose)
     build_napi(verbose)

@@ -1,6 +1,6 @@
 // Host layer of mxopt: the reference's optimizer objects and gradient utilities over raw
 // device buffers.  Declarations, and the reference methods each entry point stands behind,
-// are in include/mxopt_optimizers.h.  All arithmetic happens in the kernels (mxopt_kernels.hip).
+// are in include/mxopt_optimizers.h.  All arithmetic happens in the kernels (the *_kernels.hip files).
 #include "mxopt_optimizers.h"
 
 #include <hip/hip_runtime_api.h>

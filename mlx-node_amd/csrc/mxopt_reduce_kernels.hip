@@ -1,0 +1,275 @@
+// mxopt kernels for gfx950, part 2: global-norm reduction (optionally fused with gradient accumulation)
+// and the synthetic-data generator.
+#include "mxopt_kernels_common.h"
+
+namespace mxopt {
+
+// ------------------------------------------------------------------------------------
+// Sum of squares, pass 1 (one float64 partial per workgroup), optionally fused with the
+// accumulation  acc = first ? g : acc + g.
+//   MODE 0: square tensor.g                 MODE 1: square tensor.g_out
+//   MODE 2: g_out = first ? g : acc + g, square the new contents (partials optional); acc is
+//           tensor.p when set (out of place), else g_out itself
+//   MODE 3: square (g_out + g) without storing it (the update kernel adds g again itself)
+// AD: dtype of the stream that is squared / accumulated into; GD: dtype of g (MODE 2, 3).
+// ------------------------------------------------------------------------------------
+
+
+template <int AD, int GD>
+__device__ __forceinline__ float accumulate_op(float acc, float g, bool first) {
+  float s = first ? g : acc + g;
+  // bf16 + bf16 -> bf16 and friends: the store rounds.  Squares are taken of the stored value.
+  return Elem<AD>::round(s);
+}
+
+template <int MODE, int AD, int GD, bool NT>
+struct SumsqChunk {
+  static constexpr bool kTwoStreams = MODE >= 2;
+  static constexpr int E = (AD != MXOPT_F32 || (kTwoStreams && GD != MXOPT_F32)) ? 8 : 4;
+  static constexpr int U = kElemsPerLane / E;
+  float x[U][E], g[U][E];
+
+  static __device__ __forceinline__ const void* squared_stream(const ChunkView& cv) {
+    if (MODE == 0) return cv.t.g;
+    if (MODE == 2 && cv.t.p != nullptr) return cv.t.p;
+    return cv.t.g_out;
+  }
+
+  __device__ __forceinline__ void load(const ChunkView& cv, uint32_t tid, bool first) {
+    const void* X = squared_stream(cv);
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
+      if (MODE != 2 || !first) {
+        load_group<AD, E, NT>(X, off, x[j]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[j][e] = 0.0f;
+      }
+      if (kTwoStreams) load_group<GD, E, NT>(cv.t.g, off, g[j]);
+    }
+  }
+
+  // Returns this lane's float32 sum of squares over the chunk; stores the new sum in MODE 2.
+  __device__ __forceinline__ float finish(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
+    float s32 = 0.0f;
+    const bool clamped = (pr.flags & kPrepClampPre) != 0;
+    bool hidden_inf = false;
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
+        if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
+        const float y = norm_value(pr, x[j][e], clamped, hidden_inf);
+        s32 = fmaf(y, y, s32);
+      }
+      if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+    }
+    return hidden_inf ? __builtin_nanf("") : s32;
+  }
+
+  // Partial or unaligned chunk.
+  static __device__ __forceinline__ float slow(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
+    const void* X = squared_stream(cv);
+    const void* G = cv.t.g;
+    void* A = cv.t.g_out;
+    float s32 = 0.0f;
+    const bool clamped = (pr.flags & kPrepClampPre) != 0;
+    const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
+    for (uint32_t q = tid; q < ngroups; q += kThreads) {
+      const uint64_t off = cv.start + (uint64_t)q * E;
+      float x[E], g[E];
+      if (MODE != 2 || !first) {
+        load_group<AD, E, false>(X, off, x);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[e] = 0.0f;
+      }
+      if (kTwoStreams) load_group<GD, E, false>(G, off, g);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
+        if (MODE == 3) x[e] = accumulate_op<AD, GD>(x[e], g[e], false);
+        bool bad = false;
+        const float y = norm_value(pr, x[e], clamped, bad);
+        s32 = bad ? __builtin_nanf("") : fmaf(y, y, s32);
+      }
+      if (MODE == 2) store_group<AD, E, false>(A, off, x);
+    }
+    for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) s32 = one_element(cv, pr, cv.start + i, first, s32);
+    return s32;
+  }
+
+  // Element `off` of the tensor on its own: s32 + its square.
+  static __device__ __forceinline__ float one_element(const ChunkView& cv, const PrepRegs& pr, uint64_t off,
+                                                      bool first, float s32) {
+    const void* X = squared_stream(cv);
+    float x = (MODE != 2 || !first) ? Elem<AD>::load(X, off) : 0.0f;
+    if (MODE == 2) {
+      x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), first);
+      Elem<AD>::store(cv.t.g_out, off, x);
+    }
+    if (MODE == 3) x = accumulate_op<AD, GD>(x, Elem<GD>::load(cv.t.g, off), false);
+    bool bad = false;
+    const float y = norm_value(pr, x, (pr.flags & kPrepClampPre) != 0, bad);
+    return bad ? __builtin_nanf("") : fmaf(y, y, s32);
+  }
+};
+
+template <int MODE, int AD, int GD, bool NT>
+__global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __restrict__ T,
+                                                         const DevChunk* __restrict__ C, DevTensor one,
+                                                         uint32_t nchunks, DevPrep prep, int first_i,
+                                                         double* __restrict__ partial_sum) {
+  using Chunk = SumsqChunk<MODE, AD, GD, NT>;
+  const PrepRegs pr = load_prep(prep);
+  const uint32_t tid = threadIdx.x;
+  const bool first = first_i != 0;
+  double acc_sum = 0.0;
+
+  uint32_t c = blockIdx.x;
+  for (; c < nchunks; c += gridDim.x) {
+    const ChunkView cv = locate(T, C, one, c);
+    float s;
+    if (cv.fast) {
+      Chunk k;
+      k.load(cv, tid, first);
+      s = k.finish(cv, pr, tid, first);
+    } else {
+      s = Chunk::slow(cv, pr, tid, first);
+    }
+    if (tid < cv.head) s = Chunk::one_element(cv, pr, tid, first, s);
+    // A lane's float32 partial covers <= 16 squares of one chunk; chunks are combined in float64.
+    // A NaN/Inf element (or squares that overflow float32) makes the partial, and so the total,
+    // non-finite: that is the validity check (the reference's sum-based one, grpo/engine.rs:1692-1698).
+    acc_sum += (double)s;
+  }
+
+  if (partial_sum != nullptr) {
+    unsigned long long unused = 0;
+    block_sum(acc_sum, unused);
+    if (tid == 0) partial_sum[blockIdx.x] = acc_sum;
+  }
+}
+
+
+// Pass 2: one workgroup folds the partials in a fixed order and derives norm and scale.
+__global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __restrict__ partial_sum,
+                                                               uint32_t npartials, double max_norm, int has_max,
+                                                               int clip_mode, mxopt_norm_result* __restrict__ out) {
+  double s = 0.0;
+  unsigned long long unused = 0;
+  for (uint32_t i = threadIdx.x; i < npartials; i += kThreads) s += partial_sum[i];
+  block_sum(s, unused);
+  if (threadIdx.x == 0) {
+    const double sumsq = s;
+    const double norm = sqrt(sumsq);
+    const float norm32 = (float)norm;
+    float scale = 1.0f;
+    if (has_max) {
+      if (clip_mode == MXOPT_CLIP_ALWAYS_MULTIPLY) {
+        // optimizers/mod.rs:87-96: all float32 scalars
+        float d = norm32 + (float)1e-6;
+        float q = (float)max_norm / d;
+        scale = (q != q) ? q : fminf(q, 1.0f);  // a NaN norm gives a NaN scale
+      } else {
+        // gradients/mod.rs:255-270: float64 on the host, gradients unchanged when norm <= max
+        if (!(norm <= max_norm)) scale = (float)(max_norm / (norm + 1e-6));
+      }
+    }
+    out->sumsq = sumsq;
+    out->norm = norm;
+    out->norm_f32 = norm32;
+    out->scale = scale;
+    out->nonfinite = (sumsq - sumsq == 0.0) ? 0ull : 1ull;  // x - x is 0 exactly for finite x only
+  }
+}
+
+template <int MODE, int AD, int GD>
+static void launch_sumsq_t(const Launch& L, const DevPrep& prep, int first, double* ps) {
+  if (L.nontemporal) MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, true>), L, prep, first, ps);
+  else MXOPT_LAUNCH((sumsq_kernel<MODE, AD, GD, false>), L, prep, first, ps);
+}
+
+template <int MODE, int AD>
+static bool sumsq_for_ad(int gd, const Launch& L, const DevPrep& prep, int first, double* ps) {
+  if (MODE < 2) { launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps); return true; }
+  switch (gd) {
+    case MXOPT_F32: launch_sumsq_t<MODE, AD, MXOPT_F32>(L, prep, first, ps); return true;
+    case MXOPT_BF16: launch_sumsq_t<MODE, AD, MXOPT_BF16>(L, prep, first, ps); return true;
+    case MXOPT_F16: launch_sumsq_t<MODE, AD, MXOPT_F16>(L, prep, first, ps); return true;
+  }
+  return false;
+}
+
+template <int MODE>
+static bool sumsq_for_mode(int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* ps) {
+  switch (ad) {
+    case MXOPT_F32: return sumsq_for_ad<MODE, MXOPT_F32>(gd, L, prep, first, ps);
+    case MXOPT_BF16: return sumsq_for_ad<MODE, MXOPT_BF16>(gd, L, prep, first, ps);
+    case MXOPT_F16: return sumsq_for_ad<MODE, MXOPT_F16>(gd, L, prep, first, ps);
+  }
+  return false;
+}
+
+bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep, int first, double* partial_sum) {
+  switch (mode) {
+    case 0: return sumsq_for_mode<0>(ad, gd, L, prep, first, partial_sum);
+    case 1: return sumsq_for_mode<1>(ad, gd, L, prep, first, partial_sum);
+    case 2: return sumsq_for_mode<2>(ad, gd, L, prep, first, partial_sum);
+    case 3: return sumsq_for_mode<3>(ad, gd, L, prep, first, partial_sum);
+  }
+  return false;
+}
+
+// ------------------------------------------------------------------------------------
+// Synthetic data.  Element i = f(hash(seed, first_index + i)): integer hashing and exact integer
+// -> float conversions followed by one or two rounded float32 operations, so that a host
+// restatement produces the same bits for any slice of any buffer without materialising it.
+// ------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint64_t synth_hash(uint64_t seed, uint64_t idx) {
+  uint64_t z = seed + (idx + 1ull) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <int OD>
+__global__ __launch_bounds__(kThreads) void synth_kernel(void* __restrict__ out, uint64_t n, uint64_t seed,
+                                                         uint64_t first_index, int dist, float a, float b) {
+  for (uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kThreads) {
+    const uint64_t z = synth_hash(seed, first_index + i);
+    float x;
+    if (dist == MXOPT_SYNTH_UNIFORM) {
+      x = (float)(uint32_t)(z >> 40) * a;   // a = (hi - lo) / 2^24, b = lo
+      x = x + b;
+    } else {
+      // sum of four 16-bit uniforms, centred: a bell shape on [-131070, 131070] with an exactly known variance
+      const int32_t sum = (int32_t)((z & 0xffffu) + ((z >> 16) & 0xffffu) + ((z >> 32) & 0xffffu) + (z >> 48)) - 131070;
+      x = (float)sum * a;                    // a = sigma / sqrt((65536^2 - 1) / 3)
+      if (dist == MXOPT_SYNTH_NORMAL_OUTLIERS && synth_hash(seed ^ 0xA5A5A5A5A5A5A5A5ull, first_index + i) % 100ull == 0ull)
+        x = x * b;                           // b = outlier multiplier
+    }
+    Elem<OD>::store(out, i, x);
+  }
+}
+
+bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
+                  uint32_t grid, hipStream_t stream) {
+  switch (od) {
+    case MXOPT_F32: hipLaunchKernelGGL(synth_kernel<MXOPT_F32>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+    case MXOPT_BF16: hipLaunchKernelGGL(synth_kernel<MXOPT_BF16>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+    case MXOPT_F16: hipLaunchKernelGGL(synth_kernel<MXOPT_F16>, dim3(grid), dim3(kThreads), 0, stream, out, n, seed, first_index, dist, a, b); return true;
+  }
+  return false;
+}
+
+void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t npartials, double max_norm,
+                        int has_max, int clip_mode, mxopt_norm_result* d_out) {
+  hipLaunchKernelGGL(norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, partial_sum, npartials, max_norm,
+                     has_max, clip_mode, d_out);
+}
+
+}  // namespace mxopt
