@@ -33,3 +33,16 @@ def test_functions_and_structs_match_the_ctypes_side():
         body = re.search(r"pub struct %s \{(.*?)\n\}" % name, text, flags=re.S).group(1)
         fields = [f.replace("r#", "") for f in re.findall(r"pub (\S+):", body)]
         assert fields == [f[0] for f in ct._fields_], name
+
+
+def test_pointer_types_are_translated_with_their_constness():
+    sys.path.insert(0, os.path.dirname(GEN))
+    import gen_rust_sys as G
+    opaque, structs = {"mxopt_ctx"}, {"mxopt_array"}
+    cases = {"const char* const*": "*const *const c_char", "const float* const*": "*const *const f32",
+             "mxopt_ctx**": "*mut *mut mxopt_ctx", "const mxopt_ctx*": "*const mxopt_ctx", "void*": "*mut c_void",
+             "const void* const*": "*const *const c_void", "float**": "*mut *mut f32", "uint64_t": "u64",
+             "const mxopt_array*": "*const mxopt_array", "unsigned long long": "u64", "size_t": "usize",
+             "const double*": "*const f64", "int64_t*": "*mut i64", "char*": "*mut c_char"}
+    for c, want in cases.items():
+        assert G.rust_type(c, opaque, structs) == want, c
