@@ -47,3 +47,16 @@ def test_key_function_matches_the_library():
     for args in ((0x5EED0001, 5, 0, 0, 0), (0x5EED0001, 5, 9, 3, 398), (2 ** 64 - 1, 0, 2 ** 31, 65535, 2 ** 32)):
         assert lib.mxopt_synthetic_key(*[C.c_uint64(v & (2 ** 64 - 1)) for v in args]) == O.synthetic_key(*args), args
     assert O.synthetic_key(1, 2, 3, 4, 5) != O.synthetic_key(1, 2, 3, 4, 6)
+
+
+def test_known_answers_freeze_the_generator():
+    """The definition must never drift: benchmark inputs of earlier runs stay reproducible.  Six elements of
+    each distribution from one key, as bit patterns (the fifth element of the second row is a x100 outlier)."""
+    key = O.synthetic_key(0x5EED0001, 5, 0, 3, 17)
+    assert key == 0xF5409BCF2ED3FA2A
+    normal = O.synthetic(6, "f32", key, O.SYNTH_NORMAL, 1e-3, 0.0, first_index=1000003)
+    assert [int(v) for v in normal.view(np.uint32)] == [0xBA5FD61E, 0xB8FC2194, 0xB9FD7291, 0x3A934168, 0x39DCF0BE, 0x3A68FB4B]
+    outliers = O.synthetic(6, "bf16", key, O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0, first_index=1000003)
+    assert [int(v) for v in outliers] == [0xBA60, 0xB8FC, 0xB9FD, 0x3A93, 0x3D2D, 0x3A69]
+    uniform = O.synthetic(6, "f32", key, O.SYNTH_UNIFORM, 0.9, 1.1, first_index=1000003)
+    assert [int(v) for v in uniform.view(np.uint32)] == [0x3F66DAB6, 0x3F7799CB, 0x3F6EC035, 0x3F848C60, 0x3F799660, 0x3F6C8862]
