@@ -23,6 +23,10 @@
  * may be used from different threads.  Kernels are enqueued on the context's stream;
  * no call synchronises with the host except mxopt_synchronize / mxopt_read_*.
  *
+ * Logging: the environment variable MXOPT_LOG (read once per process) = "error" prints every refused
+ * call to stderr, "debug" also one line per launch group, table change and engine decision (the
+ * counterpart of the reference's MLX_NODE_LOG filter, crates/mlx-core/src/tracing.rs:3-21).
+ *
  * HIP graphs: the kernel entry points (mxopt_adam ... mxopt_norm_with_pending_list) only launch
  * kernels -- no allocation, copy or memset -- once the first reduction call on a context has
  * allocated its per-workgroup partials buffer, so a step may be recorded into a graph after

@@ -4,6 +4,9 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <new>
@@ -19,9 +22,30 @@ namespace mxopt {
 
 static thread_local std::string g_thread_error;
 
+int log_level() {
+  static const int level = [] {
+    const char* e = std::getenv("MXOPT_LOG");
+    if (!e) return 0;
+    if (!std::strcmp(e, "debug") || !std::strcmp(e, "trace")) return 2;
+    if (!std::strcmp(e, "error") || !std::strcmp(e, "warn") || !std::strcmp(e, "info")) return 1;
+    return 0;
+  }();
+  return level;
+}
+
+void log_line(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  std::fprintf(stderr, "mxopt: %s\n", buf);
+}
+
 int fail(mxopt_ctx* ctx, int code, const std::string& msg) {
   if (ctx) ctx->err = msg;
   g_thread_error = msg;
+  if (log_level() >= 1) log_line("error %d: %s", code, msg.c_str());
   return code;
 }
 
@@ -169,6 +193,8 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
     Launch L = make_launch(ctx, t, g, want || !(mode == 2 && first) || ctx->persistent != 0);
     if (mode != 2) L.nontemporal = ctx->nontemporal_reduce;
     const int ad = mode == 0 ? g.gd : g.god;
+    MXOPT_DEBUG("%s (reduction mode %d%s): %s, %u chunks in %u workgroups", op, mode, first ? ", first" : "",
+                dtype_names(g).c_str(), g.nchunks, L.grid);
     if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr))
       return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
     int rc = check_launch(ctx, op);
@@ -184,6 +210,8 @@ static int run_update(mxopt_ctx* ctx, const mxopt_table* t, const char* op, F&& 
   DeviceGuard guard(ctx->device);
   for (const Group& g : t->groups) {
     Launch L = make_launch(ctx, t, g, ctx->persistent != 0);
+    MXOPT_DEBUG("%s: %s, %u chunks in %u workgroups, %zu tensors / %llu elements in the table", op,
+                dtype_names(g).c_str(), g.nchunks, L.grid, t->host.size(), (unsigned long long)t->total_elems);
     if (!launch_one(g, L)) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
     int rc = check_launch(ctx, op);
     if (rc) return rc;
@@ -351,6 +379,8 @@ int mxopt_hbm_spread_begin(mxopt_ctx* ctx, size_t block_bytes, int keep_one_in, 
     if (i % (size_t)keep_one_in == 0) s->kept.push_back(all[i]);
     else (void)hipFree(all[i]);
   }
+  MXOPT_DEBUG("placement window: %zu blocks of %zu MiB taken (%zu MiB were free), %zu kept until the window closes",
+              all.size(), block_bytes >> 20, free_b >> 20, s->kept.size());
   *out = s;
   return MXOPT_OK;
 }
@@ -435,6 +465,8 @@ int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxo
     delete t;
     return hip_fail(ctx, e, "mxopt_table_build");
   }
+  MXOPT_DEBUG("table built: %zu tensors, %llu elements, %llu chunks, %zu dtype group(s)", n,
+              (unsigned long long)t->total_elems, (unsigned long long)t->num_chunks, t->groups.size());
   *out = t;
   return MXOPT_OK;
 }
@@ -474,10 +506,14 @@ int mxopt_table_set_step_scalars(mxopt_table* t, const float* bc1, const float* 
   return upload_descriptors(t);
 }
 
-int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n) {
-  if (!t || (n && !tensors)) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: null argument");
+}  // extern "C"
+
+int mxopt::table_retarget_quiet(mxopt_table* t, const mxopt_tensor* tensors, size_t n, std::string* why) {
   mxopt_ctx* ctx = t->ctx;
-  if (n != t->host.size()) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: different number of tensors");
+  if (n != t->host.size()) {
+    *why = "different number of tensors";
+    return MXOPT_ERR_INVALID_ARG;
+  }
   std::vector<DevTensor> dev(n);
   for (size_t i = 0; i < n; ++i) {
     const mxopt_tensor& a = t->host[i];
@@ -488,13 +524,27 @@ int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n) 
                       (!a.g_out || a.g_out_dtype == b.g_out_dtype);
     fill_dev_tensor(b, dev[i]);
     // The chunk list depends on the head and on which path the tensor takes.
-    if (!same || dev[i].head != t->dev[i].head || ((dev[i].flags ^ t->dev[i].flags) & kTfUnaligned))
-      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: tensor " + std::to_string(i) + " has a different layout");
+    if (!same || dev[i].head != t->dev[i].head || ((dev[i].flags ^ t->dev[i].flags) & kTfUnaligned)) {
+      *why = "tensor " + std::to_string(i) + " has a different layout";
+      return MXOPT_ERR_INVALID_ARG;
+    }
   }
   DeviceGuard guard(ctx->device);
   t->host.assign(tensors, tensors + n);
   t->dev.swap(dev);
+  MXOPT_DEBUG("table retargeted: %zu tensors keep their chunk list", n);
+  why->clear();
   return upload_descriptors(t);
+}
+
+extern "C" {
+
+int mxopt_table_retarget(mxopt_table* t, const mxopt_tensor* tensors, size_t n) {
+  if (!t || (n && !tensors)) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_table_retarget: null argument");
+  std::string why;
+  const int rc = table_retarget_quiet(t, tensors, n, &why);
+  if (rc && !why.empty()) return fail(t->ctx, rc, "mxopt_table_retarget: " + why);
+  return rc;
 }
 
 int mxopt_table_set_pending(mxopt_table* t, int k, const void* const* streams, int dtype) {
@@ -861,6 +911,8 @@ int mxopt_norm_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxo
     L.grid = list_grid(g.nchunks);
     L.nontemporal = ctx->nontemporal_reduce;
     attach_pending(t, L);
+    MXOPT_DEBUG("%s: %s, %d pending stream(s), %u chunks in %u workgroups", op, dtype_names(g).c_str(), t->pending_k,
+                g.nchunks, L.grid);
     if (!launch_sumsq_list(g.gd, t->pending_k ? t->pending_dtype : g.gd, L, dp, ctx->d_partial_sum + offset))
       return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
     rc = check_launch(ctx, op);

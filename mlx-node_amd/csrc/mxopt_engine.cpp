@@ -157,6 +157,9 @@ int apply_accumulated(mxopt_engine* e, double lr, double weight_decay, const mxo
 }
 
 void end_cycle(mxopt_engine* e) {
+  // the reference's debug!("Applied gradients with lr ...") (grpo/engine.rs:684)
+  MXOPT_DEBUG("%s engine: applied gradients with lr %g%s", e->cfg.kind == MXOPT_ENGINE_GRPO ? "GRPO" : "SFT",
+              e->cfg.learning_rate, e->cfg.defer_accumulation ? " (deferred accumulation)" : "");
   for (Slot& s : e->slots) s.in_acc = false;
   e->have_acc = false;
   e->micro_step = 0;
@@ -264,6 +267,8 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     if ((rc = mxopt_read_norm_result(ctx, d_result, &h))) return rc;
   }
   if (h.nonfinite) {  // engine.rs:571-633: skip the whole micro-batch, touch nothing
+    MXOPT_DEBUG("GRPO engine: NaN/Inf gradient, micro-batch skipped (%llu so far)",
+                (unsigned long long)e->nan_gradient_count + 1);
     e->nan_gradient_count += 1;
     e->consecutive_nan_count += 1;
     if (e->nan_gradient_count >= max_nan(e)) {

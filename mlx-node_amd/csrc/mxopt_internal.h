@@ -14,7 +14,21 @@
 namespace mxopt {
 
 int fail(mxopt_ctx* ctx, int code, const std::string& msg);
+// mxopt_table_retarget without the error report: a refusal because the layout differs sets *why and
+// leaves the table as it was; *why stays empty when the descriptor upload itself failed.
+int table_retarget_quiet(mxopt_table* t, const mxopt_tensor* tensors, size_t n, std::string* why);
 int hip_fail(mxopt_ctx* ctx, hipError_t e, const char* what);
+
+// Logging to stderr, filtered by the environment variable MXOPT_LOG (read once): unset or "off" = nothing,
+// "error" = refused calls, "debug" = also one line per launch group, table change and engine decision.
+// The counterpart of the reference's tracing subscriber filtered by MLX_NODE_LOG
+// (crates/mlx-core/src/tracing.rs:3-21) and of its debug!("Applied gradients ...") (grpo/engine.rs:684).
+int log_level();  // 0 off, 1 error, 2 debug
+void log_line(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+#define MXOPT_DEBUG(...)                                      \
+  do {                                                        \
+    if (::mxopt::log_level() >= 2) ::mxopt::log_line(__VA_ARGS__); \
+  } while (0)
 
 #define HIP_TRY(ctx, call)                                            \
   do {                                                                \

@@ -60,9 +60,9 @@ int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** 
   // The least recently used candidate goes first so that alternating buffer sets each keep a table.
   for (size_t i = 0; i < cache.size(); ++i) {
     if (cache[i].key.size() != key.size() || key.empty()) continue;
-    const std::string saved = ctx->err;
-    if (mxopt_table_retarget(cache[i].table, rows.data(), rows.size()) != MXOPT_OK) {
-      ctx->err = saved;  // a layout mismatch here is not the caller's error
+    std::string why;  // a layout mismatch here is not the caller's error: try the next candidate
+    if (const int rc = table_retarget_quiet(cache[i].table, rows.data(), rows.size(), &why)) {
+      if (why.empty()) return rc;  // the descriptor upload failed and has said so
       continue;
     }
     mxopt_ctx::CachedTable hit = std::move(cache[i]);
@@ -368,10 +368,9 @@ static int prepare_many(mxopt_optimizer* opt, size_t n, const char* const* param
     // chunk list and swap the pointers; anything else is a new table.
     bool moved = false;
     if (opt->many_table) {
-      const std::string saved = ctx->err;
-      moved = mxopt_table_retarget(opt->many_table, rows.data(), rows.size()) == MXOPT_OK;
+      std::string why;
+      moved = table_retarget_quiet(opt->many_table, rows.data(), rows.size(), &why) == MXOPT_OK;
       if (!moved) {
-        ctx->err = saved;
         mxopt_table_destroy(opt->many_table);
         opt->many_table = nullptr;
       }
