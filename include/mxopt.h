@@ -286,6 +286,12 @@ int mxopt_norm_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxo
 int mxopt_adam_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_adam_hp* hp,
                                  const mxopt_grad_prep* prep);
 
+/* mxopt_sgd and mxopt_rmsprop on the gradient prep(g + x0 + ...); p_out must have p's dtype. */
+int mxopt_sgd_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp,
+                                const mxopt_grad_prep* prep);
+int mxopt_rmsprop_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* hp,
+                                    const mxopt_grad_prep* prep);
+
 /* mxopt_sgd_plain on the gradient prep(g + x0 + ...), which is float32 (the sum promotes);
  * the SFT engine's boundary (sft/engine.rs:293-371) without its accumulation buffer. */
 int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,

@@ -69,8 +69,10 @@ int mxopt_optimizer_update_single(mxopt_optimizer* opt, const char* param_name, 
 /* The same as calling update_single for i = 0 .. n-1 in that order (so with bias correction
  * tensor i sees t = step + i + 1), but one launch per dtype group for the whole list.  The
  * table is cached while the same buffers are passed.  `prep` (nullable) applies fused gradient
- * pre-processing (clip scale etc.).  No counterpart in the reference; it is what its callers'
- * `for (name, param) in params { opt.update_single(..) }` loops collapse into. */
+ * pre-processing (clip scale etc.).  SGD with momentum refuses prep->d_skip_if_nonzero while a
+ * parameter of the list has no velocity yet: the first step stores it, and the host cannot know
+ * afterwards whether a conditional one ran.  No counterpart in the reference; it is what its
+ * callers' `for (name, param) in params { opt.update_single(..) }` loops collapse into. */
 int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* const* param_names,
                                 const mxopt_array* params, const mxopt_array* grads, const mxopt_array* outs,
                                 const mxopt_grad_prep* prep);
@@ -80,10 +82,10 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
  * right in float32 -- the sum k-1 calls of Qwen3Model::accumulate_gradients (model.rs:2217-2243)
  * would have left in a float32 buffer -- then `prep`, then, when max_norm >= 0, the clip factor of
  * GradientUtils::clip_grad_norm (optimizers/mod.rs:67-107; clip_mode as in mxopt_global_norm) of
- * that gradient's global norm, then the Adam/AdamW update with update_many's per-call step
- * counting.  Two launches per dtype group, no accumulation buffer, no host synchronisation.
+ * that gradient's global norm, then the optimizer's own update (any of the four kinds) with
+ * update_many's per-call step counting.  Two launches per dtype group, no accumulation buffer, no host synchronisation.
  * 1 <= k <= MXOPT_MAX_PENDING + 1; micro-batches 2..k share one dtype, the first has it or is
- * float32; outs[i] has params[i]'s dtype (it may be params[i] itself); Adam and AdamW only.
+ * float32; outs[i] has params[i]'s dtype (it may be params[i] itself).
  * d_norm (nullable, device memory) receives norm, clip factor and the non-finite flag; pass
  * prep->d_skip_if_nonzero = &d_norm->nonfinite to leave everything untouched on a NaN/Inf gradient. */
 int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, const char* const* param_names,

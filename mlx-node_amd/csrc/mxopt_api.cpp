@@ -766,6 +766,34 @@ int mxopt_adam_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxo
   });
 }
 
+int mxopt_sgd_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_sgd_hp* hp,
+                                const mxopt_grad_prep* prep) {
+  const char* op = "mxopt_sgd_with_pending_list";
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": hp is NULL");
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | (hp->has_momentum ? kNeedV : 0), op);
+  if (rc) return rc;
+  if (hp->nesterov && !hp->has_momentum)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "Nesterov momentum requires momentum > 0 and dampening = 0");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, op, [&](const Group& g, Launch& L) {
+    attach_pending(t, L);
+    return launch_sgd_list(g.pd, g.gd, g.pod, t->pending_k ? t->pending_dtype : g.gd, L, *hp, dp);
+  });
+}
+
+int mxopt_rmsprop_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, const mxopt_rmsprop_hp* hp,
+                                    const mxopt_grad_prep* prep) {
+  const char* op = "mxopt_rmsprop_with_pending_list";
+  int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG | kNeedV, op);
+  if (rc) return rc;
+  if (!hp) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": hp is NULL");
+  const DevPrep dp = make_prep(prep);
+  return run_update(ctx, t, op, [&](const Group& g, Launch& L) {
+    attach_pending(t, L);
+    return launch_rmsprop_list(g.pd, g.gd, g.pod, t->pending_k ? t->pending_dtype : g.gd, L, *hp, dp);
+  });
+}
+
 int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
                                       double weight_decay, const mxopt_grad_prep* prep) {
   int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG, "mxopt_sgd_plain_with_pending_list");

@@ -50,6 +50,9 @@ bool launch_sumsq(int mode, int ad, int gd, const Launch& L, const DevPrep& prep
 bool launch_adam_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep);
 bool launch_sgd_plain_list(int pd, int gd, int od, int xd, const Launch& L, float lr_p, float wd, int has_wd,
                            const DevPrep& prep);
+bool launch_sgd_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_sgd_hp& hp, const DevPrep& prep);
+bool launch_rmsprop_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_rmsprop_hp& hp,
+                         const DevPrep& prep);
 bool launch_sumsq_list(int gd, int xd, const Launch& L, const DevPrep& prep, double* partial_sum);
 bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
                   uint32_t grid, hipStream_t stream);

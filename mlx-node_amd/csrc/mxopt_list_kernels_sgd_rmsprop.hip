@@ -1,0 +1,27 @@
+// mxopt kernels for gfx950, part 4: deferred accumulation for SGD with momentum and RMSprop.
+#include "mxopt_list_kernels.h"
+
+namespace mxopt {
+
+bool launch_sgd_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_sgd_hp& hp, const DevPrep& prep) {
+  if (od != pd) return false;
+  switch (pd) {
+    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, SgdMath{hp}, prep);
+    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, SgdMath{hp}, prep);
+    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, SgdMath{hp}, prep);
+  }
+  return false;
+}
+
+bool launch_rmsprop_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_rmsprop_hp& hp,
+                         const DevPrep& prep) {
+  if (od != pd) return false;
+  switch (pd) {
+    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, RmspropMath{hp}, prep);
+    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, RmspropMath{hp}, prep);
+    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, RmspropMath{hp}, prep);
+  }
+  return false;
+}
+
+}  // namespace mxopt

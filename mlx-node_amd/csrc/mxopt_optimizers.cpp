@@ -341,8 +341,8 @@ int mxopt_optimizer_update_single(mxopt_optimizer* opt, const char* param_name, 
 // Rows, per-call step scalars and the cached table of one batched update; shared by update_many and
 // update_many_accumulated.  On return opt->many_table describes `rows` and *hp holds the coefficients.
 static int prepare_many(mxopt_optimizer* opt, size_t n, const char* const* param_names, const mxopt_array* params,
-                        const mxopt_array* grads, const mxopt_array* outs, std::vector<StateEntry*>* states_out,
-                        Hp* hp_out) {
+                        const mxopt_array* grads, const mxopt_array* outs, const mxopt_grad_prep* prep,
+                        std::vector<StateEntry*>* states_out, Hp* hp_out) {
   mxopt_ctx* ctx = opt->ctx;
   std::vector<mxopt_tensor> rows(n);
   std::vector<StateEntry*>& states = *states_out;
@@ -356,6 +356,14 @@ static int prepare_many(mxopt_optimizer* opt, size_t n, const char* const* param
       return rc;
     }
   }
+  // A first momentum step writes the velocity that every later step reads.  Whether a conditional
+  // update ran is known on the device only, so the host could not tell afterwards which kind of step
+  // comes next.
+  if (prep && prep->d_skip_if_nonzero)
+    for (const mxopt_tensor& r : rows)
+      if (r.flags & MXOPT_TF_FIRST)
+        return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                    "SGD with momentum: the first update of a parameter cannot be conditional (prep->d_skip_if_nonzero)");
   int rc = make_hp(opt, &hp);
   if (rc) return rc;
   // Same buffers as last time?  Then only the per-step scalars change.
@@ -403,7 +411,7 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
   if (n && (!param_names || !params || !grads || !outs)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "update_many: null argument");
   std::vector<StateEntry*> states;
   Hp hp;
-  int rc = prepare_many(opt, n, param_names, params, grads, outs, &states, &hp);
+  int rc = prepare_many(opt, n, param_names, params, grads, outs, prep, &states, &hp);
   if (rc) return rc;
   switch (opt->kind) {
     case Kind::Adam:
@@ -424,7 +432,6 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
   const char* op = "update_many_accumulated";
   if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": optimizer is NULL");
   mxopt_ctx* ctx = opt->ctx;
-  if (!is_adam(opt)) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": Adam and AdamW only");
   if (k < 1 || k > (size_t)MXOPT_MAX_PENDING + 1)
     return fail(ctx, MXOPT_ERR_INVALID_ARG,
                 std::string(op) + ": between 1 and " + std::to_string(MXOPT_MAX_PENDING + 1) + " micro-batches");
@@ -448,7 +455,7 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
   const int64_t step_before = opt->step;
   std::vector<StateEntry*> states;
   Hp hp;
-  int rc = prepare_many(opt, n, param_names, params, grads, outs, &states, &hp);
+  int rc = prepare_many(opt, n, param_names, params, grads, outs, prep, &states, &hp);
   if (rc) return rc;
   std::vector<const void*> streams((k - 1) * n);
   for (size_t j = 1; j < k; ++j)
@@ -462,10 +469,22 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
     if (!rc) rc = mxopt_norm_with_pending_list(ctx, opt->many_table, &local, max_norm, clip_mode, slot);
     local.d_scale = &slot->scale;
   }
-  if (!rc) rc = mxopt_adam_with_pending_list(ctx, opt->many_table, &hp.adam, &local);
+  if (!rc) {
+    switch (opt->kind) {
+      case Kind::Adam:
+      case Kind::AdamW: rc = mxopt_adam_with_pending_list(ctx, opt->many_table, &hp.adam, &local); break;
+      case Kind::Sgd: rc = mxopt_sgd_with_pending_list(ctx, opt->many_table, &hp.sgd, &local); break;
+      case Kind::Rmsprop: rc = mxopt_rmsprop_with_pending_list(ctx, opt->many_table, &hp.rms, &local); break;
+    }
+  }
   (void)mxopt_table_set_pending(opt->many_table, 0, nullptr, 0);
-  if (rc) opt->step = step_before;  // the update was not launched
-  return rc;
+  if (rc) {
+    opt->step = step_before;  // the update was not launched
+    return rc;
+  }
+  if (opt->kind == Kind::Sgd && opt->momentum != 0.0)
+    for (StateEntry* st : states) st->has_velocity = true;
+  return MXOPT_OK;
 }
 
 int mxopt_optimizer_reset(mxopt_optimizer* opt) {

@@ -95,6 +95,8 @@ SIGNATURES = {
     "mxopt_norm_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
                                                C.c_void_p]),
     "mxopt_adam_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
+    "mxopt_sgd_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
+    "mxopt_rmsprop_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),
     "mxopt_sgd_plain_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
                                                     C.POINTER(GradPrep)]),
     "mxopt_sgd_plain_with_pending_list_each": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,

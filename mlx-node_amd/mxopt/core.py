@@ -234,6 +234,16 @@ def _adam_with_pending_list(self, table: "Table", hp: L.AdamHp, prep: Optional[L
                                                   C.byref(prep) if prep else None), self.handle)
 
 
+def _sgd_with_pending_list(self, table: "Table", hp: L.SgdHp, prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_sgd_with_pending_list(self.handle, table.handle, C.byref(hp),
+                                                 C.byref(prep) if prep else None), self.handle)
+
+
+def _rmsprop_with_pending_list(self, table: "Table", hp: L.RmspropHp, prep: Optional[L.GradPrep] = None) -> None:
+    L.check(self.lib.mxopt_rmsprop_with_pending_list(self.handle, table.handle, C.byref(hp),
+                                                     C.byref(prep) if prep else None), self.handle)
+
+
 def _sgd_plain_with_pending_list(self, table: "Table", learning_rate: float, weight_decay: float = 0.0,
                                  prep: Optional[L.GradPrep] = None) -> None:
     L.check(self.lib.mxopt_sgd_plain_with_pending_list(self.handle, table.handle, learning_rate, weight_decay,
@@ -278,6 +288,8 @@ Context.accumulate_norm_only = _accumulate_norm_only
 Context.norm_with_pending_list = _norm_with_pending_list
 Context.adam_with_pending_list = _adam_with_pending_list
 Context.sgd_plain_with_pending_list = _sgd_plain_with_pending_list
+Context.sgd_with_pending_list = _sgd_with_pending_list
+Context.rmsprop_with_pending_list = _rmsprop_with_pending_list
 Context.accumulate_transformed = _accumulate_transformed
 Context.fill_synthetic = _fill_synthetic
 Context.sgd_plain_with_pending = _sgd_plain_with_pending

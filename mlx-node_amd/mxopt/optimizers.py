@@ -100,7 +100,7 @@ class _Optimizer:
                                 outs: Optional[Sequence[torch.Tensor]] = None, prep: Optional[L.GradPrep] = None,
                                 max_norm: float = -1.0, clip_mode: int = L.CLIP_ALWAYS_MULTIPLY,
                                 norm_out=None) -> List[torch.Tensor]:
-        """One Adam/AdamW step on the sum of `micro_batches` (added in registers, in order, in float32),
+        """One optimizer step on the sum of `micro_batches` (added in registers, in order, in float32),
         clipped to `max_norm` by its global norm when max_norm >= 0.  In place unless `outs` is given."""
         if outs is None:
             outs = list(params)

@@ -126,6 +126,82 @@ def test_adamw_over_deferred_micro_batches(mx, ctx, combo, k, layout):
     table.close()
 
 
+@pytest.mark.parametrize("which", ["sgd_first", "sgd_later", "sgd_nesterov", "rmsprop"])
+@pytest.mark.parametrize("combo", [("bf16", "bf16", "bf16"), ("f32", "f32", "f32"), ("bf16", "f32", "bf16"),
+                                   ("f16", "f16", "f16")], ids=lambda c: "-".join(c))
+@pytest.mark.parametrize("k", [1, 3, 6])
+@pytest.mark.parametrize("layout", ["aligned", "head", "elementwise"])
+def test_sgd_and_rmsprop_over_deferred_micro_batches(mx, ctx, which, combo, k, layout):
+    """The momentum-SGD and RMSprop kernels on g + x0 + ... with the clip factor taken from the device:
+    first step (velocity = gradient), a later step (velocity read), Nesterov, RMSprop with decay."""
+    pk, gk, xk = combo
+    seed = 3000 + 10 * k + len(layout)
+    off = {"aligned": {"f32": 0, "bf16": 0, "f16": 0}, "head": {"f32": 3, "bf16": 7, "f16": 7},
+           "elementwise": {"f32": 3, "bf16": 3, "f16": 3}}[layout]
+    kind_of = {np.dtype(np.float32): "f32", np.dtype(np.uint16): "bf16", np.dtype(np.float16): "f16"}
+
+    def place(a):
+        return to_dev(a, off[kind_of[a.dtype]])
+
+    ps = lists(seed, SIZES, pk, 0.02)
+    first = lists(seed + 1, SIZES, gk, 1e-3)
+    pending = [lists(seed + 2 + j, SIZES, xk, 1e-3) for j in range(k)]
+    v0 = [np.abs(a) for a in lists(seed + 20, SIZES, "f32", 1e-3)]   # RMSprop's average of squares is >= 0
+    dp = [place(p) for p in ps]
+    dg = [place(g) for g in first]
+    dx = [[place(g) for g in s] for s in pending]
+    dv = [place(v) for v in v0]
+    if which == "rmsprop":
+        ref = O.RMSprop(1e-2, 0.95, 1e-8, 1e-3)
+        hp, run, flags = mx.rmsprop_hp(1e-2, 0.95, 1e-8, 1e-3), ctx.rmsprop_with_pending_list, 0
+    else:
+        nesterov = which == "sgd_nesterov"
+        args = (0.05, 0.9, 0.0, 0.0, True) if nesterov else (0.05, 0.9, 1e-3, 0.1, False)
+        ref = O.SGD(*args)
+        hp, run = mx.sgd_hp(*args), ctx.sgd_with_pending_list
+        flags = mx.TF_FIRST if which == "sgd_first" else 0
+    if flags == 0:
+        for i in range(len(SIZES)):
+            ref.state[str(i)] = v0[i].copy()
+    table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v, flags=flags) for p, g, v in zip(dp, dg, dv)])
+    table.set_pending(dx)
+    res = ctx.norm_result()
+    ctx.norm_with_pending_list(table, res, max_norm=1e-2)
+    acc = oracle_sum(first, pending)
+    scale = device_scale(ctx, res, acc, 1e-2)
+    run(table, hp, mx.make_prep(scale=res))
+    for i, n in enumerate(SIZES):
+        want = to_param_dtype(ref.update_single(str(i), ps[i], acc[i] * scale), pk)
+        assert_bit_equal(to_host(dp[i]), want, f"p {i} (n={n})")
+        assert_bit_equal(to_host(dv[i]), ref.state[str(i)], f"v {i}")
+    for i in range(len(SIZES)):
+        assert_bit_equal(to_host(dg[i]), first[i], f"g {i}")
+        for j in range(k):
+            assert_bit_equal(to_host(dx[j][i]), pending[j][i], f"x{j} {i}")
+    table.close()
+
+
+def test_first_momentum_step_cannot_be_conditional(mx, ctx):
+    """The first SGD-with-momentum step stores the velocity every later step reads; the host cannot know
+    whether a device-side conditional update ran, so that combination is refused, and accepted afterwards."""
+    names, ps, gs = ["a", "b"], lists(7, [4096, 33], "f32", 0.02), lists(8, [4096, 33], "f32", 1e-3)
+    dp, dg = [to_dev(p) for p in ps], [to_dev(g) for g in gs]
+    res = ctx.norm_result()
+    opt = mx.SGD(0.05, 0.9, ctx=ctx)
+    with pytest.raises(mx.InvalidArg, match="cannot be conditional"):
+        opt.update_many(names, dp, dg, outs=dp, prep=mx.make_prep(skip_if_nonfinite=res))
+    for i in range(2):
+        assert_bit_equal(to_host(dp[i]), ps[i], "refused call changed a parameter")
+    opt.update_many(names, dp, dg, outs=dp)
+    opt.update_many_accumulated(names, dp, [dg, dg], prep=mx.make_prep(skip_if_nonfinite=res), max_norm=1.0, norm_out=res)
+    ref = O.SGD(0.05, 0.9)
+    cur = [ref.update_single(n, p, g) for n, p, g in zip(names, ps, gs)]
+    acc = oracle_sum(gs, [gs])
+    scale = device_scale(ctx, res, acc, 1.0)
+    for i, n in enumerate(names):
+        assert_bit_equal(to_host(dp[i]), ref.update_single(n, cur[i], acc[i] * scale), n)
+
+
 def test_deferred_equals_buffered_path_bit_for_bit(mx, ctx):
     """Four bf16 micro-batches: accumulate x3 + accumulate_norm_only + adam_with_pending (float32 buffer)
     against norm_with_pending_list + adam_with_pending_list (no buffer): same sum of squares (to float64
@@ -251,16 +327,26 @@ def test_set_pending_rejects_what_the_kernels_cannot_walk(mx, ctx):
     t.close()
 
 
+OPTIMIZERS = {
+    "adamw": (lambda mx, ctx: mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True, ctx=ctx),
+              lambda: O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True)),
+    "sgd": (lambda mx, ctx: mx.SGD(0.05, 0.9, 1e-3, 0.1, False, ctx=ctx), lambda: O.SGD(0.05, 0.9, 1e-3, 0.1, False)),
+    "sgd_nesterov": (lambda mx, ctx: mx.SGD(0.05, 0.9, 0.0, 0.0, True, ctx=ctx), lambda: O.SGD(0.05, 0.9, 0.0, 0.0, True)),
+    "sgd_plain": (lambda mx, ctx: mx.SGD(0.05, ctx=ctx), lambda: O.SGD(0.05)),
+    "rmsprop": (lambda mx, ctx: mx.RMSprop(1e-2, 0.95, 1e-8, 1e-3, ctx=ctx), lambda: O.RMSprop(1e-2, 0.95, 1e-8, 1e-3)),
+}
+
+
+@pytest.mark.parametrize("which", list(OPTIMIZERS))
 @pytest.mark.parametrize("kind", ["bf16", "f32"])
-def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind):
+def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind, which):
     """update_many_accumulated == accumulate_gradients (float32 buffer) k-1 times, clip_grad_norm,
     then update_single tensor by tensor, including the per-call step count under bias correction;
     two optimizer steps, the second with fresh buffers (table retargeted) and fewer micro-batches."""
     sizes = [3, 4096, 5000, 70001]
     names = [f"layers.{i}.w" for i in range(len(sizes))]
     ps = lists(41, sizes, kind, 0.02)
-    opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True, ctx=ctx)
-    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+    opt, ref = OPTIMIZERS[which][0](mx, ctx), OPTIMIZERS[which][1]()
     dp = [to_dev(p) for p in ps]
     res = ctx.norm_result()
     cur = ps
@@ -275,14 +361,20 @@ def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind):
             want = cast(ref.update_single(name, cur[i], acc[i] * scale), kind)
             assert_bit_equal(to_host(dp[i]), want, f"step {step} {name}")
             m, v = opt.state(name)
-            assert_bit_equal(to_host(m), ref.state[name][0], f"m {name}")
-            assert_bit_equal(to_host(v), ref.state[name][1], f"v {name}")
+            if which == "adamw":
+                assert_bit_equal(to_host(m), ref.state[name][0], f"m {name}")
+                assert_bit_equal(to_host(v), ref.state[name][1], f"v {name}")
+            elif which == "sgd_plain":
+                assert m is None and v is None
+            else:                              # velocity / running average of squares
+                assert m is None
+                assert_bit_equal(to_host(v), ref.state[name], f"v {name}")
             nxt.append(want)
         cur = nxt
-        assert opt.step == ref.step == (step + 1) * len(names)
+        if which == "adamw":
+            assert opt.step == ref.step == (step + 1) * len(names)
     # a refused call leaves the counter alone
     with pytest.raises(mx.InvalidArg, match="between 1 and 8"):
         opt.update_many_accumulated(names, dp, [dmicro[0]] * 9)
-    with pytest.raises(mx.InvalidArg, match="Adam and AdamW only"):
-        mx.SGD(0.1, ctx=ctx).update_many_accumulated(names, dp, dmicro)
-    assert opt.step == 3 * len(names)
+    if which == "adamw":
+        assert opt.step == 3 * len(names)

@@ -88,8 +88,6 @@ def test_random_optimizer_sequences(mx, tmp_path_factory, kind, bf16, g_bf16, op
             for k in names:
                 ref_step(k, gs[k])
         elif op == "accumulated":
-            if not adam_like:
-                continue
             names = [k for k in SIZES if rng.random() < 0.7] or ["embed"]
             n_micro = int(rng.integers(1, 9))
             micro = [{k: grad(k) for k in names} for _ in range(n_micro)]
