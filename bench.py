@@ -398,7 +398,9 @@ class Workload:
         defer = bool(self.args.defer)
         # deferred accumulation reads every micro-batch of the cycle at the end: they must all be resident
         self.micro = [dict(zip(self.names, self.g))]
-        for _ in range(self.n_micro - 1 if defer else 0):
+        # (with more than eight in a cycle the engine adds the oldest into its float32 buffers as later ones
+        # arrive, so eight buffers used in turn are enough)
+        for _ in range(min(self.n_micro, mx.MAX_PENDING + 1) - 1 if defer else 0):
             self.micro.append(dict(zip(self.names, self._randn_list(bf, 1e-3))))
         if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
             self.engine = mx.GRPOEngineOptimizerSide(params, learning_rate=1e-6, gradient_accumulation_steps=N,
@@ -428,6 +430,15 @@ class Workload:
         self.step_bytes_per_elem = (self.bytes_per_elem.get("micro_batch_first", 0) +
                                     (N - 2) * self.bytes_per_elem.get("micro_batch", 0) +
                                     self.bytes_per_elem["micro_batch_apply"])
+        if defer and N > mx.MAX_PENDING + 1:
+            # the ninth micro-batch moves the two oldest into the float32 buffers (6 + 10 B), every later one
+            # one more (10 B); the applying call reads that buffer and seven deferred streams
+            spill = 6 + 10 * (N - mx.MAX_PENDING - 1)
+            norms = 2 * N if kind == "grpo" else 4 + 2 * mx.MAX_PENDING
+            apply = 4 + 2 * mx.MAX_PENDING + 4
+            self.bytes_per_elem = {"micro_batch_apply": apply + (2 if kind == "grpo" else norms)}
+            self.step_bytes_per_elem = spill + norms + apply
+            self.note += "; more than eight micro-batches: the oldest are added into float32 buffers as later ones arrive"
         self.dominant = "micro_batch_apply"
         self.dtype = "f32"
         self.storage = ("bf16 parameters and gradients, no accumulation buffer" if defer

@@ -301,10 +301,12 @@ int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, doub
  * gradient = prep_0(g) + prep_1(x0) + ..., where prep_j is `prep` (d_scale ignored) with the clip factor
  * read from d_scales[j] (k + 1 device pointers, or all NULL for no factor) -- the GRPO engine's
  * "clamp, clip by this micro-batch's own norm, accumulate" (grpo/engine.rs:636-661) followed by its
- * apply_gradients (:666-692), without the accumulation buffer. */
+ * apply_gradients (:666-692), without the accumulation buffer.  first_is_sum != 0: tensor.g is a
+ * float32 buffer into which earlier micro-batches were added after their own pre-processing (more
+ * micro-batches than streams); it is added as it is and d_scales[0] must be NULL. */
 int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
                                            double weight_decay, const mxopt_grad_prep* prep,
-                                           const float* const* d_scales);
+                                           const float* const* d_scales, int first_is_sum);
 
 /* ---- global norm ------------------------------------------------------------------ */
 

@@ -57,11 +57,13 @@ typedef struct mxopt_engine_config {
                                           registers (float32, arrival order: the numbers of the float32
                                           buffer, bit for bit).  The caller keeps every gradient buffer of
                                           a cycle alive and unchanged until the call that applies them
-                                          (or flush_gradients / reset) has returned.  Needs
-                                          gradient_accumulation_steps <= MXOPT_MAX_PENDING + 1, the same
-                                          gradient names in every micro-batch of a cycle, SFT:
-                                          accumulate_in_f32 = 1, GRPO: apply = SGD.  No counterpart in
-                                          the reference. */
+                                          (or flush_gradients / reset) has returned.  With more than
+                                          MXOPT_MAX_PENDING + 1 micro-batches in a cycle the oldest ones
+                                          are added into a float32 buffer as the later ones arrive (their
+                                          buffers are free again after that call); the last
+                                          MXOPT_MAX_PENDING stay deferred.  Needs the same gradient names
+                                          in every micro-batch of a cycle, SFT: accumulate_in_f32 = 1,
+                                          GRPO: apply = SGD.  No counterpart in the reference. */
 } mxopt_engine_config;
 
 /* The reference's defaults for `kind` (GRPOEngineConfig::default, SftEngineConfig::default). */

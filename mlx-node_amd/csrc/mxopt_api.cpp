@@ -811,7 +811,7 @@ int mxopt_sgd_plain_with_pending_list(mxopt_ctx* ctx, const mxopt_table* t, doub
 
 int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t, double learning_rate,
                                            double weight_decay, const mxopt_grad_prep* prep,
-                                           const float* const* d_scales) {
+                                           const float* const* d_scales, int first_is_sum) {
   const char* op = "mxopt_sgd_plain_with_pending_list_each";
   int rc = require(ctx, t, kNeedP | kNeedPOut | kNeedG, op);
   if (rc) return rc;
@@ -820,13 +820,20 @@ int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t,
   dp.d_scale = nullptr;
   dp.flags |= kPrepEachStream;
   StreamScales sc{};
+  const int from = first_is_sum ? 1 : 0;
+  if (first_is_sum) {
+    if (d_scales[0]) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of prepared micro-batches has no clip factor");
+    for (const Group& g : t->groups)
+      if (g.gd != MXOPT_F32) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of micro-batches is float32");
+    dp.flags |= kPrepFirstIsSum;
+  }
   int with = 0;
-  for (int j = 0; j <= t->pending_k; ++j) {
+  for (int j = from; j <= t->pending_k; ++j) {
     sc.s[j] = d_scales[j];
     with += d_scales[j] != nullptr;
   }
-  if (with != 0 && with != t->pending_k + 1)
-    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": either every stream has a clip factor or none");
+  if (with != 0 && with != t->pending_k + 1 - from)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": either every micro-batch has a clip factor or none");
   const float lr32 = (float)learning_rate;
   const float wd32 = (float)weight_decay;
   const int has_wd = weight_decay > 0.0;

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -48,6 +49,11 @@ struct mxopt_engine {
   // entry belongs to slot held_slots[c] (the order of the cycle's first micro-batch).
   std::vector<size_t> held_slots;
   std::vector<std::vector<mxopt_array>> held;
+  // More micro-batches than the kernels have streams for: the oldest ones have been added into the
+  // slots' float32 buffers, which then stand in entry 0 (held_is_sum).  held_result[j]: which of the
+  // device norm slots holds entry j's clip factor (GRPO), -1 for the sum.
+  bool held_is_sum = false;
+  std::vector<int> held_result;
 };
 
 namespace {
@@ -165,6 +171,8 @@ void end_cycle(mxopt_engine* e) {
   e->micro_step = 0;
   e->held.clear();
   e->held_slots.clear();
+  e->held_result.clear();
+  e->held_is_sum = false;
 }
 
 // ---- deferred accumulation ---------------------------------------------------------------
@@ -213,6 +221,70 @@ int defer_record(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_ar
   return MXOPT_OK;
 }
 
+constexpr int kResultSlots = MXOPT_MAX_PENDING + 2;  // every held micro-batch and the one that arrives
+
+// A device norm slot that no held micro-batch uses.
+int free_result_slot(const mxopt_engine* e) {
+  for (int slot = 0; slot < kResultSlots; ++slot)
+    if (std::find(e->held_result.begin(), e->held_result.end(), slot) == e->held_result.end()) return slot;
+  return kResultSlots - 1;  // not reached: at most MXOPT_MAX_PENDING + 1 entries are held
+}
+
+mxopt_grad_prep grpo_clamp(const mxopt_engine* e) {
+  const double clip_value = e->cfg.has_gradient_clip_value ? e->cfg.gradient_clip_value : 1.0;  // grpo/engine.rs:636
+  mxopt_grad_prep prep = no_prep();
+  prep.has_clamp_pre = 1;
+  prep.pre_lo = (float)(-clip_value);
+  prep.pre_hi = (float)clip_value;
+  return prep;
+}
+
+// Every stream is taken and one more micro-batch is about to be held: the two oldest entries become
+// one.  Entry 0 is copied (GRPO: clamped and clipped by its own factor) into the slots' float32
+// buffers unless it is such a sum already, entry 1 is added to it the same way -- the additions the
+// buffered path makes, in the same order -- and the buffers take the place of entry 0.
+int defer_spill(mxopt_engine* e) {
+  mxopt_ctx* ctx = e->ctx;
+  const size_t n = e->held_slots.size();
+  const bool grpo = e->cfg.kind == MXOPT_ENGINE_GRPO;
+  for (size_t c = 0; c < n; ++c) {
+    int rc = ensure_acc(e, e->slots[e->held_slots[c]], MXOPT_F32);
+    if (rc) return rc;
+  }
+  for (size_t j = e->held_is_sum ? 1 : 0; j < 2; ++j) {
+    if (n == 0) break;
+    std::vector<mxopt_tensor> rows(n, blank_tensor());
+    for (size_t c = 0; c < n; ++c) {
+      const Slot& s = e->slots[e->held_slots[c]];
+      rows[c].g = e->held[j][c].data; rows[c].g_dtype = (uint8_t)e->held[j][c].dtype;
+      rows[c].g_out = s.acc; rows[c].g_out_dtype = MXOPT_F32;
+      rows[c].n = s.param.n;
+    }
+    mxopt_table* t = nullptr;
+    int rc = cached_table(ctx, rows, &t);
+    if (rc) return rc;
+    if (grpo) {
+      mxopt_grad_prep prep = grpo_clamp(e);
+      if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result[e->held_result[j]].scale;
+      rc = mxopt_accumulate_transformed(ctx, t, j == 0, &prep);
+    } else {
+      rc = mxopt_accumulate(ctx, t, j == 0, nullptr, -1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, nullptr);
+    }
+    if (rc) return rc;
+  }
+  MXOPT_DEBUG("%s engine: deferred accumulation spilled the oldest micro-batch into the float32 buffers",
+              grpo ? "GRPO" : "SFT");
+  for (size_t c = 0; c < n; ++c) {
+    const Slot& s = e->slots[e->held_slots[c]];
+    e->held[0][c] = mxopt_array{s.acc, s.param.n, MXOPT_F32};
+  }
+  e->held_is_sum = true;
+  e->held_result[0] = -1;
+  e->held.erase(e->held.begin() + 1);
+  e->held_result.erase(e->held_result.begin() + 1);
+  return MXOPT_OK;
+}
+
 // Table over the held columns: parameters updated in place, g = the first micro-batch, the later ones
 // attached as pending streams.
 int defer_table(mxopt_engine* e, mxopt_table** out) {
@@ -242,15 +314,13 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
                      mxopt_engine_metrics* out) {
   mxopt_ctx* ctx = e->ctx;
   const size_t n = idx.size();
-  const double clip_value = e->cfg.has_gradient_clip_value ? e->cfg.gradient_clip_value : 1.0;  // engine.rs:636
-  mxopt_grad_prep prep = no_prep();
-  prep.has_clamp_pre = 1;
-  prep.pre_lo = (float)(-clip_value);
-  prep.pre_hi = (float)clip_value;
+  mxopt_grad_prep prep = grpo_clamp(e);
   mxopt_norm_result h;
   std::memset(&h, 0, sizeof h);
   h.scale = 1.0f;
-  mxopt_norm_result* d_result = e->d_result;
+  // deferred: every accepted micro-batch of the cycle keeps its own clip factor on the device
+  const int result_slot = e->cfg.defer_accumulation ? free_result_slot(e) : 0;
+  mxopt_norm_result* d_result = e->d_result + result_slot;
   int rc;
   if (n) {
     // One read of the gradients: validity of the raw values and the norm of the clamped ones.
@@ -261,8 +331,6 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     mxopt_table* t = nullptr;
     if ((rc = cached_table(ctx, rows, &t))) return rc;
     const double max_norm = e->cfg.has_gradient_clip_norm ? e->cfg.gradient_clip_norm : -1.0;
-    // deferred: every accepted micro-batch of the cycle keeps its own clip factor on the device
-    if (e->cfg.defer_accumulation) d_result += e->held.size();
     if ((rc = mxopt_global_norm(ctx, t, 0, &prep, max_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, d_result))) return rc;
     if ((rc = mxopt_read_norm_result(ctx, d_result, &h))) return rc;
   }
@@ -291,7 +359,9 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
   if (e->cfg.defer_accumulation) {
     // Nothing is accumulated: the micro-batch is only remembered.  At the end of the cycle one pass
     // over p and the held gradients forms sum_j clip_j(clamp(g_j)) in registers and applies lr/N.
+    if (e->held.size() > (size_t)MXOPT_MAX_PENDING && (rc = defer_spill(e))) return rc;
     if ((rc = defer_record(e, idx, grads))) return rc;
+    e->held_result.push_back(result_slot);
     e->have_acc = true;
     e->micro_step += 1;
     int applied = 0;
@@ -301,9 +371,11 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
         if ((rc = defer_table(e, &t))) return rc;
         const float* scales[MXOPT_MAX_PENDING + 1] = {};
         if (e->cfg.has_gradient_clip_norm)
-          for (size_t j = 0; j < e->held.size(); ++j) scales[j] = &e->d_result[j].scale;
+          for (size_t j = 0; j < e->held.size(); ++j)
+            scales[j] = e->held_result[j] >= 0 ? &e->d_result[e->held_result[j]].scale : nullptr;
         prep.d_scale = nullptr;
-        rc = mxopt_sgd_plain_with_pending_list_each(ctx, t, e->cfg.learning_rate / (double)N, 0.0, &prep, scales);
+        rc = mxopt_sgd_plain_with_pending_list_each(ctx, t, e->cfg.learning_rate / (double)N, 0.0, &prep, scales,
+                                                    e->held_is_sum ? 1 : 0);
         (void)mxopt_table_set_pending(t, 0, nullptr, 0);
         if (rc) return rc;
       }
@@ -510,8 +582,10 @@ int sft_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt
   const size_t n = idx.size();
   e->consecutive_nan_count = 0;  // sft/engine.rs:261-267
   if (e->cfg.defer_accumulation) {
-    int rc = defer_record(e, idx, grads);
-    if (rc) return rc;
+    int rc;
+    if (e->held.size() > (size_t)MXOPT_MAX_PENDING && (rc = defer_spill(e))) return rc;
+    if ((rc = defer_record(e, idx, grads))) return rc;
+    e->held_result.push_back(-1);
     e->have_acc = true;
     e->micro_step += 1;
     int applied = 0;
@@ -686,10 +760,6 @@ int mxopt_engine_new(mxopt_ctx* ctx, const mxopt_engine_config* config, size_t n
   if (config->apply != MXOPT_ENGINE_APPLY_SGD && config->apply != MXOPT_ENGINE_APPLY_ADAMW)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: unknown apply mode");
   if (config->defer_accumulation) {
-    if (config->gradient_accumulation_steps > MXOPT_MAX_PENDING + 1)
-      return fail(ctx, MXOPT_ERR_INVALID_ARG,
-                  "mxopt_engine_new: defer_accumulation holds at most " + std::to_string(MXOPT_MAX_PENDING + 1) +
-                      " micro-batches");
     if (config->kind == MXOPT_ENGINE_SFT && !config->accumulate_in_f32)
       return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_new: defer_accumulation adds in float32 (set accumulate_in_f32)");
     if (config->kind == MXOPT_ENGINE_GRPO && config->apply != MXOPT_ENGINE_APPLY_SGD)
@@ -715,8 +785,8 @@ int mxopt_engine_new(mxopt_ctx* ctx, const mxopt_engine_config* config, size_t n
   int rc = MXOPT_OK;
   {
     DeviceGuard guard(ctx->device);
-    // one slot per micro-batch a deferred cycle can hold; slot 0 serves everything else
-    hipError_t err = hipMalloc((void**)&e->d_result, (MXOPT_MAX_PENDING + 1) * sizeof(mxopt_norm_result));
+    // one slot per micro-batch a deferred cycle can hold and one for the arriving one; slot 0 serves everything else
+    hipError_t err = hipMalloc((void**)&e->d_result, kResultSlots * sizeof(mxopt_norm_result));
     if (err != hipSuccess) rc = hip_fail(ctx, err, "mxopt_engine_new: hipMalloc");
   }
   if (!rc && config->apply == MXOPT_ENGINE_APPLY_ADAMW) {
@@ -802,6 +872,8 @@ int mxopt_engine_reset(mxopt_engine* e) {
   e->have_acc = false;
   e->held.clear();
   e->held_slots.clear();
+  e->held_result.clear();
+  e->held_is_sum = false;
   e->micro_step = 0;
   e->step = 0;
   e->nan_gradient_count = 0;

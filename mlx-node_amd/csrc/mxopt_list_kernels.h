@@ -60,6 +60,10 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
     ps_regs[j].has_scale = has;
     ps_regs[j].scale = has ? *scales.s[j] : 1.0f;
   }
+  if (pr.flags & kPrepFirstIsSum) {  // a buffer of earlier micro-batches, each prepared before it was added
+    ps_regs[0].flags = 0;
+    ps_regs[0].has_scale = false;
+  }
   auto gradient = [&](float g, const float (&x)[KMAX]) {
     if (!each) {
       float s = g;

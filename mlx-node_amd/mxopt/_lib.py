@@ -100,7 +100,7 @@ SIGNATURES = {
     "mxopt_sgd_plain_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
                                                     C.POINTER(GradPrep)]),
     "mxopt_sgd_plain_with_pending_list_each": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double, C.c_double,
-                                                         C.POINTER(GradPrep), C.POINTER(C.c_void_p)]),
+                                                         C.POINTER(GradPrep), C.POINTER(C.c_void_p), C.c_int]),
     "mxopt_adam_with_pending": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(SgdHp), C.POINTER(GradPrep)]),
     "mxopt_rmsprop": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(RmspropHp), C.POINTER(GradPrep)]),

@@ -251,11 +251,14 @@ def _sgd_plain_with_pending_list(self, table: "Table", learning_rate: float, wei
 
 
 def _sgd_plain_with_pending_list_each(self, table: "Table", learning_rate: float, scales: Sequence[Optional[int]],
-                                      weight_decay: float = 0.0, prep: Optional[L.GradPrep] = None) -> None:
-    """scales: one device address of a float per stream (tensor.g first), or None for all of them."""
+                                      weight_decay: float = 0.0, prep: Optional[L.GradPrep] = None,
+                                      first_is_sum: bool = False) -> None:
+    """scales: one device address of a float per stream (tensor.g first), or None for all of them.
+    first_is_sum: tensor.g is a float32 sum of already prepared micro-batches (scales[0] is None then)."""
     arr = (C.c_void_p * max(len(scales), 1))(*scales)
     L.check(self.lib.mxopt_sgd_plain_with_pending_list_each(self.handle, table.handle, learning_rate, weight_decay,
-                                                            C.byref(prep) if prep else None, arr), self.handle)
+                                                            C.byref(prep) if prep else None, arr,
+                                                            int(first_is_sum)), self.handle)
 
 
 Context.sgd_plain_with_pending_list_each = _sgd_plain_with_pending_list_each

@@ -213,8 +213,10 @@ def test_one_micro_batch_per_step(mx, kind, apply, bf16):
 # ---------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("n_acc", [1, 3, 4, 6])
+@pytest.mark.parametrize("n_acc", [1, 3, 4, 6, 8, 9, 11])
 def test_grpo_deferred_sequence(mx, bf16, n_acc):
+    """More than eight micro-batches in a cycle: the oldest are added into the float32 buffers as the later
+    ones arrive (clamped and clipped by their own factors), the last seven stay deferred."""
     rng = np.random.default_rng(107 + n_acc)
     params = make_params(rng, bf16)
     dparams = {k: to_dev(v) for k, v in params.items()}
@@ -223,6 +225,7 @@ def test_grpo_deferred_sequence(mx, bf16, n_acc):
     dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
     ref = O.GRPOEngineOptimizerSide(params, **kw)
     script = ["ok", "ok", "nan", "inf", "ok", "ok", "-inf", "ok", "ok", "ok", "ok", "ok", "ok", "ok", "ok"]
+    script += ["ok", "nan"] + ["ok"] * 10 if n_acc > 6 else []
     for it, kind in enumerate(script):
         grads = make_grads(rng, bf16, 0.01 * (1 + it % 3))
         if kind != "ok":
@@ -249,7 +252,7 @@ def test_grpo_deferred_sequence(mx, bf16, n_acc):
 
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("apply", ["sgd", "adamw"])
-@pytest.mark.parametrize("n_acc", [3, 6])
+@pytest.mark.parametrize("n_acc", [3, 6, 9, 12])
 def test_sft_deferred_sequence(mx, bf16, apply, n_acc):
     rng = np.random.default_rng(123)
     params = make_params(rng, bf16)
@@ -274,12 +277,31 @@ def test_sft_deferred_sequence(mx, bf16, apply, n_acc):
     assert dev.flush_gradients() is False and ref.flush_gradients() is False
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_sft_deferred_flush_after_the_oldest_micro_batches_were_spilled(mx, bf16):
+    """Ten of twelve micro-batches, then flush: three have gone into the float32 buffers, seven are still
+    deferred; the average is over the ten."""
+    rng = np.random.default_rng(77)
+    params = make_params(rng, bf16)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.02, gradient_accumulation_steps=12, gradient_clip_norm=0.5, weight_decay=0.01)
+    dev = mx.SFTEngineOptimizerSide(dparams, accumulate_in_f32=True, defer_accumulation=True, **kw)
+    ref = O.SFTEngineOptimizerSide(params, **kw)
+    for cycle in range(2):                                   # the second cycle reuses the buffers of the first
+        for it in range(10):
+            grads = make_grads(rng, bf16, 0.01)
+            m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+            ref.micro_batch({k: O.as_f32(g) for k, g in grads.items()})
+            assert not m.gradients_applied
+        assert dev.flush_gradients() is True
+        assert ref.flush_gradients(norm_sumsq=dev.last_metrics.grad_sumsq) is True
+        check_state(dev, ref, dparams, f"after flush {cycle}")
+
+
 def test_deferred_mode_refuses_what_it_cannot_hold(mx):
     rng = np.random.default_rng(5)
     params = make_params(rng, False)
     dparams = {k: to_dev(v) for k, v in params.items()}
-    with pytest.raises(ValueError, match="at most 8 micro-batches"):
-        mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=9, accumulate_in_f32=True, defer_accumulation=True)
     with pytest.raises(ValueError, match="adds in float32"):
         mx.SFTEngineOptimizerSide(dparams, gradient_accumulation_steps=2, defer_accumulation=True)
     with pytest.raises(ValueError, match="plain SGD only"):

@@ -58,9 +58,9 @@ def both(what, dev_call, ref_call, mx):
 @settings(max_examples=SOAK or 120, deadline=None, derandomize=not SOAK, database=None,
           suppress_health_check=list(HealthCheck))
 @given(kind=st.sampled_from(["grpo", "sft"]), bf16=st.booleans(), apply=st.sampled_from(["sgd", "adamw"]),
-       n_acc=st.sampled_from([1, 2, 3, 5]), defer=st.booleans(), acc_f32=st.booleans(),
+       n_acc=st.sampled_from([1, 2, 3, 5, 9]), defer=st.booleans(), acc_f32=st.booleans(),
        clip_norm=st.sampled_from([None, 0.5]), clip_value=st.sampled_from([None, 0.003]),
-       wd=st.sampled_from([0.0, 0.01]), ops=st.lists(OPS, min_size=1, max_size=14), seed=st.integers(0, 2 ** 31))
+       wd=st.sampled_from([0.0, 0.01]), ops=st.lists(OPS, min_size=1, max_size=22), seed=st.integers(0, 2 ** 31))
 def test_random_engine_sequences(mx, kind, bf16, apply, n_acc, defer, acc_f32, clip_norm, clip_value, wd, ops, seed):
     rng = np.random.default_rng(seed)
     if kind == "grpo" and defer:

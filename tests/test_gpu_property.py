@@ -331,6 +331,9 @@ def test_deferred_accumulation_kernels_match_the_oracle(mx, sizes, k, head, pd, 
 
     if kind == "sgd_plain_each":
         # one norm per stream, of the clamped values (grpo/engine.rs:636-653)
+        # an even seed with a float32 first stream: that stream is a sum of earlier, already prepared
+        # micro-batches and is added untouched
+        first_is_sum = gd == "f32" and seed % 2 == 0
         results, scales, bad = [], [], False
         for j in range(k + 1):
             res = ctx.norm_result()
@@ -347,12 +350,17 @@ def test_deferred_accumulation_kernels_match_the_oracle(mx, sizes, k, head, pd, 
             return          # the engine drops such a micro-batch before anything is added
         prep = mx.make_prep(clamp_pre=(-clamp_pre, clamp_pre) if clamp_pre else None)
         ptrs = [r.scale_ptr for r in results] if clip else [None] * (k + 1)
-        ctx.sgd_plain_with_pending_list_each(table, lr, ptrs, prep=prep)
+        if first_is_sum:
+            ptrs[0] = None
+        ctx.sgd_plain_with_pending_list_each(table, lr, ptrs, prep=prep, first_is_sum=first_is_sum)
         want_g = []
         for i in range(len(sizes)):
             total = None
             for j in range(k + 1):
-                t = prep_oracle(streams[j][i], None, clamp_pre, scales[j] if clip else None, None)[1]
+                if j == 0 and first_is_sum:
+                    t = O.as_f32(streams[0][i])
+                else:
+                    t = prep_oracle(streams[j][i], None, clamp_pre, scales[j] if clip else None, None)[1]
                 total = t if total is None else total + t
             want_g.append(total)
     else:
