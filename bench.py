@@ -436,7 +436,8 @@ class Workload:
             spill = 6 + 10 * (N - mx.MAX_PENDING - 1)
             norms = 2 * N if kind == "grpo" else 4 + 2 * mx.MAX_PENDING
             apply = 4 + 2 * mx.MAX_PENDING + 4
-            self.bytes_per_elem = {"micro_batch_apply": apply + (2 if kind == "grpo" else norms)}
+            # the applying call first makes room for its own micro-batch (10 B), like every call after the eighth
+            self.bytes_per_elem = {"micro_batch_apply": 10 + apply + (2 if kind == "grpo" else norms)}
             self.step_bytes_per_elem = spill + norms + apply
             self.note += "; more than eight micro-batches: the oldest are added into float32 buffers as later ones arrive"
         self.dominant = "micro_batch_apply"
