@@ -64,7 +64,18 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
     ps_regs[0].flags = 0;
     ps_regs[0].has_scale = false;
   }
+  // The GRPO engine's case, every stream clamped and multiplied by its own factor (1 when it has none,
+  // which changes no value), without a branch per stage and stream.
+  const bool each_clamp_scale = each && (pr.flags & (kPrepPreMul | kPrepClampPre | kPrepClampPost)) == kPrepClampPre;
+  const bool first_raw = (pr.flags & kPrepFirstIsSum) != 0;
   auto gradient = [&](float g, const float (&x)[KMAX]) {
+    if (each_clamp_scale) {
+      float s = first_raw ? g : clamp_keep_nan(g, pr.pre_lo, pr.pre_hi) * ps_regs[0].scale;
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k)
+        if (k < kx) s = s + clamp_keep_nan(x[k], pr.pre_lo, pr.pre_hi) * ps_regs[k + 1].scale;
+      return s;
+    }
     if (!each) {
       float s = g;
 #pragma unroll
