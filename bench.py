@@ -399,7 +399,7 @@ class Workload:
         # deferred accumulation reads every micro-batch of the cycle at the end: they must all be resident
         self.micro = [dict(zip(self.names, self.g))]
         # (with more than eight in a cycle the engine adds the oldest into its float32 buffers as later ones
-        # arrive, so eight buffers used in turn are enough)
+        # arrive; the synthetic buffers are never rewritten, so eight of them used in turn stand for any number)
         for _ in range(min(self.n_micro, mx.MAX_PENDING + 1) - 1 if defer else 0):
             self.micro.append(dict(zip(self.names, self._randn_list(bf, 1e-3))))
         if kind == "grpo":   # clamp 1.0 + clip 1.0 per micro-batch, float32 accumulation, p -= lr/N * acc
