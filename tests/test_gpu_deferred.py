@@ -181,6 +181,32 @@ def test_sgd_and_rmsprop_over_deferred_micro_batches(mx, ctx, which, combo, k, l
     table.close()
 
 
+def test_first_is_sum_wants_a_float32_buffer_without_a_clip_factor(mx, ctx):
+    ps, gs, xs = lists(1, [4096], "bf16", 0.02), lists(2, [4096], "bf16", 1e-3), lists(3, [4096], "bf16", 1e-3)
+    dp, dg, dx = to_dev(ps[0]), to_dev(gs[0]), to_dev(xs[0])
+    dsum = to_dev(O.as_f32(gs[0]))
+    res = ctx.norm_result()
+    t16 = ctx.table([mx.TensorSpec(p=dp, p_out=dp, g=dg)])
+    t16.set_pending([[dx]])
+    with pytest.raises(mx.InvalidArg, match="is float32"):
+        ctx.sgd_plain_with_pending_list_each(t16, 0.1, [None, None], first_is_sum=True)
+    t32 = ctx.table([mx.TensorSpec(p=dp, p_out=dp, g=dsum)])
+    t32.set_pending([[dx]])
+    with pytest.raises(mx.InvalidArg, match="has no clip factor"):
+        ctx.sgd_plain_with_pending_list_each(t32, 0.1, [res.scale_ptr, res.scale_ptr], first_is_sum=True)
+    with pytest.raises(mx.InvalidArg, match="either every micro-batch"):
+        ctx.sgd_plain_with_pending_list_each(t32, 0.1, [res.scale_ptr, None])
+    assert_bit_equal(to_host(dp), ps[0], "a refused call changed the parameter")
+    # the sum is taken as it is: no clamp, no factor; the pending stream is clamped
+    ctx.sgd_plain_with_pending_list_each(t32, 0.1, [None, None], prep=mx.make_prep(clamp_pre=(-1e-3, 1e-3)),
+                                         first_is_sum=True)
+    total = O.as_f32(gs[0]) + np.clip(O.as_f32(xs[0]), F(-1e-3), F(1e-3))
+    want = O.apply_gradients({"p": ps[0]}, {"p": total}, 0.1)["p"]
+    assert_bit_equal(to_host(dp), want, "p")
+    t16.close()
+    t32.close()
+
+
 def test_first_momentum_step_cannot_be_conditional(mx, ctx):
     """The first SGD-with-momentum step stores the velocity every later step reads; the host cannot know
     whether a device-side conditional update ran, so that combination is refused, and accepted afterwards."""
