@@ -87,7 +87,9 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
  * 1 <= k <= MXOPT_MAX_PENDING + 1; micro-batches 2..k share one dtype, the first has it or is
  * float32; outs[i] has params[i]'s dtype (it may be params[i] itself).
  * d_norm (nullable, device memory) receives norm, clip factor and the non-finite flag; pass
- * prep->d_skip_if_nonzero = &d_norm->nonfinite to leave everything untouched on a NaN/Inf gradient. */
+ * prep->d_skip_if_nonzero = &d_norm->nonfinite to leave parameters and state untouched on a NaN/Inf
+ * gradient.  The skip happens on the device: the host's call counter (Adam/AdamW bias correction)
+ * advances all the same; a caller that must not count such a step reads d_norm and decides itself. */
 int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, const char* const* param_names,
                                             const mxopt_array* params, size_t k, const mxopt_array* grads,
                                             const mxopt_array* outs, const mxopt_grad_prep* prep, double max_norm,
