@@ -83,9 +83,12 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
  * would have left in a float32 buffer -- then `prep`, then, when max_norm >= 0, the clip factor of
  * GradientUtils::clip_grad_norm (optimizers/mod.rs:67-107; clip_mode as in mxopt_global_norm) of
  * that gradient's global norm, then the optimizer's own update (any of the four kinds) with
- * update_many's per-call step counting.  Two launches per dtype group, no accumulation buffer, no host synchronisation.
- * 1 <= k <= MXOPT_MAX_PENDING + 1; micro-batches 2..k share one dtype, the first has it or is
- * float32; outs[i] has params[i]'s dtype (it may be params[i] itself).
+ * update_many's per-call step counting.  Two launches per dtype group, no accumulation buffer,
+ * no host synchronisation.  k >= 1.  The kernels read MXOPT_MAX_PENDING + 1 streams: with a larger
+ * k the oldest micro-batches are first added, in order, into a float32 buffer per parameter that
+ * the optimizer keeps with its state (4 B/elem, freed by reset), and that buffer stands in for
+ * them.  Of the streams the kernels read, the second to the last share one dtype and the first has
+ * it or is float32; outs[i] has params[i]'s dtype (it may be params[i] itself).
  * d_norm (nullable, device memory) receives norm, clip factor and the non-finite flag; pass
  * prep->d_skip_if_nonzero = &d_norm->nonfinite to leave parameters and state untouched on a NaN/Inf
  * gradient.  The skip happens on the device: the host's call counter (Adam/AdamW bias correction)

@@ -22,6 +22,7 @@ struct StateEntry {
   float* v = nullptr;  // second moment, or SGD velocity
   uint64_t n = 0;
   bool has_velocity = false;  // SGD: velocity written at least once (sgd.rs:98-114)
+  float* sum = nullptr;       // update_many_accumulated with more micro-batches than streams: the oldest, added up
 };
 
 enum class Kind { Adam, AdamW, Sgd, Rmsprop };
@@ -126,6 +127,7 @@ void free_state(mxopt_optimizer* o) {
   for (auto& kv : o->state) {
     if (kv.second.m) (void)hipFree(kv.second.m);
     if (kv.second.v) (void)hipFree(kv.second.v);
+    if (kv.second.sum) (void)hipFree(kv.second.sum);
   }
   o->state.clear();
 }
@@ -425,6 +427,53 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
   return MXOPT_OK;
 }
 
+}  // extern "C"
+
+// More micro-batches than the kernels have streams for: micro-batches 0 .. k - MXOPT_MAX_PENDING - 1 are
+// added, in order, into a float32 buffer per parameter that the optimizer keeps with its state
+// (accumulate_gradients' own additions, models/qwen3/model.rs:2217-2243); on return *folded holds those
+// buffers followed by the last MXOPT_MAX_PENDING micro-batches.
+static int fold_oldest(mxopt_optimizer* opt, size_t n, const char* const* param_names, const mxopt_array* params,
+                       size_t k, const mxopt_array* grads, std::vector<mxopt_array>* folded) {
+  mxopt_ctx* ctx = opt->ctx;
+  const size_t spill = k - (size_t)MXOPT_MAX_PENDING;
+  std::vector<float*> sums(n, nullptr);
+  DeviceGuard guard(ctx->device);
+  for (size_t i = 0; i < n; ++i) {
+    if (!param_names[i]) return fail(ctx, MXOPT_ERR_INVALID_ARG, "param_name is NULL");
+    int rc = check_array(ctx, &params[i], "param");
+    if (rc) return rc;
+    StateEntry* st = nullptr;
+    if ((rc = get_state(opt, param_names[i], params[i].n, &st))) return rc;
+    if (!st->sum && st->n) HIP_TRY(ctx, hipMalloc((void**)&st->sum, st->n * sizeof(float)));
+    sums[i] = st->sum;
+  }
+  for (size_t j = 0; j < spill; ++j) {
+    std::vector<mxopt_tensor> rows(n, blank_tensor());
+    for (size_t i = 0; i < n; ++i) {
+      const mxopt_array& g = grads[j * n + i];
+      int rc = check_array(ctx, &g, "update_many_accumulated: gradient");
+      if (rc) return rc;
+      if (g.n != params[i].n)
+        return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string("'") + param_names[i] + "': param and grad differ in size");
+      rows[i].g = g.data; rows[i].g_dtype = (uint8_t)g.dtype;
+      rows[i].g_out = sums[i]; rows[i].g_out_dtype = MXOPT_F32;
+      rows[i].n = g.n;
+    }
+    mxopt_table* t = nullptr;
+    int rc = cached_table(ctx, rows, &t);
+    if (!rc) rc = mxopt_accumulate(ctx, t, j == 0, nullptr, -1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, nullptr);
+    if (rc) return rc;
+  }
+  folded->resize(((size_t)MXOPT_MAX_PENDING + 1) * n);
+  for (size_t i = 0; i < n; ++i) (*folded)[i] = mxopt_array{sums[i], params[i].n, MXOPT_F32};
+  for (size_t j = 0; j < (size_t)MXOPT_MAX_PENDING; ++j)
+    for (size_t i = 0; i < n; ++i) (*folded)[(j + 1) * n + i] = grads[(spill + j) * n + i];
+  return MXOPT_OK;
+}
+
+extern "C" {
+
 int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, const char* const* param_names,
                                             const mxopt_array* params, size_t k, const mxopt_array* grads,
                                             const mxopt_array* outs, const mxopt_grad_prep* prep, double max_norm,
@@ -432,11 +481,16 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
   const char* op = "update_many_accumulated";
   if (!opt) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": optimizer is NULL");
   mxopt_ctx* ctx = opt->ctx;
-  if (k < 1 || k > (size_t)MXOPT_MAX_PENDING + 1)
-    return fail(ctx, MXOPT_ERR_INVALID_ARG,
-                std::string(op) + ": between 1 and " + std::to_string(MXOPT_MAX_PENDING + 1) + " micro-batches");
+  if (k < 1) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": at least one micro-batch");
   if (n && (!param_names || !params || !grads || !outs))
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
+  std::vector<mxopt_array> folded;
+  if (k > (size_t)MXOPT_MAX_PENDING + 1) {
+    int rc = fold_oldest(opt, n, param_names, params, k, grads, &folded);
+    if (rc) return rc;
+    grads = folded.data();
+    k = (size_t)MXOPT_MAX_PENDING + 1;
+  }
   if (prep && prep->d_scale && max_norm >= 0.0)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": prep->d_scale and max_norm exclude each other");
   // Every later micro-batch must look like the first: same sizes, one dtype.

@@ -1,6 +1,6 @@
 """Random call sequences against the optimizer objects (state by name, per-call step counting, cached and
 retargeted tables, first-step velocity, checkpoints): update_single in and out of place, update_many over
-subsets in any order with the same or with moved buffers, update_many_accumulated over 1..8 un-summed
+subsets in any order with the same or with moved buffers, update_many_accumulated over 1..12 un-summed
 micro-batches with or without clipping, reset, save_file/load_file into a fresh object.  After every call
 the parameters must equal the oracle's bit for bit.  Derandomised; MXOPT_PROPERTY_EXAMPLES=<n> draws n
 fresh random sequences instead."""
@@ -89,7 +89,7 @@ def test_random_optimizer_sequences(mx, tmp_path_factory, kind, bf16, g_bf16, op
                 ref_step(k, gs[k])
         elif op == "accumulated":
             names = [k for k in SIZES if rng.random() < 0.7] or ["embed"]
-            n_micro = int(rng.integers(1, 9))
+            n_micro = int(rng.integers(1, 13))
             micro = [{k: grad(k) for k in names} for _ in range(n_micro)]
             clip = bool(rng.integers(0, 2))
             res = ctx.norm_result()
