@@ -448,7 +448,7 @@ static int fold_oldest(mxopt_optimizer* opt, size_t n, const char* const* param_
     if (!st->sum && st->n) HIP_TRY(ctx, hipMalloc((void**)&st->sum, st->n * sizeof(float)));
     sums[i] = st->sum;
   }
-  for (size_t j = 0; j < spill; ++j) {
+  for (size_t j = 0; j < spill && n; ++j) {
     std::vector<mxopt_tensor> rows(n, blank_tensor());
     for (size_t i = 0; i < n; ++i) {
       const mxopt_array& g = grads[j * n + i];
