@@ -448,7 +448,7 @@ static int fold_oldest(mxopt_optimizer* opt, size_t n, const char* const* param_
     if (!st->sum && st->n) HIP_TRY(ctx, hipMalloc((void**)&st->sum, st->n * sizeof(float)));
     sums[i] = st->sum;
   }
-  for (size_t j = 0; j < spill && n; ++j) {
+  for (size_t j = 0; j < spill; ++j) {
     std::vector<mxopt_tensor> rows(n, blank_tensor());
     for (size_t i = 0; i < n; ++i) {
       const mxopt_array& g = grads[j * n + i];
@@ -484,6 +484,7 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
   if (k < 1) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": at least one micro-batch");
   if (n && (!param_names || !params || !grads || !outs))
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
+  if (n == 0) return MXOPT_OK;
   std::vector<mxopt_array> folded;
   if (k > (size_t)MXOPT_MAX_PENDING + 1) {
     int rc = fold_oldest(opt, n, param_names, params, k, grads, &folded);

@@ -402,5 +402,6 @@ def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind, which
     # a refused call leaves the counter alone
     with pytest.raises(mx.InvalidArg, match="at least one micro-batch"):
         opt.update_many_accumulated(names, dp, [])
+    opt.update_many_accumulated([], [], [[] for _ in range(10)])   # an empty list is a no-op for any k
     if which == "adamw":
         assert opt.step == 5 * len(names)
