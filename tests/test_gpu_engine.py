@@ -298,6 +298,29 @@ def test_sft_deferred_flush_after_the_oldest_micro_batches_were_spilled(mx, bf16
         check_state(dev, ref, dparams, f"after flush {cycle}")
 
 
+@pytest.mark.parametrize("kind", ["sft", "grpo"])
+@pytest.mark.parametrize("n_acc", [3, 10])
+def test_deferred_cycles_with_an_empty_and_a_one_element_tensor(mx, kind, n_acc):
+    rng = np.random.default_rng(1)
+    params = {"a": np.zeros(0, F), "b": rng.normal(0, 0.1, 5000).astype(F), "c": rng.normal(0, 0.1, 1).astype(F)}
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=0.5)
+    if kind == "sft":
+        dev = mx.SFTEngineOptimizerSide(dparams, accumulate_in_f32=True, defer_accumulation=True, **kw)
+        ref = O.SFTEngineOptimizerSide(params, **kw)
+    else:
+        dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
+        ref = O.GRPOEngineOptimizerSide(params, **kw)
+    for it in range(2 * n_acc):
+        grads = {k: rng.normal(0, 0.01, v.size).astype(F) for k, v in params.items()}
+        m = dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+        if kind == "grpo" or m.gradients_applied:
+            ref.micro_batch(grads, norm_sumsq=m.grad_sumsq)
+        else:
+            ref.micro_batch(grads)
+    check_state(dev, ref, dparams, f"{kind} N={n_acc}")
+
+
 def test_deferred_mode_refuses_what_it_cannot_hold(mx):
     rng = np.random.default_rng(5)
     params = make_params(rng, False)
