@@ -136,6 +136,58 @@ static void known_answers(void) {
   for (int k = 0; k < 4; ++k) CHECK_HIP(hipFree(held[k]));
 }
 
+/* Twelve micro-batches per step through the SFT engine (clip by global norm, decay), once with its
+ * float32 accumulation buffer and once deferred -- more than the kernels have streams for, so the
+ * oldest are added into a buffer as later ones arrive.  The parameters must come out bit-identical. */
+static void long_cycle(void) {
+  enum { N = 5003, MICRO = 12, CYCLES = 2 };
+  static float host[N], a_out[N], b_out[N];
+  for (int i = 0; i < N; ++i) host[i] = (float)((i * 37) % 201 - 100) * 1e-3f;
+  float* w[2] = {to_device(host, N), to_device(host, N)};
+  float* g[MICRO];
+  mxopt_engine* eng[2] = {NULL, NULL};
+  const char* names[1] = {"w"};
+  for (int e = 0; e < 2; ++e) {
+    mxopt_engine_config cfg;
+    mxopt_engine_config_default(MXOPT_ENGINE_SFT, &cfg);
+    cfg.learning_rate = 0.02;
+    cfg.gradient_accumulation_steps = MICRO;
+    cfg.has_gradient_clip_norm = 1;
+    cfg.gradient_clip_norm = 0.5;
+    cfg.weight_decay = 0.01;
+    cfg.accumulate_in_f32 = 1;
+    cfg.defer_accumulation = e;
+    mxopt_array aw = {w[e], N, MXOPT_F32};
+    CHECK_MX(mxopt_engine_new(ctx, &cfg, 1, names, &aw, &eng[e]));
+  }
+  for (int c = 0; c < CYCLES; ++c) {
+    for (int k = 0; k < MICRO; ++k) {
+      for (int i = 0; i < N; ++i)
+        host[i] = (float)((int)(((unsigned)i * 2654435761u + (unsigned)(c * MICRO + k) * 40503u) % 2001u) - 1000) * 1e-4f;
+      g[k] = to_device(host, N);
+      for (int e = 0; e < 2; ++e) {
+        mxopt_array a = {g[k], N, MXOPT_F32};
+        mxopt_engine_metrics m;
+        CHECK_MX(mxopt_engine_micro_batch(eng[e], 1, names, &a, &m));
+        if (m.gradients_applied != (k == MICRO - 1)) { fprintf(stderr, "FAIL long cycle bookkeeping at %d\n", k); exit(1); }
+      }
+    }
+    CHECK_MX(mxopt_synchronize(ctx));
+    for (int k = 0; k < MICRO; ++k) CHECK_HIP(hipFree(g[k]));  /* the deferred engine needed them until here */
+  }
+  CHECK_HIP(hipMemcpy(a_out, w[0], sizeof a_out, hipMemcpyDeviceToHost));
+  CHECK_HIP(hipMemcpy(b_out, w[1], sizeof b_out, hipMemcpyDeviceToHost));
+  if (memcmp(a_out, b_out, sizeof a_out) != 0 || a_out[1] == (float)((37 % 201) - 100) * 1e-3f) {
+    fprintf(stderr, "FAIL deferred and buffered SFT engines differ after %d micro-batches\n", MICRO);
+    exit(1);
+  }
+  printf("PASS SFT engine, %d micro-batches per step: deferred accumulation bit-identical to the float32 buffer\n", MICRO);
+  for (int e = 0; e < 2; ++e) {
+    mxopt_engine_free(eng[e]);
+    CHECK_HIP(hipFree(w[e]));
+  }
+}
+
 /* Qwen3-0.6B: vocab 151936, hidden 1024, 28 layers, q 2048x1024, k/v 1024x1024, o 1024x2048,
  * gate/up 3072x1024, down 1024x3072, four norm vectors per layer, final norm, tied embedding. */
 static size_t qwen3_06b(size_t* sizes) {
@@ -201,6 +253,7 @@ int main(int argc, char** argv) {
   CHECK_MX(mxopt_create(0, NULL, &ctx));
   printf("%s\n", mxopt_version());
   known_answers();
+  long_cycle();
   if (argc < 2 || strcmp(argv[1], "--no-timing") != 0) timing();
   mxopt_destroy(ctx);
   return 0;

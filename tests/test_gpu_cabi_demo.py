@@ -18,7 +18,7 @@ def test_plain_c_host_known_answers_and_timing():
     proc = subprocess.run([DEMO], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     passed = [l for l in proc.stdout.splitlines() if l.startswith("PASS")]
-    assert len(passed) == 5, proc.stdout
+    assert len(passed) == 6, proc.stdout
     m = re.search(r"TIMING tensors=(\d+) elements=(\d+) update_single_loop_ms=([\d.]+) \(host enqueue ([\d.]+)\) "
                   r"update_many_ms=([\d.]+)", proc.stdout)
     assert m, proc.stdout
