@@ -822,9 +822,11 @@ int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t,
   StreamScales sc{};
   const int from = first_is_sum ? 1 : 0;
   if (first_is_sum) {
-    if (d_scales[0]) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of prepared micro-batches has no clip factor");
+    if (d_scales[0])
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of prepared micro-batches has no clip factor");
     for (const Group& g : t->groups)
-      if (g.gd != MXOPT_F32) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of micro-batches is float32");
+      if (g.gd != MXOPT_F32)
+        return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": a sum of micro-batches is float32");
     dp.flags |= kPrepFirstIsSum;
   }
   int with = 0;

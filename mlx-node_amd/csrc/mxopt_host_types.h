@@ -44,7 +44,8 @@ struct DevChunk {
 constexpr uint32_t kPrepPreMul = 1u, kPrepClampPre = 2u, kPrepClampPost = 4u;
 constexpr uint32_t kPrepPendingOnly = 8u;  // update kernels with a pending gradient: g + prep(g2), not prep(g + g2)
 constexpr uint32_t kPrepEachStream = 16u;  // list kernels: prep every stream (own clip factor), then add
-constexpr uint32_t kPrepFirstIsSum = 32u;  // with kPrepEachStream: tensor.g holds already prepared micro-batches, added as it is
+// with kPrepEachStream: tensor.g holds already prepared micro-batches and is added as it is
+constexpr uint32_t kPrepFirstIsSum = 32u;
 struct DevPrep {  // kernel argument
   const float* d_scale;
   const unsigned long long* d_skip_if_nonzero;
