@@ -321,6 +321,22 @@ int mxopt_sgd_plain_with_pending_list_each(mxopt_ctx* ctx, const mxopt_table* t,
 int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep,
                       double max_norm, int clip_mode, mxopt_norm_result* d_result);
 
+/* mxopt_global_norm for callers that cannot allocate device memory (a step being captured into a HIP
+ * graph, a serving loop that forbids hipMalloc, a harness that counts allocations).  It has no
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical *d_result; the one
+ * difference is where the per-workgroup partial sums live: in a fixed array of
+ * MXOPT_STATIC_NORM_WORKGROUPS float64 values (128 KiB) inside the library's code object, of which
+ * every GPU the library runs on holds one copy until the process ends, instead of a buffer the
+ * context allocates on first use and grows on demand.  The call allocates and frees nothing on the
+ * device and records no memset.  A table whose reduction takes more workgroups than the array has
+ * slots (sum over dtype groups of min(chunks, CUs x grid_blocks_per_cu); 4096 per group by default)
+ * is refused with MXOPT_ERR_INVALID_ARG.  All contexts on one GPU share that GPU's array: every slot
+ * a call reads was written by the same call, so nothing has to be cleared, but two such calls that
+ * overlap in time on one GPU (different streams) race and must be ordered by the caller. */
+#define MXOPT_STATIC_NORM_WORKGROUPS 16384
+int mxopt_global_norm_static(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep,
+                             double max_norm, int clip_mode, mxopt_norm_result* d_result);
+
 /* g_out = prep(g) element-wise (scale and/or clamps): the scale pass of clip_grad_norm
  * (optimizers/mod.rs:98-102), clip_grad_value (:164-166), clip_gradients_by_value
  * (gradients/mod.rs:299-312).  Only needed when the clipped gradients themselves must be

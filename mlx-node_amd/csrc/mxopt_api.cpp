@@ -165,15 +165,18 @@ std::string dtype_names(const Group& g) {
 
 // Second pass shared by mxopt_global_norm and mxopt_accumulate.
 int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode,
-                       mxopt_norm_result* d_result) {
+                       mxopt_norm_result* d_result, const double* partials) {
   const int has_max = max_norm >= 0.0;
-  launch_norm_finish(ctx->stream, ctx->d_partial_sum, npartials, max_norm, has_max, clip_mode,
+  launch_norm_finish(ctx->stream, partials ? partials : ctx->d_partial_sum, npartials, max_norm, has_max, clip_mode,
                      d_result);
   return check_launch(ctx, "norm_finish_kernel");
 }
 
+// static_partials: the partial sums go to the library's fixed device array instead of the context's
+// buffer, and nothing is allocated; a table that wants more workgroups than the array has slots is refused.
 static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, const mxopt_grad_prep* prep,
-                     double max_norm, int clip_mode, mxopt_norm_result* d_result, const char* op) {
+                     double max_norm, int clip_mode, mxopt_norm_result* d_result, const char* op,
+                     bool static_partials = false) {
   if (clip_mode != MXOPT_CLIP_ALWAYS_MULTIPLY && clip_mode != MXOPT_CLIP_IF_ABOVE)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unknown clip mode");
   DeviceGuard guard(ctx->device);
@@ -181,9 +184,19 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
   size_t total_grid = 0;
   for (const Group& g : t->groups) total_grid += persistent_grid(ctx, g.nchunks);
   const bool want = d_result != nullptr;
-  if (want) {
+  double* partials = nullptr;
+  if (static_partials) {
+    if (total_grid > kStaticPartials)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  std::string(op) + ": this table takes " + std::to_string(total_grid) +
+                      " workgroups (one partial sum each), the fixed array holds " +
+                      std::to_string(kStaticPartials) + "; lower grid_blocks_per_cu or use mxopt_global_norm");
+    if (!ctx->d_static_partials) return fail(ctx, MXOPT_ERR_FAILURE, std::string(op) + ": the fixed array has no address");
+    partials = ctx->d_static_partials;
+  } else if (want) {
     int rc = ensure_partials(ctx, std::max<size_t>(total_grid, 1));
     if (rc) return rc;
+    partials = ctx->d_partial_sum;
   }
   size_t offset = 0;
   for (const Group& g : t->groups) {
@@ -195,13 +208,13 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
     const int ad = mode == 0 ? g.gd : g.god;
     MXOPT_DEBUG("%s (reduction mode %d%s): %s, %u chunks in %u workgroups", op, mode, first ? ", first" : "",
                 dtype_names(g).c_str(), g.nchunks, L.grid);
-    if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? ctx->d_partial_sum + offset : nullptr))
+    if (!launch_sumsq(mode, ad, g.gd, L, dp, first, want ? partials + offset : nullptr))
       return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": unsupported dtypes " + dtype_names(g));
     int rc = check_launch(ctx, op);
     if (rc) return rc;
     offset += L.grid;
   }
-  if (want) return finish_norm(ctx, (uint32_t)offset, max_norm, clip_mode, d_result);
+  if (want) return finish_norm(ctx, (uint32_t)offset, max_norm, clip_mode, d_result, partials);
   return MXOPT_OK;
 }
 
@@ -282,6 +295,14 @@ int mxopt_create(int device, void* hip_stream, mxopt_ctx** out) {
   ctx->device = device;
   ctx->stream = (hipStream_t)hip_stream;
   ctx->num_cus = prop.multiProcessorCount;
+  {
+    DeviceGuard guard(device);
+    const hipError_t e = static_partials_address(device, &ctx->d_static_partials);
+    if (e != hipSuccess) {
+      delete ctx;
+      return hip_fail(nullptr, e, "mxopt_create: hipGetSymbolAddress(fixed partial-sum array)");
+    }
+  }
   *out = ctx;
   return MXOPT_OK;
 }
@@ -905,6 +926,16 @@ int mxopt_global_norm(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxo
   if (rc) return rc;
   if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm: d_result is NULL");
   return run_sumsq(ctx, t, which, 0, prep, max_norm, clip_mode, d_result, "mxopt_global_norm");
+}
+
+int mxopt_global_norm_static(mxopt_ctx* ctx, const mxopt_table* t, int which, const mxopt_grad_prep* prep,
+                             double max_norm, int clip_mode, mxopt_norm_result* d_result) {
+  if (which != 0 && which != 1)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm_static: which must be 0 or 1");
+  int rc = require(ctx, t, which == 0 ? kNeedG : kNeedGOut, "mxopt_global_norm_static");
+  if (rc) return rc;
+  if (!d_result) return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_global_norm_static: d_result is NULL");
+  return run_sumsq(ctx, t, which, 0, prep, max_norm, clip_mode, d_result, "mxopt_global_norm_static", true);
 }
 
 int mxopt_accumulate(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep, double max_norm,

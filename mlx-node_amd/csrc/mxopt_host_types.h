@@ -79,6 +79,7 @@ struct mxopt_ctx {
   int nontemporal_reduce = 1;   // streaming-hint loads in the read-only reduction kernels
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
   size_t partial_cap = 0;
+  double* d_static_partials = nullptr;        // this device's copy of the library's fixed partial-sum array
   mxopt_norm_result* d_norm_scratch = nullptr;  // result slot of the gradient utilities
   struct CachedTable {                          // tables built by the host layer, most recent last
     std::vector<mxopt_tensor> key;

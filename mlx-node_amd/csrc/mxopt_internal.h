@@ -56,7 +56,9 @@ bool prep_active(const mxopt_grad_prep* p);
 uint32_t persistent_grid(const mxopt_ctx* ctx, uint32_t nchunks);
 int ensure_partials(mxopt_ctx* ctx, size_t need);
 int check_launch(mxopt_ctx* ctx, const char* what);
-int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode, mxopt_norm_result* d_result);
+// partials == NULL: the context's own buffer.
+int finish_norm(mxopt_ctx* ctx, uint32_t npartials, double max_norm, int clip_mode, mxopt_norm_result* d_result,
+                const double* partials = nullptr);
 void fill_dev_tensor(const mxopt_tensor& s, DevTensor& d);
 uint64_t chunks_of(const DevTensor& d);  // chunk-table entries (= workgroups of work) of one tensor
 // A launch over the single tensor `t` (descriptor passed in the kernel arguments).

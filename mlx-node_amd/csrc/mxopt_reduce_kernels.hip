@@ -1,5 +1,7 @@
 // mxopt kernels for gfx950, part 2: global-norm reduction (optionally fused with gradient accumulation)
 // and the synthetic-data generator.
+#include <mutex>
+
 #include "mxopt_kernels_common.h"
 
 namespace mxopt {
@@ -270,6 +272,33 @@ void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t 
                         int has_max, int clip_mode, mxopt_norm_result* d_out) {
   hipLaunchKernelGGL(norm_finish_kernel, dim3(1), dim3(kThreads), 0, stream, partial_sum, npartials, max_norm,
                      has_max, clip_mode, d_out);
+}
+
+// ------------------------------------------------------------------------------------
+// Partial sums that need no allocation: a fixed array in the code object's own device memory, one
+// copy per GPU, for callers that may not allocate (mxopt_global_norm_static).  On the host the
+// array's name is only a handle for hipGetSymbolAddress: kernels are given the address that call
+// returned for the device they run on, never the name.
+// ------------------------------------------------------------------------------------
+
+static __device__ __align__(256) double scratch[kStaticPartials];
+
+// Looked up once per device, with that device current (mxopt_create calls this), and kept.
+hipError_t static_partials_address(int device, double** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static double* known[kMaxDevices];
+  *out = nullptr;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (known[device] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    known[device] = (double*)ptr;
+  }
+  *out = known[device];
+  return hipSuccess;
 }
 
 }  // namespace mxopt

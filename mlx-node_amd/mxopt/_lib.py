@@ -109,6 +109,8 @@ SIGNATURES = {
                                                C.c_int]),
     "mxopt_global_norm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
                                     C.c_void_p]),
+    "mxopt_global_norm_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,
+                                           C.c_void_p]),
     "mxopt_grad_transform": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep)]),
     "mxopt_accumulate_transformed": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep)]),
     "mxopt_accumulate": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(GradPrep), C.c_double, C.c_int,

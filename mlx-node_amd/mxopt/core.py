@@ -181,6 +181,14 @@ class Context:
         L.check(self.lib.mxopt_global_norm(self.handle, table.handle, which, C.byref(prep) if prep else None,
                                            max_norm, clip_mode, C.c_void_p(out.ptr)), self.handle)
 
+    def global_norm_static(self, table: "Table", out: NormResultBuffer, which: int = 0,
+                           prep: Optional[L.GradPrep] = None, max_norm: float = -1.0,
+                           clip_mode: int = L.CLIP_ALWAYS_MULTIPLY) -> None:
+        """global_norm with its partial sums in the library's fixed device array: allocates nothing."""
+        L.check(self.lib.mxopt_global_norm_static(self.handle, table.handle, which,
+                                                  C.byref(prep) if prep else None, max_norm, clip_mode,
+                                                  C.c_void_p(out.ptr)), self.handle)
+
     def grad_transform(self, table: "Table", prep: Optional[L.GradPrep]) -> None:
         L.check(self.lib.mxopt_grad_transform(self.handle, table.handle, C.byref(prep) if prep else None),
                 self.handle)
