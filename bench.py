@@ -15,8 +15,10 @@ bytes per launch / its average duration measured with events on the launch strea
 bounded sample of the same workload and scales it to the full parameter list.
 `deferred_accumulation` (default workload only, when four micro-batch buffers fit) is the same step on
 the same buffers with the micro-batches added in registers instead of into the float32 buffer.
-The buffers are allocated inside mxopt_hbm_spread_begin/_end unless --placement plain is given
-(`config.placement` says which).
+Every buffer comes from a region-interleaved arena (mxopt_hbm_pool_create, `config.placement`) unless
+--placement plain or spread is given.  The default run also measures the four bare streaming probes on
+memory from the same arena (`roofline.measured_ceiling`) and, after config 5's buffers are released,
+BASELINE's configs 1 - 4 for a few steps each (`other_configs`).
 """
 from __future__ import annotations
 
@@ -32,11 +34,25 @@ sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per element per launch of the dominant kernel, measured with rocprofv3 FETCH_SIZE and
-# WRITE_SIZE (each scaled by what the same counter reads for this library's plain copy kernel:
-# 1.98445 and 1.00000); the runs and raw values are in profiles/hbm_traffic_pmc_cfg5_and_copy.txt.
+# HBM bytes per element per launch of the dominant kernel from an EARLIER rocprofv3 run, not from this
+# one (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for this library's plain
+# copy kernel: 1.98445 and 1.00000).  Printed as roofline.traffic with roofline.traffic_source naming
+# the file; null when a kernel source is newer than that file.
 # (workload, fold_last) -> bytes per element
+TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc_cfg5_and_copy.txt"
 MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.97, ("cfg5", 0): 23.93, ("cfg5-deferred", 1): 27.89}
+PROBE_PROFILE = "profiles/probe_streams_pool_and_plain.txt"
+OTHER_CONFIGS = ["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat"]
+
+
+def traffic_profile_is_current():
+    """False when a kernel source changed after the counters were taken."""
+    prof = os.path.join(ROOT, TRAFFIC_PROFILE)
+    if not os.path.exists(prof):
+        return False
+    csrc = os.path.join(ROOT, "mlx-node_amd", "csrc")
+    kernel_files = ("mxopt_kernels.hip", "mxopt_kernels_common.h", "mxopt_device.h", "mxopt_list_kernels.h")
+    return all(os.path.getmtime(os.path.join(csrc, f)) <= os.path.getmtime(prof) for f in kernel_files)
 
 
 def parse_args():
@@ -46,7 +62,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
                     choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
-                             "cfg4", "cfg4-flat", "cfg5", "cfg5-deferred", "copy", "grpo-engine", "sft-engine"])
+                             "cfg4", "cfg4-flat", "cfg5", "cfg5-deferred", "copy", "probes", "grpo-engine", "sft-engine"])
     ap.add_argument("--cpu-sample", type=int, default=512 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
     ap.add_argument("--scale", type=float, default=1.0,
@@ -55,9 +71,16 @@ def parse_args():
     ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab", "packed"],
                     help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
                          "tensors are 512-byte aligned views into it")
-    ap.add_argument("--placement", default="spread", choices=["spread", "plain"],
-                    help="spread: the buffers are allocated inside mxopt_hbm_spread_begin/end (their physical pages "
-                         "interleaved with released memory); plain: wherever the driver puts them")
+    ap.add_argument("--placement", default="pool", choices=["pool", "spread", "plain"],
+                    help="pool: every buffer comes from a region-interleaved arena (mxopt_hbm_pool_create); spread: the "
+                         "buffers are allocated inside mxopt_hbm_spread_begin/end (their physical pages interleaved with "
+                         "released memory, a matter of luck); plain: wherever the driver puts them")
+    ap.add_argument("--pool-regions", type=int, default=2, help="--placement pool: regions to alternate between (0 = all found)")
+    ap.add_argument("--pool-chunk-mb", type=int, default=0, help="--placement pool: chunk size (0 = the library's 64)")
+    ap.add_argument("--others", type=int, default=-1,
+                    help="1: after the main workload, run BASELINE's configs 1-4 for a few steps each and report them as "
+                         "other_configs; default: only when the workload is cfg5 at full scale")
+    ap.add_argument("--others-steps", type=int, default=5)
     ap.add_argument("--spread-block-mb", type=int, default=0, help="--placement spread: block size (0 = the library's 64)")
     ap.add_argument("--spread-keep", type=int, default=0, help="--placement spread: every n-th block is kept (0 = 3)")
     ap.add_argument("--micro", type=int, default=4,
@@ -87,6 +110,8 @@ def tensor_sizes(args):
         return sizes, f"qwen3-{model.lower()}"
     if args.workload == "copy":
         return [int((1 << 30) * args.scale)], "one-flat-f32-tensor"
+    if args.workload == "probes":
+        return [max(4096, int((1 << 30) * args.scale) // 4096 * 4096)], "four-flat-f32-streams"
     import numpy as np
     rng = np.random.default_rng(0x5EED0001)
     sizes = np.floor(np.exp(rng.uniform(np.log(64), np.log(65536), 10000))).astype(np.int64).tolist()
@@ -98,25 +123,46 @@ def tensor_sizes(args):
 class Workload:
     """Holds device buffers + tables and knows how to run one step and what it costs."""
 
-    def __init__(self, args, torch, mx):
+    def __init__(self, args, torch, mx, ctx, pool=None):
         self.args, self.torch, self.mx = args, torch, mx
-        self.ctx = mx.Context()
-        for opt in args.option:
-            k, v = opt.split("=")
-            self.ctx.set_option(k, int(v))
+        self.ctx, self.pool = ctx, pool
         self.sizes, self.list_name = tensor_sizes(args)
         self.n = int(sum(self.sizes))
         self.kernel_events = {}     # kernel name -> list of (start, end) events
         self.res = self.ctx.norm_result()
-        with (self.ctx.hbm_spread(args.spread_block_mb << 20, args.spread_keep) if args.placement == "spread"
-              else contextlib.nullcontext()):
+        if pool is not None:
+            self.mem_pool = pool.torch_pool()     # torch allocates this workload's buffers from the arena
+            window = torch.cuda.use_mem_pool(self.mem_pool)
+        elif args.placement == "spread":
+            window = self.ctx.hbm_spread(args.spread_block_mb << 20, args.spread_keep)
+        else:
+            window = contextlib.nullcontext()
+        with window:
             getattr(self, "_setup_" + args.workload.replace("-", "_"))()
             torch.cuda.synchronize()
+
+    def free_bytes(self):
+        """Device memory this workload may still take."""
+        if self.pool is not None:
+            i = self.pool.info()
+            return i.capacity_bytes - i.used_bytes
+        return self.torch.cuda.mem_get_info()[0]
+
+    def close(self):
+        """Gives the buffers back (to the arena, or to the driver)."""
+        self.torch.cuda.synchronize()
+        for k in list(vars(self)):
+            if k not in ("args", "torch", "mx", "ctx", "pool", "n", "sizes", "list_name"):
+                delattr(self, k)
+        import gc
+        gc.collect()
+        self.torch.cuda.empty_cache()
 
     # -- helpers
     SEED = 0x5EED0001
     CONFIG_ID = {"cfg1": 1, "cfg1-update-single": 1, "cfg1-update-many": 1, "cfg2": 2, "cfg3-sgd": 3, "cfg3-rmsprop": 3,
-                 "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "cfg5-deferred": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8}
+                 "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "cfg5-deferred": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8,
+                 "probes": 9}
 
     def _fill(self, views, stream_id, dist, a, b=0.0):
         """Counter-based synthetic data (mxopt_fill_synthetic): every element is a function of
@@ -179,7 +225,7 @@ class Workload:
         t, mx = self.torch, self.mx
         bf = t.bfloat16
         need = self.n * (2 + 8 + 4)
-        free, _ = t.cuda.mem_get_info()
+        free = self.free_bytes()
         self.n_micro = 4
         n_gbuf = 4 if free > need + 4 * self.n * 2 + (3 << 30) else 1
         self.p = self._randn_list(bf, 0.02)
@@ -473,6 +519,24 @@ class Workload:
     def _step_copy(self):
         self._timed("copy", lambda: self.ctx.grad_transform(self.t_copy, None))
 
+    # -- probes: the bare streaming kernels (mxopt_probe_stream), one launch each per step: the measured
+    #    ceilings of a read-only, a write-only, a copy and a 4-read/3-write pass on this memory
+    def _setup_probes(self):
+        t = self.torch
+        self.streams = [t.zeros(self.n, dtype=t.float32, device="cuda") for _ in range(4)]
+        self.dtype = "u32"
+        self.bytes_per_elem = {"probe_read": 4, "probe_write": 4, "probe_copy": 8, "probe_mix43": 28}
+        self.step_bytes_per_elem = 44
+        self.dominant = "probe_mix43"
+        self.note = "bare kernels: no table, no tails, no arithmetic; mix43 = float32 AdamW's four read and three write streams"
+
+    def _step_probes(self):
+        c, mx, s = self.ctx, self.mx, self.streams
+        self._timed("probe_read", lambda: c.probe_stream(mx.PROBE_READ, s[0]))
+        self._timed("probe_write", lambda: c.probe_stream(mx.PROBE_WRITE, s[1]))
+        self._timed("probe_copy", lambda: c.probe_stream(mx.PROBE_COPY, s[0], s[1]))
+        self._timed("probe_mix43", lambda: c.probe_stream(mx.PROBE_MIX43, *s))
+
     def step(self):
         getattr(self, "_step_" + self.args.workload.replace("-", "_"))()
 
@@ -554,6 +618,88 @@ def cpu_baseline(args, n_total):
 
 # ----------------------------------------------------------------------------------------
 
+def cpu_baseline_cfg1_full():
+    """BASELINE's config 1 on the host in full: the Qwen3-0.6B list (310 tensors, 596 M elements), inputs from the
+    library's synthetic generator (the host twin regenerates what the device would hold), one AdamW step as the
+    reference runs it: per tensor, 13 separate float32 passes."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle_c_binding as B
+    from mxopt.qwen3_shapes import QWEN3, numel, param_list
+    import mxopt
+    oc = B.load()
+    sizes = [numel(shape) for _, shape in param_list(QWEN3["0.6B"])]
+    key = lambda stream, i: mxopt.synthetic_key(Workload.SEED, 1, 0, stream, i)
+    ps = [oc.fill_synthetic(n, "f32", key(1, i), 0, 0.02) for i, n in enumerate(sizes)]
+    gs = [oc.fill_synthetic(n, "f32", key(2, i), 0, 1e-3) for i, n in enumerate(sizes)]
+    ms = [np.zeros(n, np.float32) for n in sizes]
+    vs = [np.zeros(n, np.float32) for n in sizes]
+    a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    best = {}
+    for fused in (False, True):
+        best[fused] = float("inf")
+        for _ in range(2):
+            t0 = time.perf_counter()
+            for p, g, m, v in zip(ps, gs, ms, vs):
+                oc.adam(p, g, m, v, a, fused=fused)
+            best[fused] = min(best[fused], time.perf_counter() - t0)
+    return {"value": round(1.0 / best[False], 4), "unit": "steps/s", "cores": oc.num_threads(), "kind": "port",
+            "sample": f"the whole list ({len(sizes)} tensors, {sum(sizes)} elements), synthetic inputs of the library's "
+                      "generator regenerated on the host, best of 2; AdamW as 13 separate float32 passes per tensor "
+                      "(adamw.rs:84-116)",
+            "fused_single_pass_value": round(1.0 / best[True], 4)}
+
+
+def measure(wl, steps, warmup):
+    """Warm-up, then `steps` timed steps bracketed by device synchronisation; per-kernel times from events."""
+    torch = wl.torch
+    for _ in range(warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    wl.kernel_events.clear()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        marks[i].record(wl.ctx.stream)
+        wl.step()
+    marks[-1].record(wl.ctx.stream)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    step_ms = sorted(a.elapsed_time(b) for a, b in zip(marks[:-1], marks[1:]))
+    n = wl.n
+    kernels = {}
+    for name, bpe in wl.bytes_per_elem.items():
+        ms = wl.kernel_ms(name)
+        if not ms:
+            continue
+        avg = sum(ms) / len(ms)
+        kernels[name] = {"avg_ms": round(avg, 4), "min_ms": round(min(ms), 4), "launches": len(ms),
+                         "bytes_per_elem": bpe, "gbps": round(bpe * n / (avg * 1e-3) / 1e9, 1)}
+    return {"elapsed": elapsed, "steps": steps, "ms_per_step": elapsed * 1e3 / steps, "steps_per_s": steps / elapsed,
+            "step_ms_sorted": step_ms, "kernels": kernels,
+            "step_gbps": wl.step_bytes_per_elem * n / (elapsed / steps) / 1e9}
+
+
+def with_workload(args, name):
+    import copy
+    a = copy.copy(args)
+    a.workload = name
+    return a
+
+
+def measured_ceiling(args, torch, mx, ctx, pool):
+    """The four bare probes on 4 x 4 GiB of the same kind of memory the workload used."""
+    wl = Workload(with_workload(args, "probes"), torch, mx, ctx, pool)
+    r = measure(wl, 5, 2)
+    wl.close()
+    k = r["kernels"]
+    return {"mix43_gbps": k["probe_mix43"]["gbps"], "copy_gbps": k["probe_copy"]["gbps"],
+            "read_gbps": k["probe_read"]["gbps"], "write_gbps": k["probe_write"]["gbps"],
+            "what": "bare float32 streaming kernels (no table, no arithmetic) over 4 GiB per stream from the same "
+                    "allocator, measured in this run; mix43 = 4 read + 3 write streams in place",
+            "profile": PROBE_PROFILE}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -565,70 +711,103 @@ def main():
         sys.exit("bench.py needs an MI355X: mxopt has no CPU path")
     torch.cuda.set_device(0)
 
-    wl = Workload(args, torch, mxopt)
-    for _ in range(args.warmup):
-        wl.step()
-    torch.cuda.synchronize()
-    wl.kernel_events.clear()
+    ctx = mxopt.Context()
+    for opt in args.option:
+        k, v = opt.split("=")
+        ctx.set_option(k, int(v))
+    pool = None
+    placement = "plain"
+    if args.placement == "pool":
+        # the arena takes the free memory but for a margin left to torch's own scratch and the runtime
+        free = torch.cuda.mem_get_info()[0]
+        pool = ctx.hbm_pool(free - (8 << 30), args.pool_chunk_mb << 20, args.pool_regions)
+        pool.use_for_state()
+        i = pool.info()
+        placement = {"kind": "mxopt_hbm_pool", "chunk_mib": i.chunk_bytes >> 20, "regions_found": i.regions,
+                     "regions_used": min(args.pool_regions, i.regions) if args.pool_regions else i.regions,
+                     "arena_gib": round(i.capacity_bytes / 2**30, 1),
+                     "region_free_gib": [round(x / 2**30, 1) for x in i.region_free_bytes[:i.regions]],
+                     "probe_same_region_gbps": round(i.probe_same_region_gbps, 1),
+                     "probe_cross_region_gbps": round(i.probe_cross_region_gbps, 1),
+                     "setup_s": round(i.setup_seconds, 2), "scan_s": round(i.scan_seconds, 2), "probes": i.probes}
+    elif args.placement == "spread":
+        placement = (f"buffers allocated between mxopt_hbm_spread_begin and _end ({args.spread_block_mb or 64} MiB "
+                     f"blocks, one in {args.spread_keep or 3} kept meanwhile)")
 
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        marks[i].record(wl.ctx.stream)
-        wl.step()
-    marks[-1].record(wl.ctx.stream)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    step_ms = sorted(a.elapsed_time(b) for a, b in zip(marks[:-1], marks[1:]))
-
-    ms_per_step = elapsed * 1e3 / args.steps
-    steps_per_s = args.steps / elapsed
+    wl = Workload(args, torch, mxopt, ctx, pool)
+    r = measure(wl, args.steps, args.warmup)
     n = wl.n
-    step_gbps = wl.step_bytes_per_elem * n / (elapsed / args.steps) / 1e9
-
-    kernels = {}
-    for name, bpe in wl.bytes_per_elem.items():
-        ms = wl.kernel_ms(name)
-        if not ms:
-            continue
-        avg = sum(ms) / len(ms)
-        kernels[name] = {"avg_ms": round(avg, 4), "min_ms": round(min(ms), 4), "launches": len(ms),
-                         "bytes_per_elem": bpe, "gbps": round(bpe * n / (avg * 1e-3) / 1e9, 1)}
+    kernels = r["kernels"]
+    step_ms = r["step_ms_sorted"]
     dom = kernels[wl.dominant]
+    key = (args.workload, int(args.fold_last))
+    have_traffic = key in MEASURED_TRAFFIC_B_PER_ELEM and args.micro == 4 and traffic_profile_is_current()
     roofline = {"bound": "hbm", "achieved": dom["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(dom["gbps"] / HBM_PEAK_GBPS, 4),
-                "traffic": (round(MEASURED_TRAFFIC_B_PER_ELEM[(args.workload, int(args.fold_last))] * n)
-                            if (args.workload, int(args.fold_last)) in MEASURED_TRAFFIC_B_PER_ELEM and args.micro == 4
-                            else None),
+                "traffic": round(MEASURED_TRAFFIC_B_PER_ELEM[key] * n) if have_traffic else None,
+                "traffic_source": (TRAFFIC_PROFILE + " (rocprofv3 FETCH_SIZE + WRITE_SIZE of an earlier run of this "
+                                   "kernel, scaled per element; not counted in this run)") if have_traffic else None,
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
     deferred = wl.deferred_variant(args.steps) if args.workload == "cfg5" else None
+    config = {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
+              "bytes_per_elem_per_step": wl.step_bytes_per_elem,
+              "storage": getattr(wl, "storage", "float32 everywhere"),
+              "note": "; ".join(x for x in (wl.note,
+                                            "the gradient buffers are generated once and reused by every step (their values do "
+                                            "not change the traffic)",
+                                            "'normal' inputs are the sum of four 16-bit uniforms: exact standard deviation, "
+                                            "|x| <= 3.46 sigma") if x),
+              "scale": args.scale, "alloc": args.alloc, "placement": placement}
+    dtype = wl.dtype
+    wl.close()
 
-    no_cpu_leg = ("copy", "grpo-engine", "sft-engine")
+    full_default = args.workload == "cfg5" and args.scale == 1.0
+    if args.workload not in ("probes", "copy"):
+        roofline["measured_ceiling"] = measured_ceiling(args, torch, mxopt, ctx, pool)
+        roofline["frac_of_measured_ceiling"] = round(dom["gbps"] / roofline["measured_ceiling"]["mix43_gbps"], 4)
+
+    others = None
+    if args.others == 1 or (args.others == -1 and full_default):
+        others = {}
+        for name in OTHER_CONFIGS:
+            a = with_workload(args, name)
+            w2 = Workload(a, torch, mxopt, ctx, pool)
+            r2 = measure(w2, args.others_steps, 2)
+            d2 = r2["kernels"][w2.dominant]
+            others[name] = {"list": w2.list_name, "tensors": len(w2.sizes), "elements": w2.n,
+                            "steps": args.others_steps, "steps_per_s": round(r2["steps_per_s"], 3),
+                            "ms_per_step": round(r2["ms_per_step"], 4),
+                            "bytes_per_elem_per_step": w2.step_bytes_per_elem,
+                            "step_hbm_gbps": round(r2["step_gbps"], 1),
+                            "dominant_kernel": w2.dominant, "dominant_kernel_ms": d2["avg_ms"],
+                            "dominant_kernel_gbps": d2["gbps"], "frac": round(d2["gbps"] / HBM_PEAK_GBPS, 4),
+                            "kernels": r2["kernels"]}
+            w2.close()
+        if args.cpu_sample > 0:
+            others["cfg1"]["cpu_baseline"] = cpu_baseline_cfg1_full()
+
+    no_cpu_leg = ("copy", "probes", "grpo-engine", "sft-engine")
     cpu = cpu_baseline(args, n) if args.cpu_sample > 0 and args.workload not in no_cpu_leg else None
 
     out = {
         "metric": "optimizer steps/s + achieved HBM GB/s (% of 8 TB/s), AdamW on Qwen3-8B shapes",
-        "value": round(steps_per_s, 4), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "ms_per_step_median": round(step_ms[len(step_ms) // 2], 4),
+        "value": round(r["steps_per_s"], 4), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["ms_per_step"], 4), "ms_per_step_median": round(step_ms[len(step_ms) // 2], 4),
         "ms_per_step_min": round(step_ms[0], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": wl.dtype, "data": "synthetic (counter-based generator of the library, seed 0x5EED0001; reproducible on the host)",
-        "config": {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
-                   "bytes_per_elem_per_step": wl.step_bytes_per_elem,
-                   "storage": getattr(wl, "storage", "float32 everywhere"), "note": wl.note, "scale": args.scale,
-                   "alloc": args.alloc,
-                   "placement": (f"buffers allocated between mxopt_hbm_spread_begin and _end "
-                                 f"({args.spread_block_mb or 64} MiB blocks, one in {args.spread_keep or 3} kept meanwhile)"
-                                 if args.placement == "spread" else "plain")},
-        "elements_per_s": round(n * steps_per_s, 1),
-        "step_hbm_gbps": round(step_gbps, 1), "step_hbm_frac": round(step_gbps / HBM_PEAK_GBPS, 4),
+        "dtype": dtype, "data": "synthetic (counter-based generator of the library, seed 0x5EED0001; reproducible on the host)",
+        "config": config,
+        "elements_per_s": round(n * r["steps_per_s"], 1),
+        "step_hbm_gbps": round(r["step_gbps"], 1), "step_hbm_frac": round(r["step_gbps"] / HBM_PEAK_GBPS, 4),
         "kernels": kernels,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
     if deferred:
         out["deferred_accumulation"] = deferred
+    if others:
+        out["other_configs"] = others
     print(json.dumps(out))
 
 

@@ -96,6 +96,71 @@ typedef struct mxopt_hbm_spread mxopt_hbm_spread;
 int mxopt_hbm_spread_begin(mxopt_ctx* ctx, size_t block_bytes, int keep_one_in, mxopt_hbm_spread** out);
 int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
 
+/* ---- region-interleaved device memory ------------------------------------------------
+ * Device memory on this part is made of three physical regions of 96 GiB.  A kernel that reads AND
+ * writes (every update and accumulation kernel here) runs at about 5.3 TB/s when all it touches lies
+ * in one region and at about 6.1 TB/s when its traffic is spread over two or three; read-only passes
+ * do not care.  A process that allocates a few tens of GB from a fresh device gets one compact
+ * physical run, i.e. one region.  Physical addresses cannot be asked for, so the pool finds the
+ * regions by timing: it takes the free memory as physical chunks, runs a 4-read/3-write probe over
+ * pairs of 1 GiB groups of them (slow = same region), maps an arena of `capacity_bytes` in which
+ * consecutive chunks alternate between the regions found, and gives every chunk it does not need
+ * back to the driver before it returns (about 1 - 3 s, once per process, at start-up; synchronises
+ * with the device).  Whatever is allocated from the arena has its traffic spread over the regions,
+ * whichever streams a kernel combines; this replaces the luck of mxopt_hbm_spread_begin/_end.
+ * If all free memory lies in one region (regions == 1 in the info) the arena still works, without
+ * the gain.  chunk_bytes = 0: 64 MiB (a power of two in [2 MiB, 1 GiB]).  max_regions = 0: alternate
+ * between all regions found; 2: between the two with the most free memory (read-only passes lose about
+ * 3 % on memory interleaved over two regions and 6 - 10 % over three, read-write passes gain 13 - 20 %
+ * either way).  Allocations are 512-byte
+ * aligned, first fit, thread-safe; contents are not cleared.  Destroy the pool after everything that
+ * allocated from it.  No counterpart in the reference (MLX owns its allocator there). */
+#define MXOPT_HBM_MAX_REGIONS 8
+typedef struct mxopt_hbm_pool mxopt_hbm_pool;
+typedef struct mxopt_hbm_pool_info {
+  uint64_t capacity_bytes;
+  uint64_t used_bytes;
+  uint64_t chunk_bytes;
+  int32_t regions;                                       /* regions found among the free memory */
+  int32_t reserved_;
+  uint64_t region_free_bytes[MXOPT_HBM_MAX_REGIONS];     /* free memory per region when the pool was made */
+  uint64_t region_arena_bytes[MXOPT_HBM_MAX_REGIONS];    /* how much of the arena lies in each */
+  double probe_same_region_gbps;                         /* the probe with all four streams in one region */
+  double probe_cross_region_gbps;                        /* ... with two of them in another (0 if regions == 1) */
+  double setup_seconds;                                  /* whole of mxopt_hbm_pool_create */
+  double create_seconds;                                 /* ... of which taking the free memory as chunks */
+  double scan_seconds;                                   /* ... and timing probes to find the regions */
+  int32_t probes;                                        /* probe measurements taken */
+  int32_t reserved2_;
+} mxopt_hbm_pool_info;
+int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
+                          mxopt_hbm_pool** out);
+void mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool);
+int mxopt_hbm_pool_alloc(mxopt_hbm_pool* pool, size_t bytes, void** out);
+int mxopt_hbm_pool_free(mxopt_hbm_pool* pool, void* ptr);
+int mxopt_hbm_pool_owns(const mxopt_hbm_pool* pool, const void* ptr);   /* 1 if ptr lies inside the arena */
+int mxopt_hbm_pool_get_info(mxopt_hbm_pool* pool, mxopt_hbm_pool_info* out);
+/* The memory the library itself owns on behalf of the reference's objects -- the optimizers' moments
+ * (init_state: adam.rs:148-153, adamw.rs:152-157, rmsprop.rs:123-127), the engines' accumulation buffers
+ * (grpo/engine.rs:2632-2666, sft/engine.rs:282-306) -- is taken from `pool` while it has room (NULL: from
+ * the driver again).  Objects created before the call keep what they have. */
+int mxopt_set_state_pool(mxopt_ctx* ctx, mxopt_hbm_pool* pool);
+/* For hosts whose allocator takes plug-in functions (torch's CUDAPluggableAllocator has exactly these
+ * signatures): allocations on the target pool's device come from its arena while it has room and from
+ * hipMalloc otherwise; frees find their way back by address. */
+int mxopt_hbm_pool_set_hook_target(mxopt_hbm_pool* pool);
+void* mxopt_hbm_pool_hook_alloc(ptrdiff_t size, int device, void* stream);
+void mxopt_hbm_pool_hook_free(void* ptr, ptrdiff_t size, int device, void* stream);
+
+/* ---- bare streaming probes ------------------------------------------------------------
+ * The measured ceilings the update kernels are compared with: float32 buffers of n_elems elements
+ * (a positive multiple of 4096, 16-byte aligned), no table, no tails, no arithmetic to speak of.
+ *   MXOPT_PROBE_READ   reads a                       MXOPT_PROBE_WRITE  writes a
+ *   MXOPT_PROBE_COPY   reads a, writes b             MXOPT_PROBE_MIX43  reads a, b, c, d and writes a, c, d
+ * (MIX43 is float32 AdamW's byte mix, 28 B/elem.)  One launch on the context's stream. */
+enum { MXOPT_PROBE_READ = 0, MXOPT_PROBE_WRITE = 1, MXOPT_PROBE_COPY = 2, MXOPT_PROBE_MIX43 = 3 };
+int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n_elems);
+
 /* ---- tensor table ------------------------------------------------------------------
  * One descriptor per tensor.  Which fields a kernel reads is listed at that kernel;
  * unused pointers may be NULL.  All buffers are dense, `n` elements long.

@@ -22,7 +22,7 @@ OUT = os.path.join(HERE, "mxopt_sys.rs")
 
 SCALARS = {
     "void": "c_void", "char": "c_char", "int": "c_int", "float": "f32", "double": "f64", "size_t": "usize",
-    "uint8_t": "u8", "uint32_t": "u32", "int32_t": "i32", "uint64_t": "u64", "int64_t": "i64",
+    "uint8_t": "u8", "uint32_t": "u32", "int32_t": "i32", "uint64_t": "u64", "int64_t": "i64", "ptrdiff_t": "isize",
 }
 RUST_KEYWORDS = {"type", "ref", "in", "fn", "loop", "match", "move", "mod", "use", "where", "self", "box"}
 
@@ -86,8 +86,8 @@ def parse(text: str):
             decl = " ".join(decl.split())
             if not decl:
                 continue
-            # `float bc1, bc2` and `const void* p`
-            mm = re.match(r"(.+?[\s\*])([\w\s,]+)$", decl)
+            # `float bc1, bc2`, `const void* p` and `uint64_t per_region[MXOPT_N]`
+            mm = re.match(r"(.+?[\s\*])([\w\s,\[\]]+)$", decl)
             ctype, names = mm.group(1).strip(), [n.strip() for n in mm.group(2).split(",")]
             for n in names:
                 fields.append((ctype, n))
@@ -153,7 +153,11 @@ def generate() -> str:
         for sname, fields in s:
             out += ["#[repr(C)]", "#[derive(Clone, Copy)]", f"pub struct {sname} {{"]
             for ctype, fname in fields:
-                out.append(f"    pub {ident(fname)}: {rust_type(ctype, opaque, struct_names)},")
+                rt = rust_type(ctype, opaque, struct_names)
+                arr = re.match(r"(\w+)\[(\w+)\]$", fname)
+                if arr:     # fixed-size array member
+                    fname, rt = arr.group(1), f"[{rt}; {arr.group(2)} as usize]"
+                out.append(f"    pub {ident(fname)}: {rt},")
             out += ["}", ""]
         out.append('extern "C" {')
         for ret, fname, params in f:

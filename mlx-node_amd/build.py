@@ -17,7 +17,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxopt.so")
 
-SOURCES = ["mxopt_kernels.hip", "mxopt_reduce_kernels.hip", "mxopt_list_kernels.hip", "mxopt_list_kernels_sgd_rmsprop.hip",
+SOURCES = ["mxopt_kernels.hip", "mxopt_reduce_kernels.hip", "mxopt_list_kernels.hip", "mxopt_list_kernels_sgd_rmsprop.hip", "mxopt_hbm_pool.hip",
            "mxopt_api.cpp",
            "mxopt_optimizers.cpp", "mxopt_engine.cpp", "mxopt_checkpoint.cpp"]
 

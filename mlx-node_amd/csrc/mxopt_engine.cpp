@@ -95,10 +95,10 @@ int ensure_acc(mxopt_engine* e, Slot& s, int dtype) {
   DeviceGuard guard(e->ctx->device);
   if (s.acc) {
     HIP_TRY(e->ctx, hipStreamSynchronize(e->ctx->stream));
-    (void)hipFree(s.acc);
+    state_free(e->ctx, s.acc);
     s.acc = nullptr;
   }
-  if (s.param.n) HIP_TRY(e->ctx, hipMalloc(&s.acc, s.param.n * (size_t)dtype_bytes(dtype)));
+  if (s.param.n) HIP_TRY(e->ctx, state_alloc(e->ctx, &s.acc, s.param.n * (size_t)dtype_bytes(dtype)));
   s.acc_dtype = dtype;
   return MXOPT_OK;
 }
@@ -807,7 +807,7 @@ void mxopt_engine_free(mxopt_engine* e) {
   DeviceGuard guard(e->ctx->device);
   (void)hipStreamSynchronize(e->ctx->stream);
   for (Slot& s : e->slots)
-    if (s.acc) (void)hipFree(s.acc);
+    state_free(e->ctx, s.acc);
   if (e->d_result) (void)hipFree(e->d_result);
   if (e->adamw) mxopt_optimizer_free(e->adamw);
   delete e;

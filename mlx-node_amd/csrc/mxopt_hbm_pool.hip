@@ -1,0 +1,599 @@
+// Bare streaming probes (the measured ceilings the update kernels are compared with) and the
+// region-interleaved device-memory pool.
+//
+// What the pool is for.  Device memory on this part consists of three physical regions of 96 GiB.
+// A kernel that reads and writes several streams runs at about 5.3 TB/s when everything it touches
+// lies in one region and at about 6.1 TB/s when its traffic is spread over two or three of them
+// (read-only streams do not care).  A fresh process that allocates a few tens of GB gets one compact
+// physical run, i.e. one region.  The pool takes the free memory as physical chunks (64 MiB), finds
+// out by timing which chunks share a region, and maps an arena in which consecutive chunks alternate
+// between the regions; everything allocated from the arena then has its traffic spread evenly
+// whatever streams a kernel combines.  The physical memory it does not need goes back to the driver
+// before mxopt_hbm_pool_create returns.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <unordered_map>
+#include <vector>
+
+#include "mxopt_internal.h"
+
+namespace mxopt {
+
+typedef uint32_t pu32x4 __attribute__((ext_vector_type(4)));
+constexpr int kProbeThreads = 256;
+constexpr int kProbeVecs = 4;                                    // 16-byte pieces per lane per stream
+constexpr uint64_t kProbeTileElems = kProbeThreads * kProbeVecs * 4;  // float32 elements per workgroup trip
+
+// One read stream.
+__global__ __launch_bounds__(kProbeThreads) void probe_read_kernel(const pu32x4* __restrict__ a, uint32_t ntiles,
+                                                                  uint32_t* __restrict__ sink) {
+  uint32_t s = 0;
+  for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
+    pu32x4 r[kProbeVecs];
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) r[j] = __builtin_nontemporal_load(a + b + j * kProbeThreads);
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) s ^= r[j].x ^ r[j].y ^ r[j].z ^ r[j].w;
+  }
+  if (s == 0x9E3779B9u && sink != nullptr) *sink = s;  // keeps the loads alive
+}
+
+// One write stream.
+__global__ __launch_bounds__(kProbeThreads) void probe_write_kernel(pu32x4* __restrict__ a, uint32_t ntiles) {
+  for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
+    const pu32x4 r = {t, t, t, t};
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) a[b + j * kProbeThreads] = r;
+  }
+}
+
+// One read and one write stream.
+__global__ __launch_bounds__(kProbeThreads) void probe_copy_kernel(const pu32x4* __restrict__ a, pu32x4* __restrict__ o,
+                                                                  uint32_t ntiles) {
+  for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
+    pu32x4 r[kProbeVecs];
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) r[j] = a[b + j * kProbeThreads];
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) o[b + j * kProbeThreads] = r[j];
+  }
+}
+
+// AdamW's float32 byte mix without its arithmetic: reads a, b, c, d; writes a, c, d in place.
+__global__ __launch_bounds__(kProbeThreads) void probe_mix43_kernel(pu32x4* __restrict__ a, const pu32x4* __restrict__ g,
+                                                                   pu32x4* __restrict__ c, pu32x4* __restrict__ d,
+                                                                   uint32_t ntiles) {
+  for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
+    pu32x4 ra[kProbeVecs], rg[kProbeVecs], rc[kProbeVecs], rd[kProbeVecs];
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) {
+      ra[j] = a[b + j * kProbeThreads]; rg[j] = g[b + j * kProbeThreads];
+      rc[j] = c[b + j * kProbeThreads]; rd[j] = d[b + j * kProbeThreads];
+    }
+#pragma unroll
+    for (int j = 0; j < kProbeVecs; ++j) {
+      a[b + j * kProbeThreads] = ra[j] ^ rg[j];
+      c[b + j * kProbeThreads] = rc[j] + rg[j];
+      d[b + j * kProbeThreads] = rd[j] ^ (rg[j] >> 1);
+    }
+  }
+}
+
+static int launch_probe(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n) {
+  const uint32_t ntiles = (uint32_t)(n / kProbeTileElems);
+  const uint32_t bounded = (uint32_t)std::min<uint64_t>(ntiles, (uint64_t)ctx->num_cus * 16u);
+  switch (kind) {
+    case MXOPT_PROBE_READ:
+      hipLaunchKernelGGL(probe_read_kernel, dim3(bounded), dim3(kProbeThreads), 0, ctx->stream, (const pu32x4*)a, ntiles,
+                         (uint32_t*)nullptr);
+      break;
+    case MXOPT_PROBE_WRITE:
+      hipLaunchKernelGGL(probe_write_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a, ntiles);
+      break;
+    case MXOPT_PROBE_COPY:
+      hipLaunchKernelGGL(probe_copy_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (const pu32x4*)a,
+                         (pu32x4*)b, ntiles);
+      break;
+    case MXOPT_PROBE_MIX43:
+      hipLaunchKernelGGL(probe_mix43_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a,
+                         (const pu32x4*)b, (pu32x4*)c, (pu32x4*)d, ntiles);
+      break;
+    default:
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: unknown kind");
+  }
+  return check_launch(ctx, "mxopt_probe_stream");
+}
+
+}  // namespace mxopt
+
+using namespace mxopt;
+
+// ---------------------------------------------------------------------------------------
+// The pool
+// ---------------------------------------------------------------------------------------
+
+struct mxopt_hbm_pool {
+  mxopt_ctx* ctx = nullptr;
+  size_t chunk = 0;
+  std::vector<hipMemGenericAllocationHandle_t> handles;  // the arena's chunks, in address order
+  char* base = nullptr;
+  size_t capacity = 0;
+  std::map<size_t, size_t> free_list;                    // offset -> bytes, coalesced
+  std::unordered_map<size_t, size_t> live;               // offset -> bytes
+  std::mutex mu;
+  mxopt_hbm_pool_info info{};
+};
+
+namespace {
+
+constexpr size_t kAlign = 512;
+constexpr size_t kSlabChunksBytes = (size_t)1 << 30;  // chunks are classified in groups of this many bytes
+
+struct Builder {  // everything pool creation holds until it either succeeds or fails
+  mxopt_ctx* ctx;
+  std::vector<hipMemGenericAllocationHandle_t> all;
+  std::vector<char> released;
+  void* probe_va = nullptr;
+  size_t probe_bytes = 0;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  ~Builder() {
+    if (probe_va) {
+      // after an error some of it may still be mapped; on the normal path these two fail harmlessly
+      (void)hipMemUnmap(probe_va, probe_bytes / 2);
+      (void)hipMemUnmap((char*)probe_va + probe_bytes / 2, probe_bytes / 2);
+      (void)hipGetLastError();
+      (void)hipMemAddressFree(probe_va, probe_bytes);
+    }
+    for (size_t i = 0; i < all.size(); ++i)
+      if (!released[i]) (void)hipMemRelease(all[i]);
+    if (ev0) (void)hipEventDestroy(ev0);
+    if (ev1) (void)hipEventDestroy(ev1);
+  }
+};
+
+hipMemAllocationProp device_prop(int device) {
+  hipMemAllocationProp prop = {};
+  prop.type = hipMemAllocationTypePinned;
+  prop.location.type = hipMemLocationTypeDevice;
+  prop.location.id = device;
+  return prop;
+}
+
+hipMemAccessDesc rw_access(int device) {
+  hipMemAccessDesc acc = {};
+  acc.location.type = hipMemLocationTypeDevice;
+  acc.location.id = device;
+  acc.flags = hipMemAccessFlagsProtReadWrite;
+  return acc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n_elems) {
+  if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: null context");
+  if (n_elems == 0 || n_elems % kProbeTileElems != 0 || n_elems / kProbeTileElems > 0xffffffffull)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: n_elems must be a positive multiple of 4096");
+  const int need = kind == MXOPT_PROBE_MIX43 ? 4 : kind == MXOPT_PROBE_COPY ? 2 : 1;
+  void* ptrs[4] = {a, b, c, d};
+  for (int i = 0; i < need; ++i)
+    if (!ptrs[i] || (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: buffers must be non-NULL and 16-byte aligned");
+  DeviceGuard guard(ctx->device);
+  return launch_probe(ctx, kind, a, b, c, d, n_elems);
+}
+
+int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
+                          mxopt_hbm_pool** out) {
+  const char* op = "mxopt_hbm_pool_create";
+  if (!ctx || !out) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
+  *out = nullptr;
+  if (chunk_bytes == 0) chunk_bytes = (size_t)64 << 20;
+  if (chunk_bytes < ((size_t)2 << 20) || (chunk_bytes & (chunk_bytes - 1)) || chunk_bytes > kSlabChunksBytes)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": chunk_bytes must be a power of two in [2 MiB, 1 GiB]");
+  if (capacity_bytes == 0) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": capacity_bytes is 0");
+  if (max_regions < 0) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": max_regions is negative");
+  const auto t_begin = std::chrono::steady_clock::now();
+  DeviceGuard guard(ctx->device);
+  HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+  size_t free_b = 0, total_b = 0;
+  HIP_TRY(ctx, hipMemGetInfo(&free_b, &total_b));
+  const size_t margin = (size_t)1 << 30;  // left to the runtime
+  const size_t want_chunks = (capacity_bytes + chunk_bytes - 1) / chunk_bytes;
+  const size_t avail_chunks = free_b > margin ? (free_b - margin) / chunk_bytes : 0;
+  if (want_chunks > avail_chunks)
+    return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": " + std::to_string(capacity_bytes >> 20) + " MiB wanted, " +
+                                        std::to_string(free_b >> 20) + " MiB free");
+  if (avail_chunks > 60000)  // the driver limits the number of live allocations of a process
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": chunk_bytes too small for this much free memory");
+
+  // 1. All free memory as physical chunks: memory far from what a small allocation would get can
+  //    only be reached by holding what lies in between.
+  Builder b{ctx};
+  const hipMemAllocationProp prop = device_prop(ctx->device);
+  b.all.reserve(avail_chunks);
+  for (size_t i = 0; i < avail_chunks; ++i) {
+    hipMemGenericAllocationHandle_t h;
+    if (hipMemCreate(&h, chunk_bytes, &prop, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      break;
+    }
+    b.all.push_back(h);
+  }
+  b.released.assign(b.all.size(), 0);
+  const auto t_created = std::chrono::steady_clock::now();
+  int probes = 0;
+  if (b.all.size() < want_chunks)
+    return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": the driver handed out fewer chunks than the capacity needs");
+
+  // 2. Which chunks share a region?  Chunks are judged in creation-order groups of 1 GiB ("slabs"):
+  //    the 4-read/3-write probe runs with two of its streams in a reference slab and two in the slab
+  //    under test; it is slow when both lie in one region.
+  const size_t per_slab = kSlabChunksBytes / chunk_bytes;
+  const size_t nslab = b.all.size() / per_slab;
+  std::vector<int> slab_region(nslab, 0);
+  int nregions = 1;
+  double same_gbps = 0.0, cross_gbps = 0.0;
+  if (nslab >= 4) {
+    const hipMemAccessDesc acc = rw_access(ctx->device);
+    b.probe_bytes = 2 * kSlabChunksBytes;
+    HIP_TRY(ctx, hipMemAddressReserve(&b.probe_va, b.probe_bytes, 0, nullptr, 0));
+    HIP_TRY(ctx, hipEventCreate(&b.ev0));
+    HIP_TRY(ctx, hipEventCreate(&b.ev1));
+    char* va_ref = (char*)b.probe_va;
+    char* va_x = va_ref + kSlabChunksBytes;
+    const uint64_t stream_elems = kSlabChunksBytes / 2 / 4;  // two streams per slab
+    auto map_slab = [&](char* va, size_t slab) -> hipError_t {
+      for (size_t k = 0; k < per_slab; ++k) {
+        hipError_t e = hipMemMap(va + k * chunk_bytes, chunk_bytes, 0, b.all[slab * per_slab + k], 0);
+        if (e != hipSuccess) return e;
+      }
+      return hipMemSetAccess(va, kSlabChunksBytes, &acc, 1);
+    };
+    // Rate of the probe with streams p, g in the (already mapped) reference slab and m, v in slab x.
+    auto probe_against_ref = [&](int x, double* out) -> int {
+      hipError_t e = map_slab(va_x, (size_t)x);
+      if (e != hipSuccess) return hip_fail(ctx, e, "mxopt_hbm_pool_create: mapping a slab");
+      void* p = va_ref;
+      void* g = va_ref + kSlabChunksBytes / 2;
+      void* m = va_x;
+      void* v = va_x + kSlabChunksBytes / 2;
+      int rc = launch_probe(ctx, MXOPT_PROBE_MIX43, p, g, m, v, stream_elems);
+      if (rc) return rc;
+      HIP_TRY(ctx, hipEventRecord(b.ev0, ctx->stream));
+      for (int rep = 0; rep < 2 && !rc; ++rep) rc = launch_probe(ctx, MXOPT_PROBE_MIX43, p, g, m, v, stream_elems);
+      if (rc) return rc;
+      HIP_TRY(ctx, hipEventRecord(b.ev1, ctx->stream));
+      HIP_TRY(ctx, hipEventSynchronize(b.ev1));
+      float ms = 0.f;
+      HIP_TRY(ctx, hipEventElapsedTime(&ms, b.ev0, b.ev1));
+      *out = 2.0 * 7.0 * (double)(kSlabChunksBytes / 2) / 1e9 / ((double)ms * 1e-3);
+      ++probes;
+      HIP_TRY(ctx, hipMemUnmap(va_x, kSlabChunksBytes));
+      return MXOPT_OK;
+    };
+    std::vector<int> todo(nslab);
+    for (size_t i = 0; i < nslab; ++i) todo[i] = (int)i;
+    std::vector<double> rate(nslab);
+    double abs_thr = 0.0;  // rate that separates "same region" from "another region", once one scan has shown both
+    int region = 0, attempts = 0;
+    while (!todo.empty() && region < MXOPT_HBM_MAX_REGIONS) {
+      if (todo.size() < 4) {  // a few boundary slabs are no region of their own
+        for (int x : todo) slab_region[x] = std::max(region - 1, 0);
+        todo.clear();
+        break;
+      }
+      // The reference must lie inside one region; a slab that straddles a boundary makes everything look
+      // fast.  First try the first slab, after a suspicious scan one further into the list.
+      const size_t ref_pos = std::min(todo.size() - 1, todo.size() * (size_t)attempts / 4);
+      const int ref = todo[ref_pos];
+      std::vector<int> others;
+      for (size_t i = 0; i < todo.size(); ++i) if (i != ref_pos) others.push_back(todo[i]);
+      hipError_t me = map_slab(va_ref, (size_t)ref);
+      if (me != hipSuccess) return hip_fail(ctx, me, "mxopt_hbm_pool_create: mapping a slab");
+      // Coarse scan (creation order is close to physical order, regions are long runs), refined below
+      // wherever two scanned neighbours disagree.
+      const size_t stride = 4;
+      std::vector<char> probed(others.size(), 0);
+      double lo = 1e30, hi = 0.0;
+      auto scan = [&](size_t k) -> int {
+        if (probed[k]) return MXOPT_OK;
+        int rc = probe_against_ref(others[k], &rate[others[k]]);
+        if (rc) return rc;
+        probed[k] = 1;
+        lo = std::min(lo, rate[others[k]]);
+        hi = std::max(hi, rate[others[k]]);
+        return MXOPT_OK;
+      };
+      for (size_t k = 0; k < others.size(); k += stride) { int rc = scan(k); if (rc) return rc; }
+      { int rc = scan(others.size() - 1); if (rc) return rc; }
+      const bool uniform = hi < lo * 1.07;
+      const double level = 0.5 * (lo + hi);
+      if (uniform) {
+        HIP_TRY(ctx, hipMemUnmap(va_ref, kSlabChunksBytes));
+        const bool straddler = abs_thr > 0.0 ? level > abs_thr : attempts < 2;
+        if (straddler && attempts < 3) {
+          if (abs_thr > 0.0) {  // known to be fast against everything: a boundary slab, lumped with its predecessors
+            slab_region[ref] = std::max(region - 1, 0);
+            todo.erase(todo.begin() + (ptrdiff_t)ref_pos);
+          }
+          ++attempts;
+          continue;
+        }
+        for (int x : todo) slab_region[x] = region;  // they all share the reference's region
+        if (abs_thr == 0.0) same_gbps = level;
+        ++region;
+        todo.clear();
+        break;
+      }
+      const double thr = abs_thr > 0.0 ? abs_thr : level;
+      for (size_t k = 0; k + 1 < others.size();) {  // refine between scanned neighbours that disagree
+        size_t k2 = k + 1;
+        while (!probed[k2]) ++k2;
+        if ((rate[others[k]] < thr) != (rate[others[k2]] < thr))
+          for (size_t q = k + 1; q < k2; ++q) { int rc = scan(q); if (rc) return rc; }
+        k = k2;
+      }
+      HIP_TRY(ctx, hipMemUnmap(va_ref, kSlabChunksBytes));
+      if (abs_thr == 0.0) { abs_thr = thr; same_gbps = lo; cross_gbps = hi; }
+      std::vector<int> rest;
+      bool same = true;
+      for (size_t k = 0; k < others.size(); ++k) {
+        if (probed[k]) same = rate[others[k]] < thr;  // slabs between two agreeing neighbours inherit
+        if (same) slab_region[others[k]] = region;
+        else rest.push_back(others[k]);
+      }
+      slab_region[ref] = region;
+      ++region;
+      attempts = 0;
+      todo.swap(rest);
+    }
+    nregions = std::max(region, 1);
+    for (int s : todo) slab_region[s] = nregions - 1;  // more groups than MXOPT_HBM_MAX_REGIONS: lumped together
+  }
+
+  const auto t_scanned = std::chrono::steady_clock::now();
+
+  // 3. The arena: consecutive chunks alternate between the regions for as long as each has chunks.
+  std::vector<std::vector<size_t>> by_region(nregions);
+  for (size_t i = 0; i < b.all.size(); ++i) {
+    const size_t slab = i / per_slab;
+    by_region[slab < nslab ? slab_region[slab] : slab_region.empty() ? 0 : slab_region[nslab - 1]].push_back(i);
+  }
+  // Regions by free memory, largest first.  Groups holding under a tenth of the chunks are leftovers of the
+  // scan (slabs whose chunks straddle regions when the free memory was fragmented): they serve last and
+  // are not counted.  With max_regions, only that many of the largest take part in the alternation.
+  std::vector<int> rank(nregions);
+  for (int r = 0; r < nregions; ++r) rank[r] = r;
+  std::stable_sort(rank.begin(), rank.end(), [&](int a, int c) { return by_region[a].size() > by_region[c].size(); });
+  int real_regions = 0;
+  for (int k = 0; k < nregions; ++k)
+    if (by_region[rank[k]].size() * 10 >= b.all.size()) ++real_regions;
+  real_regions = std::max(real_regions, 1);
+  const int active = max_regions > 0 ? std::min(max_regions, real_regions) : real_regions;
+  std::vector<size_t> order;
+  order.reserve(want_chunks);
+  std::vector<size_t> next(nregions, 0);
+  for (int lo_rank = 0; lo_rank < nregions && order.size() < want_chunks;) {
+    const int hi_rank = lo_rank == 0 ? active : nregions;  // first the alternation, then whatever is left
+    for (bool any = true; any && order.size() < want_chunks;) {
+      any = false;
+      for (int k = lo_rank; k < hi_rank && order.size() < want_chunks; ++k) {
+        const int r = rank[k];
+        if (next[r] < by_region[r].size()) {
+          order.push_back(by_region[r][next[r]++]);
+          any = true;
+        }
+      }
+    }
+    lo_rank = hi_rank;
+  }
+  if (order.size() < want_chunks) return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": ran out of chunks");
+
+  mxopt_hbm_pool* pool = new (std::nothrow) mxopt_hbm_pool();
+  if (!pool) return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": out of host memory");
+  pool->ctx = ctx;
+  pool->chunk = chunk_bytes;
+  pool->capacity = want_chunks * chunk_bytes;
+  void* base = nullptr;
+  hipError_t e = hipMemAddressReserve(&base, pool->capacity, 0, nullptr, 0);
+  if (e != hipSuccess) { delete pool; return hip_fail(ctx, e, "mxopt_hbm_pool_create: hipMemAddressReserve"); }
+  pool->base = (char*)base;
+  size_t mapped = 0;
+  for (; mapped < order.size(); ++mapped) {
+    e = hipMemMap(pool->base + mapped * chunk_bytes, chunk_bytes, 0, b.all[order[mapped]], 0);
+    if (e != hipSuccess) break;
+  }
+  if (e == hipSuccess) {
+    const hipMemAccessDesc acc = rw_access(ctx->device);
+    e = hipMemSetAccess(pool->base, pool->capacity, &acc, 1);
+  }
+  if (e != hipSuccess) {
+    if (mapped) (void)hipMemUnmap(pool->base, mapped * chunk_bytes);
+    (void)hipMemAddressFree(pool->base, pool->capacity);
+    delete pool;
+    return hip_fail(ctx, e, "mxopt_hbm_pool_create: mapping the arena");
+  }
+  for (size_t k = 0; k < order.size(); ++k) {
+    pool->handles.push_back(b.all[order[k]]);
+    b.released[order[k]] = 1;  // now owned by the pool; everything else goes back to the driver with `b`
+  }
+  pool->free_list[0] = pool->capacity;
+  mxopt_hbm_pool_info& info = pool->info;
+  info.capacity_bytes = pool->capacity;
+  info.chunk_bytes = chunk_bytes;
+  info.regions = real_regions;
+  for (int k = 0; k < nregions && k < MXOPT_HBM_MAX_REGIONS; ++k) {  // largest first; entries past `regions` are leftovers
+    info.region_free_bytes[k] = by_region[rank[k]].size() * chunk_bytes;
+    info.region_arena_bytes[k] = next[rank[k]] * chunk_bytes;
+  }
+  info.probe_same_region_gbps = same_gbps;
+  info.probe_cross_region_gbps = cross_gbps;
+  for (size_t i = 0; i < b.all.size(); ++i)   // what the arena does not use goes back to the driver now
+    if (!b.released[i]) { (void)hipMemRelease(b.all[i]); b.released[i] = 1; }
+  const auto t_end = std::chrono::steady_clock::now();
+  info.setup_seconds = std::chrono::duration<double>(t_end - t_begin).count();
+  info.create_seconds = std::chrono::duration<double>(t_created - t_begin).count();
+  info.scan_seconds = std::chrono::duration<double>(t_scanned - t_created).count();
+  info.probes = probes;
+  MXOPT_DEBUG("hbm pool: %zu MiB arena of %zu MiB chunks over %d region(s); probe %.0f GB/s inside one region, %.0f across; %.2f s",
+              pool->capacity >> 20, chunk_bytes >> 20, nregions, same_gbps, cross_gbps, info.setup_seconds);
+  *out = pool;
+  return MXOPT_OK;
+}
+
+void mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool) {
+  if (!pool) return;
+  {
+    DeviceGuard guard(pool->ctx->device);
+    (void)hipStreamSynchronize(pool->ctx->stream);
+    if (pool->base) {
+      (void)hipMemUnmap(pool->base, pool->capacity);
+      (void)hipMemAddressFree(pool->base, pool->capacity);
+    }
+    for (auto h : pool->handles) (void)hipMemRelease(h);
+    if (pool->ctx->state_pool == pool) pool->ctx->state_pool = nullptr;
+  }
+  delete pool;
+}
+
+// First fit; NULL when no free range is large enough.
+static void* pool_try_alloc(mxopt_hbm_pool* pool, size_t bytes) {
+  const size_t need = std::max<size_t>((bytes + kAlign - 1) / kAlign * kAlign, kAlign);
+  std::lock_guard<std::mutex> lock(pool->mu);
+  for (auto it = pool->free_list.begin(); it != pool->free_list.end(); ++it) {
+    if (it->second < need) continue;
+    const size_t off = it->first, left = it->second - need;
+    pool->free_list.erase(it);
+    if (left) pool->free_list[off + need] = left;
+    pool->live[off] = need;
+    return pool->base + off;
+  }
+  return nullptr;
+}
+
+int mxopt_hbm_pool_alloc(mxopt_hbm_pool* pool, size_t bytes, void** out) {
+  if (!pool || !out) return fail(pool ? pool->ctx : nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_alloc: null argument");
+  *out = pool_try_alloc(pool, bytes);
+  if (*out) return MXOPT_OK;
+  return fail(pool->ctx, MXOPT_ERR_OOM, "mxopt_hbm_pool_alloc: the arena has no free range of " + std::to_string(bytes) + " bytes");
+}
+
+int mxopt_hbm_pool_free(mxopt_hbm_pool* pool, void* ptr) {
+  if (!pool) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_free: null pool");
+  if (!ptr) return MXOPT_OK;
+  std::lock_guard<std::mutex> lock(pool->mu);
+  const size_t off = (size_t)((char*)ptr - pool->base);
+  auto it = pool->live.find(off);
+  if ((char*)ptr < pool->base || it == pool->live.end())
+    return fail(pool->ctx, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_free: not a live allocation of this pool");
+  size_t begin = off, size = it->second;
+  pool->live.erase(it);
+  auto nextf = pool->free_list.lower_bound(begin);
+  if (nextf != pool->free_list.end() && nextf->first == begin + size) {
+    size += nextf->second;
+    nextf = pool->free_list.erase(nextf);
+  }
+  if (nextf != pool->free_list.begin()) {
+    auto prev = std::prev(nextf);
+    if (prev->first + prev->second == begin) {
+      begin = prev->first;
+      size += prev->second;
+      pool->free_list.erase(prev);
+    }
+  }
+  pool->free_list[begin] = size;
+  return MXOPT_OK;
+}
+
+int mxopt_hbm_pool_owns(const mxopt_hbm_pool* pool, const void* ptr) {
+  return pool && ptr && (const char*)ptr >= pool->base && (const char*)ptr < pool->base + pool->capacity;
+}
+
+int mxopt_hbm_pool_get_info(mxopt_hbm_pool* pool, mxopt_hbm_pool_info* out) {
+  if (!pool || !out) return fail(pool ? pool->ctx : nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_get_info: null argument");
+  std::lock_guard<std::mutex> lock(pool->mu);
+  *out = pool->info;
+  size_t used = 0;
+  for (auto& kv : pool->live) used += kv.second;
+  out->used_bytes = used;
+  return MXOPT_OK;
+}
+
+int mxopt_set_state_pool(mxopt_ctx* ctx, mxopt_hbm_pool* pool) {
+  if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_set_state_pool: null context");
+  if (pool && pool->ctx->device != ctx->device)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_state_pool: the pool lives on another device");
+  ctx->state_pool = pool;
+  return MXOPT_OK;
+}
+
+// ---- hooks with the signature host allocators plug in (torch's CUDAPluggableAllocator) ------------
+
+static std::mutex g_hook_mu;
+static mxopt_hbm_pool* g_hook_pool = nullptr;
+
+int mxopt_hbm_pool_set_hook_target(mxopt_hbm_pool* pool) {
+  std::lock_guard<std::mutex> lock(g_hook_mu);
+  g_hook_pool = pool;
+  return MXOPT_OK;
+}
+
+void* mxopt_hbm_pool_hook_alloc(ptrdiff_t size, int device, void* stream) {
+  (void)stream;
+  mxopt_hbm_pool* pool;
+  {
+    std::lock_guard<std::mutex> lock(g_hook_mu);
+    pool = g_hook_pool;
+  }
+  void* p = nullptr;
+  if (pool && pool->ctx->device == device && (p = pool_try_alloc(pool, (size_t)size)) != nullptr) return p;
+  int prev = -1;                              // arena full, or no pool: plain device memory
+  (void)hipGetDevice(&prev);
+  if (prev != device) (void)hipSetDevice(device);
+  if (hipMalloc(&p, (size_t)size) != hipSuccess) { (void)hipGetLastError(); p = nullptr; }
+  if (prev >= 0 && prev != device) (void)hipSetDevice(prev);
+  return p;
+}
+
+void mxopt_hbm_pool_hook_free(void* ptr, ptrdiff_t size, int device, void* stream) {
+  (void)size; (void)device; (void)stream;
+  mxopt_hbm_pool* pool;
+  {
+    std::lock_guard<std::mutex> lock(g_hook_mu);
+    pool = g_hook_pool;
+  }
+  if (pool && mxopt_hbm_pool_owns(pool, ptr)) { (void)mxopt_hbm_pool_free(pool, ptr); return; }
+  (void)hipFree(ptr);
+}
+
+}  // extern "C"
+
+namespace mxopt {
+
+// Device memory the host layer owns (moments, accumulation buffers): from the context's pool when one
+// is attached and has room, else from the driver.
+hipError_t state_alloc(mxopt_ctx* ctx, void** out, size_t bytes) {
+  *out = nullptr;
+  if (ctx->state_pool && (*out = pool_try_alloc(ctx->state_pool, bytes)) != nullptr) return hipSuccess;
+  return hipMalloc(out, bytes);
+}
+
+void state_free(mxopt_ctx* ctx, void* ptr) {
+  if (!ptr) return;
+  if (ctx->state_pool && mxopt_hbm_pool_owns(ctx->state_pool, ptr)) { (void)mxopt_hbm_pool_free(ctx->state_pool, ptr); return; }
+  (void)hipFree(ptr);
+}
+
+}  // namespace mxopt

@@ -68,6 +68,7 @@ struct Group {
 }  // namespace mxopt
 
 struct mxopt_table;
+struct mxopt_hbm_pool;
 
 struct mxopt_ctx {
   int device = 0;
@@ -81,6 +82,7 @@ struct mxopt_ctx {
   size_t partial_cap = 0;
   double* d_static_partials = nullptr;        // this device's copy of the library's fixed partial-sum array
   mxopt_norm_result* d_norm_scratch = nullptr;  // result slot of the gradient utilities
+  mxopt_hbm_pool* state_pool = nullptr;         // where the host layer takes moments and accumulation buffers from
   struct CachedTable {                          // tables built by the host layer, most recent last
     std::vector<mxopt_tensor> key;
     mxopt_table* table;

@@ -65,6 +65,11 @@ uint64_t chunks_of(const DevTensor& d);  // chunk-table entries (= workgroups of
 Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool persistent);
 
 
+// Device memory the host layer owns (moments, accumulation buffers): from the context's pool
+// (mxopt_set_state_pool) while it has room, else from the driver.
+hipError_t state_alloc(mxopt_ctx* ctx, void** out, size_t bytes);
+void state_free(mxopt_ctx* ctx, void* ptr);
+
 // Shared by the host-layer translation units (mxopt_optimizers.cpp, mxopt_engine.cpp).
 mxopt_tensor blank_tensor();  // all pointers NULL, bc1 = bc2 = 1
 int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, bool allow_null_data = false);

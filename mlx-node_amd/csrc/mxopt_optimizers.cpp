@@ -125,9 +125,9 @@ void free_state(mxopt_optimizer* o) {
     o->many_key.clear();
   }
   for (auto& kv : o->state) {
-    if (kv.second.m) (void)hipFree(kv.second.m);
-    if (kv.second.v) (void)hipFree(kv.second.v);
-    if (kv.second.sum) (void)hipFree(kv.second.sum);
+    state_free(o->ctx, kv.second.m);
+    state_free(o->ctx, kv.second.v);
+    state_free(o->ctx, kv.second.sum);
   }
   o->state.clear();
 }
@@ -150,17 +150,17 @@ int get_state(mxopt_optimizer* o, const char* name, uint64_t n, StateEntry** out
   const bool need_v = o->kind != Kind::Sgd || o->momentum != 0.0;
   if (n) {
     if (is_adam(o)) {
-      HIP_TRY(ctx, hipMalloc((void**)&e.m, n * sizeof(float)));
+      HIP_TRY(ctx, state_alloc(ctx, (void**)&e.m, n * sizeof(float)));
       hipError_t err = hipMemsetAsync(e.m, 0, n * sizeof(float), ctx->stream);
-      if (err != hipSuccess) { (void)hipFree(e.m); return hip_fail(ctx, err, "hipMemsetAsync(m)"); }
+      if (err != hipSuccess) { state_free(ctx, e.m); return hip_fail(ctx, err, "hipMemsetAsync(m)"); }
     }
     if (need_v) {
-      hipError_t err = hipMalloc((void**)&e.v, n * sizeof(float));
+      hipError_t err = state_alloc(ctx, (void**)&e.v, n * sizeof(float));
       // SGD's velocity is written before it is ever read (first call: v = grad), no fill needed
       if (err == hipSuccess && o->kind != Kind::Sgd) err = hipMemsetAsync(e.v, 0, n * sizeof(float), ctx->stream);
       if (err != hipSuccess) {
-        if (e.m) (void)hipFree(e.m);
-        if (e.v) (void)hipFree(e.v);
+        state_free(ctx, e.m);
+        state_free(ctx, e.v);
         return hip_fail(ctx, err, "allocating optimizer state");
       }
     }
@@ -445,7 +445,7 @@ static int fold_oldest(mxopt_optimizer* opt, size_t n, const char* const* param_
     if (rc) return rc;
     StateEntry* st = nullptr;
     if ((rc = get_state(opt, param_names[i], params[i].n, &st))) return rc;
-    if (!st->sum && st->n) HIP_TRY(ctx, hipMalloc((void**)&st->sum, st->n * sizeof(float)));
+    if (!st->sum && st->n) HIP_TRY(ctx, state_alloc(ctx, (void**)&st->sum, st->n * sizeof(float)));
     sums[i] = st->sum;
   }
   for (size_t j = 0; j < spill; ++j) {

@@ -60,6 +60,20 @@ class SgdHp(C.Structure):
                 ("nesterov", C.c_int)]
 
 
+HBM_MAX_REGIONS = 8
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_MIX43 = 0, 1, 2, 3
+
+
+class HbmPoolInfo(C.Structure):
+    _fields_ = [("capacity_bytes", C.c_uint64), ("used_bytes", C.c_uint64), ("chunk_bytes", C.c_uint64),
+                ("regions", C.c_int32), ("reserved_", C.c_int32),
+                ("region_free_bytes", C.c_uint64 * HBM_MAX_REGIONS),
+                ("region_arena_bytes", C.c_uint64 * HBM_MAX_REGIONS),
+                ("probe_same_region_gbps", C.c_double), ("probe_cross_region_gbps", C.c_double),
+                ("setup_seconds", C.c_double), ("create_seconds", C.c_double), ("scan_seconds", C.c_double),
+                ("probes", C.c_int32), ("reserved2_", C.c_int32)]
+
+
 class RmspropHp(C.Structure):
     _fields_ = [("lr", C.c_float), ("alpha", C.c_float), ("one_minus_alpha", C.c_float), ("eps", C.c_float),
                 ("weight_decay", C.c_float), ("has_weight_decay", C.c_int)]
@@ -91,6 +105,17 @@ SIGNATURES = {
     "mxopt_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(AdamHp), C.POINTER(GradPrep)]),
     "mxopt_hbm_spread_begin": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
     "mxopt_hbm_spread_end": (C.c_int, [C.c_void_p]),
+    "mxopt_hbm_pool_create": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
+    "mxopt_hbm_pool_destroy": (None, [C.c_void_p]),
+    "mxopt_hbm_pool_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "mxopt_hbm_pool_free": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "mxopt_hbm_pool_owns": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "mxopt_hbm_pool_get_info": (C.c_int, [C.c_void_p, C.POINTER(HbmPoolInfo)]),
+    "mxopt_set_state_pool": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "mxopt_hbm_pool_set_hook_target": (C.c_int, [C.c_void_p]),
+    "mxopt_hbm_pool_hook_alloc": (C.c_void_p, [C.c_ssize_t, C.c_int, C.c_void_p]),
+    "mxopt_hbm_pool_hook_free": (None, [C.c_void_p, C.c_ssize_t, C.c_int, C.c_void_p]),
+    "mxopt_probe_stream": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]),
     "mxopt_table_set_pending": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.c_int]),
     "mxopt_norm_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
                                                C.c_void_p]),

@@ -290,11 +290,73 @@ class _HbmSpread:
         return False
 
 
+class HbmPool:
+    """Region-interleaved device memory (mxopt_hbm_pool_create).  `torch_pool()` makes torch allocate from
+    it: `with torch.cuda.use_mem_pool(pool.torch_pool()): p = torch.empty(...)`."""
+
+    MAX_REGIONS = L.HBM_MAX_REGIONS
+    _torch_allocator = None   # one per process: torch keeps the function pointers
+
+    def __init__(self, ctx: "Context", capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0):
+        self.ctx = ctx
+        self.handle = C.c_void_p()
+        torch.cuda.empty_cache()     # what torch caches is not free memory to the driver
+        L.check(ctx.lib.mxopt_hbm_pool_create(ctx.handle, capacity_bytes, chunk_bytes, max_regions,
+                                              C.byref(self.handle)), ctx.handle)
+
+    def info(self) -> L.HbmPoolInfo:
+        out = L.HbmPoolInfo()
+        L.check(self.ctx.lib.mxopt_hbm_pool_get_info(self.handle, C.byref(out)), self.ctx.handle)
+        return out
+
+    def alloc(self, nbytes: int) -> int:
+        p = C.c_void_p()
+        L.check(self.ctx.lib.mxopt_hbm_pool_alloc(self.handle, nbytes, C.byref(p)), self.ctx.handle)
+        return p.value
+
+    def free(self, ptr: int) -> None:
+        L.check(self.ctx.lib.mxopt_hbm_pool_free(self.handle, C.c_void_p(ptr)), self.ctx.handle)
+
+    def owns(self, ptr: int) -> bool:
+        return bool(self.ctx.lib.mxopt_hbm_pool_owns(self.handle, C.c_void_p(ptr)))
+
+    def use_for_state(self) -> None:
+        """Moments and accumulation buffers of objects created on this context from now on live here."""
+        L.check(self.ctx.lib.mxopt_set_state_pool(self.ctx.handle, self.handle), self.ctx.handle)
+
+    def torch_pool(self):
+        """A new torch.cuda.MemPool whose segments come from this pool (and from hipMalloc once it is full).
+        Dropping the MemPool and its tensors hands the segments back."""
+        L.check(self.ctx.lib.mxopt_hbm_pool_set_hook_target(self.handle), self.ctx.handle)
+        if HbmPool._torch_allocator is None:
+            HbmPool._torch_allocator = torch.cuda.memory.CUDAPluggableAllocator(
+                L.LIB_PATH, "mxopt_hbm_pool_hook_alloc", "mxopt_hbm_pool_hook_free")
+        return torch.cuda.MemPool(HbmPool._torch_allocator.allocator())
+
+    def close(self) -> None:
+        if self.handle:
+            self.ctx.lib.mxopt_hbm_pool_set_hook_target(None)
+            self.ctx.lib.mxopt_hbm_pool_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+
+def _hbm_pool(self, capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0) -> HbmPool:
+    return HbmPool(self, capacity_bytes, chunk_bytes, max_regions)
+
+
+def _probe_stream(self, kind: int, a, b=None, c=None, d=None) -> None:
+    """One launch of a bare streaming probe over float32 tensors of equal size (mxopt_probe_stream)."""
+    ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    L.check(self.lib.mxopt_probe_stream(self.handle, kind, ptr(a), ptr(b), ptr(c), ptr(d), a.numel()), self.handle)
+
+
 def _hbm_spread(self, block_bytes: int = 0, keep_one_in: int = 0) -> _HbmSpread:
     return _HbmSpread(self, block_bytes, keep_one_in)
 
 
 Context.hbm_spread = _hbm_spread
+Context.hbm_pool = _hbm_pool
+Context.probe_stream = _probe_stream
 Context.accumulate_norm_only = _accumulate_norm_only
 Context.norm_with_pending_list = _norm_with_pending_list
 Context.adam_with_pending_list = _adam_with_pending_list

@@ -1,0 +1,167 @@
+"""mxopt_hbm_pool_*: the region-interleaved arena, its allocator, the hooks a host allocator plugs in, the
+optimizer state taken from it -- and the bare streaming probes (mxopt_probe_stream), whose data movement
+is checked element by element.  Results never depend on where a buffer lies."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mxopt_oracle as O
+from gpu_util import assert_bit_equal, to_dev, to_host
+
+F = np.float32
+GiB = 1 << 30
+
+
+@pytest.fixture(scope="module")
+def mx():
+    import torch
+    import mxopt
+    assert torch.cuda.is_available()
+    return mxopt
+
+
+@pytest.fixture(scope="module")
+def ctx(mx):
+    c = mx.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def pool(mx, ctx):
+    import torch
+    torch.cuda.empty_cache()
+    free0 = torch.cuda.mem_get_info()[0]
+    p = ctx.hbm_pool(6 * GiB)
+    # what the arena does not hold went back to the driver before create returned
+    assert torch.cuda.mem_get_info()[0] > free0 - 7 * GiB
+    yield p
+    p.close()
+    assert torch.cuda.mem_get_info()[0] > free0 - GiB
+
+
+def test_pool_finds_regions_and_interleaves(mx, pool):
+    i = pool.info()
+    assert i.capacity_bytes == 6 * GiB and i.chunk_bytes == 64 << 20 and i.used_bytes == 0
+    assert 1 <= i.regions <= mx.HbmPool.MAX_REGIONS
+    assert sum(i.region_arena_bytes) == i.capacity_bytes
+    if i.regions >= 2:     # a device with most of its memory free: the arena is split evenly
+        assert i.probe_cross_region_gbps > 1.07 * i.probe_same_region_gbps
+        share = [b for b in i.region_arena_bytes[:i.regions]]
+        assert max(share) - min(share) <= i.chunk_bytes
+    assert i.probes > 0 and 0 < i.scan_seconds <= i.setup_seconds < 30
+
+
+def test_pool_allocator_first_fit_coalesces_and_refuses(mx, ctx, pool):
+    a = pool.alloc(1000)
+    b = pool.alloc(3 * GiB)
+    c = pool.alloc(1)
+    assert a % 512 == 0 and b == a + 1024 and c == b + 3 * GiB and pool.owns(a) and pool.owns(c)
+    assert pool.info().used_bytes == 1024 + 3 * GiB + 512
+    with pytest.raises(mx.MxoptError, match="no free range"):
+        pool.alloc(4 * GiB)
+    pool.free(b)
+    b2 = pool.alloc(2 * GiB)                  # first fit: the hole b left
+    assert b2 == b
+    pool.free(a)
+    pool.free(b2)
+    pool.free(c)
+    assert pool.info().used_bytes == 0
+    whole = pool.alloc(6 * GiB)               # everything coalesced again
+    pool.free(whole)
+    with pytest.raises(mx.InvalidArg, match="not a live allocation"):
+        pool.free(whole)
+    assert not pool.owns(0) and not pool.owns(whole + 6 * GiB)
+    with pytest.raises(mx.InvalidArg, match="power of two"):
+        ctx.hbm_pool(GiB, 3 << 20)
+    with pytest.raises(mx.InvalidArg, match="capacity_bytes is 0"):
+        ctx.hbm_pool(0)
+    with pytest.raises(mx.MxoptError, match="MiB free"):
+        ctx.hbm_pool(4000 * GiB)
+
+
+def test_results_do_not_depend_on_the_arena(mx, ctx, pool):
+    """AdamW on tensors torch allocated from the arena (the plug-in allocator hooks) against the oracle."""
+    import torch
+    rng = np.random.default_rng(11)
+    n = (1 << 20) + 77
+    p, g = rng.normal(0, 0.02, n).astype(F), rng.normal(0, 1e-3, n).astype(F)
+    mem = pool.torch_pool()
+    with torch.cuda.use_mem_pool(mem):
+        dp, dg = torch.empty(n, device="cuda"), torch.empty(n, device="cuda")
+        dm, dv = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    assert all(pool.owns(t.data_ptr()) for t in (dp, dg, dm, dv))
+    dp.copy_(torch.from_numpy(p))
+    dg.copy_(torch.from_numpy(g))
+    t = ctx.table([mx.TensorSpec(p=dp, p_out=dp, g=dg, m=dm, v=dv)])
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    want = p
+    for _ in range(2):
+        ctx.adam(t, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01))
+        want = ref.update_single("w", want, g)
+    assert_bit_equal(to_host(dp), want, "parameters in arena memory")
+    t.close()
+    used = pool.info().used_bytes
+    assert used > 0
+    del dp, dg, dm, dv, mem, t      # the table kept its tensors alive
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    assert pool.info().used_bytes == 0        # torch handed its segments back through the free hook
+
+
+def test_optimizer_state_comes_from_the_pool(mx, ctx, pool):
+    rng = np.random.default_rng(12)
+    n = 300_000
+    p, g = rng.normal(0, 0.02, n).astype(F), rng.normal(0, 1e-3, n).astype(F)
+    pool.use_for_state()
+    try:
+        opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, ctx=ctx)
+        out = opt.update_single("w", to_dev(p), to_dev(g))
+        m, v, cnt, hv = C.c_void_p(), C.c_void_p(), C.c_uint64(), C.c_int()
+        mx.load().mxopt_optimizer_state(opt.handle, b"w", C.byref(m), C.byref(v), C.byref(cnt), C.byref(hv))
+        assert pool.owns(m.value) and pool.owns(v.value) and cnt.value == n
+        assert pool.info().used_bytes >= 2 * 4 * n
+        assert_bit_equal(to_host(out), O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01).update_single("w", p, g), "AdamW, pooled state")
+        del opt
+        assert pool.info().used_bytes == 0    # the moments went back to the arena
+    finally:
+        ctx.lib.mxopt_set_state_pool(ctx.handle, None)
+    opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, ctx=ctx)   # detached again: state from the driver
+    opt.update_single("w", to_dev(p), to_dev(g))
+    assert pool.info().used_bytes == 0
+    del opt
+
+
+def test_probes_move_the_bytes_they_claim(mx, ctx):
+    import torch
+    n = 4096 * 37
+    rng = np.random.default_rng(13)
+    host = [rng.integers(0, 2**31 - 1, n, dtype=np.int64).astype(np.int32) for _ in range(4)]
+    a, b, c, d = [torch.from_numpy(h.copy()).cuda().view(torch.float32) for h in host]
+    before = [t.clone() for t in (a, b, c, d)]
+    ctx.probe_stream(mx.PROBE_READ, a)
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int32), before[0].view(torch.int32))
+    ctx.probe_stream(mx.PROBE_COPY, a, b)
+    torch.cuda.synchronize()
+    assert torch.equal(b.view(torch.int32), a.view(torch.int32))
+    a0, g0, c0, d0 = [t.view(torch.int32).cpu().numpy().astype(np.uint32) for t in (a, b, c, d)]
+    ctx.probe_stream(mx.PROBE_MIX43, a, b, c, d)
+    torch.cuda.synchronize()
+    got = [t.view(torch.int32).cpu().numpy().astype(np.uint32) for t in (a, b, c, d)]
+    assert np.array_equal(got[0], a0 ^ g0) and np.array_equal(got[1], g0)
+    assert np.array_equal(got[2], c0 + g0) and np.array_equal(got[3], d0 ^ (g0 >> 1))
+    ctx.probe_stream(mx.PROBE_WRITE, a)
+    torch.cuda.synchronize()
+    w = a.view(torch.int32).cpu().numpy()
+    assert np.array_equal(w, np.repeat(np.arange(n // 4096, dtype=np.int32), 4096))   # every element written, by its tile
+    with pytest.raises(mx.InvalidArg, match="multiple of 4096"):
+        ctx.probe_stream(mx.PROBE_READ, a[:1000])
+    with pytest.raises(mx.InvalidArg, match="non-NULL"):
+        ctx.probe_stream(mx.PROBE_COPY, a)
+    with pytest.raises(mx.InvalidArg, match="unknown kind"):
+        ctx.probe_stream(9, a)
