@@ -36,23 +36,30 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per element per launch of the dominant kernel from an EARLIER rocprofv3 run, not from this
 # one (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for this library's plain
-# copy kernel: 1.98445 and 1.00000).  Printed as roofline.traffic with roofline.traffic_source naming
-# the file; null when a kernel source is newer than that file.
+# copy kernel).  Printed as roofline.traffic with roofline.traffic_source naming the file; null once the
+# kernel sources no longer hash to what that file records.
 # (workload, fold_last) -> bytes per element
 TRAFFIC_PROFILE = "profiles/hbm_traffic_pmc_cfg5_and_copy.txt"
-MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.97, ("cfg5", 0): 23.93, ("cfg5-deferred", 1): 27.89}
+TRAFFIC_KERNEL_SOURCES = ["mxopt_kernels.hip", "mxopt_kernels_common.h", "mxopt_device.h", "mxopt_list_kernels.h",
+                          "mxopt_list_kernels.hip"]
+MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.91, ("cfg5-deferred", 1): 27.89}
 PROBE_PROFILE = "profiles/probe_streams_pool_and_plain.txt"
 OTHER_CONFIGS = ["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat"]
 
 
 def traffic_profile_is_current():
-    """False when a kernel source changed after the counters were taken."""
-    prof = os.path.join(ROOT, TRAFFIC_PROFILE)
-    if not os.path.exists(prof):
+    """True while the kernel sources are the ones the counters were taken on."""
+    import hashlib
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+        h = hashlib.sha256()
+        for f in TRAFFIC_KERNEL_SOURCES:
+            h.update(open(os.path.join(ROOT, "mlx-node_amd", "csrc", f), "rb").read())
+    except OSError:
         return False
-    csrc = os.path.join(ROOT, "mlx-node_amd", "csrc")
-    kernel_files = ("mxopt_kernels.hip", "mxopt_kernels_common.h", "mxopt_device.h", "mxopt_list_kernels.h")
-    return all(os.path.getmtime(os.path.join(csrc, f)) <= os.path.getmtime(prof) for f in kernel_files)
+    m = re.search(r"kernel-sources-sha256: ([0-9a-f]{64})", text)
+    return bool(m) and m.group(1) == h.hexdigest()
 
 
 def parse_args():

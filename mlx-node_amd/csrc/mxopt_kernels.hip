@@ -231,8 +231,13 @@ static bool adam_g2_for_pd(int od, int g2d, const Launch& L, const AdamMath& mat
   return false;
 }
 
+// True when a gradient stage runs before the optimizer's own ops: its result is float32 whatever g's dtype.
+static bool prep_promotes(const DevPrep& prep) {
+  return (prep.flags & (kPrepPreMul | kPrepClampPre | kPrepClampPost)) != 0 || prep.d_scale != nullptr;
+}
+
 bool launch_adam(int pd, int gd, int od, int g2d, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
-  if (g2d < 0) return dispatch_update(pd, gd, od, L, AdamMath{hp}, prep);
+  if (g2d < 0) return dispatch_update(pd, gd, od, L, AdamMath{hp, prep_promotes(prep) ? MXOPT_F32 : gd}, prep);
   if (gd != MXOPT_F32) return false;
   switch (pd) {
     case MXOPT_F32: return adam_g2_for_pd<MXOPT_F32>(od, g2d, L, AdamMath{hp}, prep);
@@ -245,7 +250,9 @@ bool launch_sgd(int pd, int gd, int od, const Launch& L, const mxopt_sgd_hp& hp,
   return dispatch_update(pd, gd, od, L, SgdMath{hp}, prep);
 }
 bool launch_rmsprop(int pd, int gd, int od, const Launch& L, const mxopt_rmsprop_hp& hp, const DevPrep& prep) {
-  return dispatch_update(pd, gd, od, L, RmspropMath{hp}, prep);
+  // with coupled decay the square is taken of g + wd * p, already float32 (rmsprop.rs:69-80)
+  const int gsq_dtype = (prep_promotes(prep) || hp.has_weight_decay) ? MXOPT_F32 : gd;
+  return dispatch_update(pd, gd, od, L, RmspropMath{hp, gsq_dtype}, prep);
 }
 
 template <int PD>

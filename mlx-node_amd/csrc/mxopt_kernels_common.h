@@ -11,9 +11,20 @@ namespace mxopt {
 // Math functors: the reference's op chains, one rounded float32 operation per line.
 // ------------------------------------------------------------------------------------
 
+// mlx square is a unary op and keeps its operand's dtype (mlx.cpp:2016-2020): the square of a 16-bit
+// gradient that reaches it as it came (no prep stage, no pending sum, no coupled decay in front of it)
+// is a 16-bit tensor, and only the multiply by the float32 scalar that follows promotes it.  g * g is
+// exact in float32 for 16-bit inputs, so rounding it once is that tensor.
+__device__ __forceinline__ float round_square_to(int dtype, float sq) {
+  if (dtype == MXOPT_BF16) return Elem<MXOPT_BF16>::round(sq);
+  if (dtype == MXOPT_F16) return Elem<MXOPT_F16>::round(sq);
+  return sq;
+}
+
 // Adam::update_single (optimizers/adam.rs:77-108) / AdamW::update_single (adamw.rs:81-116).
 struct AdamMath {
   mxopt_adam_hp hp;
+  int gsq_dtype = MXOPT_F32;  // dtype the square of the gradient is rounded to (adamw.rs:92, adam.rs:88)
   static constexpr bool kM = true;
   __device__ __forceinline__ bool uses_v(uint32_t) const { return true; }
   __device__ __forceinline__ bool reads_v(uint32_t) const { return true; }
@@ -23,7 +34,7 @@ struct AdamMath {
     float b1m = m * hp.beta1;
     float g1 = g * hp.one_minus_beta1;
     float nm = b1m + g1;
-    float gsq = g * g;
+    float gsq = round_square_to(gsq_dtype, g * g);
     float b2v = v * hp.beta2;
     float g2 = gsq * hp.one_minus_beta2;
     float nv = b2v + g2;
@@ -72,6 +83,7 @@ struct SgdMath {
 // RMSprop::update_single (optimizers/rmsprop.rs:67-112).
 struct RmspropMath {
   mxopt_rmsprop_hp hp;
+  int gsq_dtype = MXOPT_F32;  // as in AdamMath (rmsprop.rs:80)
   static constexpr bool kM = false;
   __device__ __forceinline__ bool uses_v(uint32_t) const { return true; }
   __device__ __forceinline__ bool reads_v(uint32_t) const { return true; }
@@ -81,7 +93,7 @@ struct RmspropMath {
       float w = p * hp.weight_decay;
       ge = g + w;
     }
-    float gsq = ge * ge;
+    float gsq = round_square_to(gsq_dtype, ge * ge);
     float av = v * hp.alpha;
     float g2 = gsq * hp.one_minus_alpha;
     float nv = av + g2;

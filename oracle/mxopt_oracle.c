@@ -144,8 +144,11 @@ int oracle_adam_unfused(float* p_out, const void* p, int p_dt, const void* g, in
   PASS g1[i] = G(i) * c.omb1;
 #pragma omp parallel for schedule(static)
   PASS m[i] = b1m[i] + g1[i];
+  /* mlx square keeps the operand's dtype (mlx.cpp:2016-2020): a bf16 gradient that was not scaled first
+     gives a bf16 square (exact product, one rounding) */
+  const int sq_bf16 = !c.has_scale && g_dt == DT_BF16;
 #pragma omp parallel for schedule(static)
-  PASS gsq[i] = G(i) * G(i);
+  PASS gsq[i] = sq_bf16 ? bf16_to_f32(f32_to_bf16(G(i) * G(i))) : G(i) * G(i);
 #pragma omp parallel for schedule(static)
   PASS b2v[i] = v[i] * c.beta2;
 #pragma omp parallel for schedule(static)
@@ -190,6 +193,7 @@ void oracle_adam_fused(float* p_out, const void* p, int p_dt, const void* g, int
     float g1 = gi * c.omb1;
     float nm = b1m + g1;
     float gsq = gi * gi;
+    if (!c.has_scale && g_dt == DT_BF16) gsq = bf16_to_f32(f32_to_bf16(gsq)); /* square of a bf16 tensor is bf16 */
     float b2v = v[i] * c.beta2;
     float g2 = gsq * c.omb2;
     float nv = b2v + g2;

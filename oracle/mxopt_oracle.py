@@ -32,8 +32,9 @@ What pins each function (see tests/test_oracle_*.py)
 * f32<->bf16 conversion: bit-exact against torch's CPU conversion.
 
 PARITY UNPINNED (no reference test, fixture or buildable reference covers it):
-* bf16 inputs through any optimizer (promotion to float32 is MLX's documented
-  rule but no reference test runs it);
+* bf16 inputs through any optimizer (promotion to float32 by the scalar multiplies and
+  a 16-bit ``square`` of a 16-bit gradient are MLX's documented rules, but no
+  reference test runs either);
 * the order in which MLX sums squares for the global norm (the oracle uses the
   exact float64 sum, rounded once);
 * NaN handling of ``clip`` (NaN is propagated here);
@@ -105,6 +106,24 @@ def is_bf16(x: np.ndarray) -> bool:
     return np.asarray(x).dtype == np.uint16
 
 
+def square_in_dtype_of(x: np.ndarray, xf: np.ndarray) -> np.ndarray:
+    """mlx square of the tensor ``x`` (``xf`` = its float32 widening), widened back to float32.
+
+    ``square`` is a unary MLX op and keeps its operand's dtype (crates/mlx-sys/src/mlx.cpp:2016-2020):
+    the square of a bf16 / float16 tensor is a bf16 / float16 tensor, and only the scalar multiply that
+    follows promotes it.  x*x is exact in float32 for 16-bit x, so one rounding gives that tensor
+    (torch's bf16/float16 ``square`` agrees bit for bit: tests/test_oracle_library.py).
+    """
+    sq = xf * xf
+    x = np.asarray(x)
+    if x.dtype == np.uint16:
+        return bf16_to_f32(f32_to_bf16(sq))
+    if x.dtype == np.float16:
+        with np.errstate(over="ignore"):
+            return sq.astype(np.float16).astype(np.float32)
+    return sq
+
+
 # --------------------------------------------------------------------------
 # Optimizers  (crates/mlx-core/src/optimizers/{adam,adamw,sgd,rmsprop}.rs)
 # --------------------------------------------------------------------------
@@ -138,7 +157,7 @@ class Adam:
         beta1_m = m * _f32(self.beta1)
         omb1_g = g * _f32(1.0 - self.beta1)
         new_m = beta1_m + omb1_g
-        g_sq = g * g                               # mlx square
+        g_sq = square_in_dtype_of(grad, g)         # mlx square: in the gradient's own dtype
         beta2_v = v * _f32(self.beta2)
         omb2_g2 = g_sq * _f32(1.0 - self.beta2)
         new_v = beta2_v + omb2_g2
@@ -241,9 +260,10 @@ class RMSprop:
         v = self.state[param_name]
         if self.weight_decay != 0.0:                                # rmsprop.rs:69-77
             ge = g + p * _f32(self.weight_decay)
+            g_sq = ge * ge                                          # of a float32 tensor
         else:
             ge = g
-        g_sq = ge * ge
+            g_sq = square_in_dtype_of(grad, g)                      # of the gradient as it came (rmsprop.rs:80)
         new_v = v * _f32(self.alpha) + g_sq * _f32(1.0 - self.alpha)  # rmsprop.rs:80-83
         denom = np.sqrt(new_v) + _f32(self.eps)                     # rmsprop.rs:86-88
         with np.errstate(divide="ignore", invalid="ignore"):

@@ -52,3 +52,28 @@ def assert_bit_equal(got: np.ndarray, want: np.ndarray, what: str = "") -> None:
         i = int(np.flatnonzero(bad)[0])
         raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements differ; first at {i}: "
                              f"got {got[i]!r} ({gb[i]:#x}) want {want[i]!r} ({wb[i]:#x})")
+
+
+def _ordered(a: np.ndarray) -> np.ndarray:
+    """Bit patterns mapped to integers that are ordered like the values (float32 or bf16 in uint16)."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float32:
+        u = a.view(np.uint32).astype(np.int64)
+        return np.where(u & 0x80000000, 0x80000000 - u, u)
+    u = a.astype(np.int64)
+    return np.where(u & 0x8000, 0x8000 - u, u)
+
+
+def assert_within_ulps(got: np.ndarray, want: np.ndarray, ulps: int, rel: float = 0.0, what: str = "") -> int:
+    """Every element within `ulps` units in the last place of its dtype (float32, or bf16 held as uint16), or --
+    when rel > 0, float32 only -- within rel * |want|.  Returns the largest distance seen, in ulps."""
+    assert got.dtype == want.dtype and got.shape == want.shape, (what, got.dtype, want.dtype)
+    d = np.abs(_ordered(got) - _ordered(want))
+    bad = d > ulps
+    if rel > 0.0 and got.dtype == np.float32 and bad.any():
+        bad &= np.abs(got.astype(np.float64) - want.astype(np.float64)) > rel * np.abs(want.astype(np.float64))
+    if bad.any():
+        i = int(np.flatnonzero(bad)[0])
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.size} elements are more than {ulps} ulp apart; "
+                             f"first at {i}: got {got[i]!r} want {want[i]!r} ({int(d[i])} ulp)")
+    return int(d.max()) if d.size else 0

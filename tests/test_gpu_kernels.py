@@ -134,6 +134,52 @@ def test_adam_in_place_and_fp32_grad_for_bf16_param(mx, ctx):
             assert_bit_equal(to_host(dv[i]), ref.state[str(i)][1], f"v{i} it{it}")
 
 
+@pytest.mark.parametrize("half", ["bf16", "f16"])
+def test_square_of_a_16bit_gradient_is_taken_in_its_dtype(mx, ctx, half):
+    """adamw.rs:92 / rmsprop.rs:80: mlx square keeps the gradient's dtype.  A 16-bit gradient that reaches the
+    optimizer as it came gives a 16-bit square; one that a prep stage touched first (here: x 1.0) is float32
+    by then and so is its square.  Both against the oracle, and the two must differ in v."""
+    import torch
+    rng = np.random.default_rng(31)
+    n = 4096 * 3 + 11
+    pf, gf = rng.normal(0, 0.02, n).astype(F), rng.normal(0, 1e-3, n).astype(F)
+    if half == "bf16":
+        p, g = O.f32_to_bf16(pf), O.f32_to_bf16(gf)
+    else:
+        p, g = pf.astype(np.float16), gf.astype(np.float16)
+    g32 = O.as_f32(g)
+
+    def run(launch, prep):
+        dp, dg = to_dev(p), to_dev(g)
+        do = torch.empty(n, dtype=torch.float32, device="cuda")
+        dm, dv = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+        t = ctx.table([mx.TensorSpec(p=dp, p_out=do, g=dg, m=dm, v=dv)])
+        launch(t, prep)
+        ctx.synchronize()
+        return to_host(do), to_host(dv)
+
+    adam = lambda t, prep: ctx.adam(t, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01), prep)
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    want_p = ref.update_single("w", p, g)
+    got_p, got_v = run(adam, None)
+    assert_bit_equal(got_v, ref.state["w"][1], "v, square in the gradient's dtype")
+    assert_bit_equal(got_p, want_p, "p, square in the gradient's dtype")
+    ref32 = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    want_p32 = ref32.update_single("w", p, g32 * F(1.0))
+    got_p32, got_v32 = run(adam, mx.make_prep(pre_mul=1.0))
+    assert_bit_equal(got_v32, ref32.state["w"][1], "v, gradient scaled first")
+    assert_bit_equal(got_p32, want_p32, "p, gradient scaled first")
+    assert not np.array_equal(got_v, got_v32)
+
+    for wd in (0.0, 0.1):
+        rms = lambda t, prep: ctx.rmsprop(t, mx.rmsprop_hp(1e-2, 0.99, 1e-8, wd), prep)
+        r = O.RMSprop(1e-2, 0.99, 1e-8, wd)
+        want = r.update_single("w", p, g)
+        got_p, got_v = run(rms, None)
+        assert_bit_equal(got_v, r.state["w"], f"rmsprop v, wd={wd}")
+        assert_bit_equal(got_p, want, f"rmsprop p, wd={wd}")
+
+
 @pytest.mark.parametrize("persistent,nontemporal,bpc", [(0, 0, 8), (1, 0, 1), (0, 1, 8)])
 def test_adam_launch_options_do_not_change_results(mx, persistent, nontemporal, bpc):
     import torch

@@ -32,7 +32,7 @@ pytestmark = pytest.mark.gpu
 
 import mxopt_oracle as O
 import oracle_c_binding as B
-from gpu_util import to_host
+from gpu_util import assert_within_ulps, to_host
 
 F = np.float32
 
@@ -198,6 +198,9 @@ def test_config2_full_size_every_element(oracle_c):
     res = ctx.norm_result()
     m_ref, v_ref = np.zeros(n, F), np.zeros(n, F)
     g_ref = np.empty(n, np.uint16)
+    # a second host trajectory that never sees a device value: the oracle with its OWN clip factor, from the
+    # exact float64 sum (optimizers/mod.rs:87-102 -> adamw.rs:84-116)
+    own_p, own_m, own_v = p_ref.copy(), np.zeros(n, F), np.zeros(n, F)
     for step in range(2):
         for i in range(nt):                     # fresh gradients each step: 1 % of the elements x100
             key = mx.synthetic_key(SEED, CFG, step + 1, 1, i)
@@ -214,6 +217,13 @@ def test_config2_full_size_every_element(oracle_c):
         same_bits(to_host(torch.cat(dp)), p_ref, f"p step {step}")
         same_bits(torch.cat(dm).cpu().numpy(), m_ref, f"m step {step}")
         same_bits(torch.cat(dv).cpu().numpy(), v_ref, f"v step {step}")
+        # end to end, stated tolerance: 2 float32 ulp (rel 1e-6) on the moments, 1 bf16 ulp on the parameters
+        _, own_scale = O.norm_scale_c1(oracle_c.sumsq(g_ref), 1.0)
+        own_args = B.adam_args(5e-6, 0.9, 0.999, 1e-8, 0.01, scale=float(own_scale))
+        own_p = oracle_c.f32_to_bf16(oracle_c.adam(own_p, g_ref, own_m, own_v, own_args, fused=True))
+        assert_within_ulps(torch.cat(dm).cpu().numpy(), own_m, 2, 1e-6, f"m step {step}, oracle's own clip factor")
+        assert_within_ulps(torch.cat(dv).cpu().numpy(), own_v, 2, 1e-6, f"v step {step}, oracle's own clip factor")
+        assert_within_ulps(to_host(torch.cat(dp)), own_p, 1, what=f"p step {step}, oracle's own clip factor")
     t_g.close()
     t_upd.close()
     ctx.close()
@@ -479,6 +489,17 @@ def test_config5_full_size_windows_and_norm():
     assert np.array_equal(win(p_slab), want_p), "parameters"
     assert np.array_equal(win(m_slab).view(np.uint32), ref.state["w"][0].view(np.uint32)), "first moment"
     assert np.array_equal(win(v_slab).view(np.uint32), ref.state["w"][1].view(np.uint32)), "second moment"
+
+    # End to end: the oracle with ITS OWN clip factor, taken from the float64 sum instead of the device's
+    # (optimizers/mod.rs:87-102 -> adamw.rs:84-116).  Stated tolerance: 2 float32 ulp (rel 1e-6) on the
+    # moments, 1 bf16 ulp on the parameters, norm rel 1e-5 (asserted above).
+    _, own_scale = O.norm_scale_c1(ref_sumsq, 1.0)
+    own = O.AdamW(5e-6, 0.9, 0.999, 1e-8, 0.01)
+    own.state["w"] = (m0.copy(), v0.copy())
+    own_p = O.f32_to_bf16(own.update_single("w", p0, acc * own_scale))
+    assert_within_ulps(win(m_slab), own.state["w"][0], 2, 1e-6, "first moment, oracle's own clip factor")
+    assert_within_ulps(win(v_slab), own.state["w"][1], 2, 1e-6, "second moment, oracle's own clip factor")
+    assert_within_ulps(win(p_slab), own_p, 1, what="bf16 parameters, oracle's own clip factor")
     t_acc.close()
     t_upd.close()
     ctx.close()

@@ -144,3 +144,41 @@ def test_bf16_accumulate_matches_torch():
     ab = a.view(torch.int16).numpy().view(np.uint16)
     bb = b.view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(O.accumulate_gradients({"w": ab}, {"w": bb})["w"], want)
+
+
+def test_square_of_a_16bit_gradient_is_a_16bit_tensor_like_torch():
+    """mlx square keeps its operand's dtype (crates/mlx-sys/src/mlx.cpp:2016-2020), so Adam's and RMSprop's
+    g*g of a bf16 / float16 gradient is rounded to that dtype before the float32 scalar multiply promotes it
+    (adamw.rs:92-94, rmsprop.rs:80-82).  torch's CPU square of a bf16 / float16 tensor is the same single
+    rounding of the exact product; it pins the rounding model, and the optimizers must show it in v."""
+    rng = np.random.default_rng(21)
+    x = np.concatenate([rng.normal(0, 1e-3, 4000), rng.normal(0, 30.0, 1000), [0.0, -0.0, 1e-20, 250.0, 6e4]]).astype(F)
+    bits = O.f32_to_bf16(x)
+    t = torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+    want = t.square().view(torch.int16).numpy().view(np.uint16)
+    got = O.f32_to_bf16(O.square_in_dtype_of(bits, O.bf16_to_f32(bits)))
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.bf16_to_f32(got), O.square_in_dtype_of(bits, O.bf16_to_f32(bits)))   # already a bf16 value
+    h = x.astype(np.float16)
+    want16 = torch.from_numpy(h.copy()).square().numpy()
+    got16 = O.square_in_dtype_of(h, h.astype(F))
+    assert np.array_equal(got16.astype(np.float16).view(np.uint16), want16.view(np.uint16))
+    assert np.array_equal(O.square_in_dtype_of(x, x), x * x)                                   # float32: no extra rounding
+    # the optimizers: v after one step from zero state is (1 - beta2) * square, square in the gradient's dtype
+    g = bits[:4000]
+    p = O.f32_to_bf16(rng.normal(0, 0.02, 4000).astype(F))
+    opt = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    opt.update_single("w", p, g)
+    gf = O.bf16_to_f32(g)
+    assert np.array_equal(opt.state["w"][1], O.bf16_to_f32(O.f32_to_bf16(gf * gf)) * F(1.0 - 0.999))
+    assert not np.array_equal(opt.state["w"][1], (gf * gf) * F(1.0 - 0.999))                  # the rounding shows
+    opt32 = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)
+    opt32.update_single("w", p, gf)                                                           # the same values as float32
+    assert np.array_equal(opt32.state["w"][1], (gf * gf) * F(1.0 - 0.999))
+    r = O.RMSprop(1e-2, 0.99, 1e-8, 0.0)
+    r.update_single("w", p, g)
+    assert np.array_equal(r.state["w"], O.bf16_to_f32(O.f32_to_bf16(gf * gf)) * F(1.0 - 0.99))
+    rw = O.RMSprop(1e-2, 0.99, 1e-8, 0.1)                                                     # coupled decay promotes first
+    rw.update_single("w", p, g)
+    ge = gf + O.bf16_to_f32(p) * F(0.1)
+    assert np.array_equal(rw.state["w"], (ge * ge) * F(1.0 - 0.99))
