@@ -31,6 +31,7 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as
 // (two elements per instruction), reached through the compiler's native bf16 vector type.
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
   const f32x2_t v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
