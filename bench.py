@@ -95,6 +95,8 @@ def parse_args():
     ap.add_argument("--defer", type=int, default=0,
                     help="engine workloads: 1 = defer_accumulation (four resident micro-batches, no accumulation "
                          "buffer, summed in registers by the applying call)")
+    ap.add_argument("--async-engine", type=int, default=0,
+                    help="grpo-engine: 1 = mxopt_engine_micro_batch_async (no read-back per micro-batch; settled once per step)")
     ap.add_argument("--fold-last", type=int, default=1,
                     help="cfg5: 1 = the last micro-batch is measured (norm) but folded into the update instead of "
                          "being written to the accumulation buffer; 0 = four plain accumulation passes")
@@ -505,9 +507,11 @@ class Workload:
         self._setup_engine("sft")
 
     def _step_grpo_engine(self):
+        use_async = bool(getattr(self.args, "async_engine", 0)) and self.args.workload == "grpo-engine"
         for k in range(self.n_micro):
             name = "micro_batch_apply" if k == self.n_micro - 1 else ("micro_batch_first" if k == 0 else "micro_batch")
-            self._timed(name, lambda: self.engine.micro_batch(self.micro[k % len(self.micro)]))
+            call = self.engine.micro_batch_async if use_async else self.engine.micro_batch
+            self._timed(name, lambda: call(self.micro[k % len(self.micro)]))
 
     _step_sft_engine = _step_grpo_engine
 

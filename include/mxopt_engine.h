@@ -13,7 +13,7 @@
  *
  * Per micro-batch the GRPO engine costs one read of the gradients (validity + norm of the
  * clamped values in one pass), one read-modify-write of the float32 accumulation buffer, and
- * one 32-byte read-back; nothing else leaves the device.
+ * one 32-byte read-back (none with mxopt_engine_micro_batch_async); nothing else leaves the device.
  */
 #ifndef MXOPT_ENGINE_H
 #define MXOPT_ENGINE_H
@@ -104,6 +104,24 @@ void mxopt_engine_free(mxopt_engine* e);
  * `out` may be NULL. */
 int mxopt_engine_micro_batch(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads,
                              mxopt_engine_metrics* out);
+
+/* mxopt_engine_micro_batch for the GRPO engine (apply = SGD) without its one host synchronisation: the
+ * blocking call reads the validity flag back (32 bytes) before it decides whether to accumulate, where
+ * the reference reads every gradient back for the same test (grpo/engine.rs:563-569).  Here the flag
+ * stays on the device: the norm pass writes it, every kernel of the call that would change memory
+ * does nothing when it is set, and a copy of it is on its way to pinned host memory when the call
+ * returns.  The host books the micro-batch as valid for the time being; the next engine call of any
+ * kind (or mxopt_engine_settle) looks at the flag, which has long arrived by then, and if it was set
+ * puts the bookkeeping back to what it was before that micro-batch and applies the reference's skip
+ * (NaN counters, emergency flag, `step`).  Results -- parameters, buffers, counters -- are those of the
+ * blocking calls.  Two differences in timing: metrics come from mxopt_engine_settle, and the
+ * "Training stopped" failure of a micro-batch that reaches max_nan_gradients is returned by the call
+ * that settles it.  With defer_accumulation the caller keeps a micro-batch's gradient buffers alive
+ * as for the blocking call. */
+int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads);
+/* Waits for the last async micro-batch's flag (a no-op after a blocking call) and returns the metrics the
+ * blocking call would have returned for it.  `out` may be NULL. */
+int mxopt_engine_settle(mxopt_engine* e, mxopt_engine_metrics* out);
 
 /* SFT, sft/engine.rs:459-553: apply what has been accumulated, averaged over the micro-batches
  * actually seen.  *flushed = 0 when there was nothing to apply. */

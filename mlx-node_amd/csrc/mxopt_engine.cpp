@@ -54,9 +54,57 @@ struct mxopt_engine {
   // device norm slots holds entry j's clip factor (GRPO), -1 for the sum.
   bool held_is_sum = false;
   std::vector<int> held_result;
+  // mxopt_engine_micro_batch_async: the bookkeeping above has been advanced as if the last micro-batch
+  // were valid; its kernels were told to do nothing otherwise, and its validity flag is on its way to
+  // `h_pinned`.  `before` is the bookkeeping as it was, to go back to if the flag turns out set.
+  struct Book {
+    bool have_acc, needs_emergency_save, held_is_sum;
+    int32_t micro_step;
+    int64_t step;
+    uint64_t nan_gradient_count;
+    uint32_t consecutive_nan_count;
+    std::vector<size_t> held_slots;
+    std::vector<std::vector<mxopt_array>> held;
+    std::vector<int> held_result;
+    std::vector<char> in_acc;
+  };
+  bool async_mode = false;                            // inside an async call
+  const uint64_t* async_skip = nullptr;            // ... the device flag its kernels obey
+  bool async_enqueued = false;                        // ... a flag copy was enqueued
+  bool pending = false;
+  int pending_applied = 0;
+  Book before;
+  mxopt_norm_result* h_pinned = nullptr;
+  hipEvent_t copied = nullptr;
 };
 
 namespace {
+
+mxopt_engine::Book take_book(const mxopt_engine* e) {
+  mxopt_engine::Book b;
+  b.have_acc = e->have_acc; b.needs_emergency_save = e->needs_emergency_save; b.held_is_sum = e->held_is_sum;
+  b.micro_step = e->micro_step; b.step = e->step; b.nan_gradient_count = e->nan_gradient_count;
+  b.consecutive_nan_count = e->consecutive_nan_count;
+  b.held_slots = e->held_slots; b.held = e->held; b.held_result = e->held_result;
+  b.in_acc.resize(e->slots.size());
+  for (size_t i = 0; i < e->slots.size(); ++i) b.in_acc[i] = e->slots[i].in_acc ? 1 : 0;
+  return b;
+}
+
+void put_book(mxopt_engine* e, const mxopt_engine::Book& b) {
+  e->have_acc = b.have_acc; e->needs_emergency_save = b.needs_emergency_save; e->held_is_sum = b.held_is_sum;
+  e->micro_step = b.micro_step; e->step = b.step; e->nan_gradient_count = b.nan_gradient_count;
+  e->consecutive_nan_count = b.consecutive_nan_count;
+  e->held_slots = b.held_slots; e->held = b.held; e->held_result = b.held_result;
+  for (size_t i = 0; i < e->slots.size() && i < b.in_acc.size(); ++i) e->slots[i].in_acc = b.in_acc[i] != 0;
+}
+
+// A prep for a kernel that changes memory: inside an async call it also carries the micro-batch's
+// validity flag, so that the kernel does nothing when the gradients held a NaN/Inf.
+mxopt_grad_prep guarded(const mxopt_engine* e, mxopt_grad_prep prep) {
+  if (e->async_skip) prep.d_skip_if_nonzero = e->async_skip;
+  return prep;
+}
 
 int32_t acc_steps(const mxopt_engine* e) {
   return e->cfg.gradient_accumulation_steps < 1 ? 1 : e->cfg.gradient_accumulation_steps;
@@ -264,7 +312,7 @@ int defer_spill(mxopt_engine* e) {
     int rc = cached_table(ctx, rows, &t);
     if (rc) return rc;
     if (grpo) {
-      mxopt_grad_prep prep = grpo_clamp(e);
+      mxopt_grad_prep prep = guarded(e, grpo_clamp(e));
       if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result[e->held_result[j]].scale;
       rc = mxopt_accumulate_transformed(ctx, t, j == 0, &prep);
     } else {
@@ -310,6 +358,61 @@ int defer_table(mxopt_engine* e, mxopt_table** out) {
 
 // ---- GRPO: grpo/engine.rs:561-704 ------------------------------------------------------
 
+// The bookkeeping of a micro-batch that held a NaN/Inf (engine.rs:571-633); nothing else is touched.
+int grpo_skipped(mxopt_engine* e, mxopt_engine_metrics* out) {
+  MXOPT_DEBUG("GRPO engine: NaN/Inf gradient, micro-batch skipped (%llu so far)",
+              (unsigned long long)e->nan_gradient_count + 1);
+  e->nan_gradient_count += 1;
+  e->consecutive_nan_count += 1;
+  if (e->nan_gradient_count >= max_nan(e)) {
+    fill_metrics(e, out, 0, 1);
+    return fail(e->ctx, MXOPT_ERR_FAILURE,
+                "Training stopped: exceeded maximum NaN gradient count (" + std::to_string(e->nan_gradient_count) +
+                    "/" + std::to_string(max_nan(e)) + ")");
+  }
+  if (e->consecutive_nan_count >= emergency_threshold(e)) e->needs_emergency_save = true;
+  e->step += 1;
+  fill_metrics(e, out, 0, 1);
+  return MXOPT_OK;
+}
+
+// The result of the norm pass starts its way to pinned host memory; nobody waits for it here.
+int enqueue_flag_copy(mxopt_engine* e, const mxopt_norm_result* d_result) {
+  mxopt_ctx* ctx = e->ctx;
+  DeviceGuard guard(ctx->device);
+  launch_mirror_result(ctx->stream, d_result, e->h_pinned);
+  int rc = check_launch(ctx, "mirror_result_kernel");
+  if (rc) return rc;
+  HIP_TRY(ctx, hipEventRecord(e->copied, ctx->stream));
+  e->async_skip = &d_result->nonfinite;
+  e->async_enqueued = true;
+  return MXOPT_OK;
+}
+
+// Looks at the flag of the last async micro-batch (waiting for its copy if it is still under way) and
+// puts the bookkeeping right: nothing to do when the gradients were valid; otherwise back to the state
+// before that call, then the reference's skip.  `out` gets what the blocking call would have returned.
+int settle(mxopt_engine* e, mxopt_engine_metrics* out) {
+  if (!e->pending) {
+    fill_metrics(e, out, 0, 0);
+    return MXOPT_OK;
+  }
+  mxopt_ctx* ctx = e->ctx;
+  {
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(ctx, hipEventSynchronize(e->copied));
+  }
+  e->pending = false;
+  const mxopt_norm_result h = *e->h_pinned;
+  if (h.nonfinite) {
+    put_book(e, e->before);
+    return grpo_skipped(e, out);
+  }
+  fill_metrics(e, out, e->pending_applied, 0);
+  add_norm(out, h);
+  return MXOPT_OK;
+}
+
 int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxopt_array* grads,
                      mxopt_engine_metrics* out) {
   mxopt_ctx* ctx = e->ctx;
@@ -332,24 +435,10 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     if ((rc = cached_table(ctx, rows, &t))) return rc;
     const double max_norm = e->cfg.has_gradient_clip_norm ? e->cfg.gradient_clip_norm : -1.0;
     if ((rc = mxopt_global_norm(ctx, t, 0, &prep, max_norm, MXOPT_CLIP_ALWAYS_MULTIPLY, d_result))) return rc;
-    if ((rc = mxopt_read_norm_result(ctx, d_result, &h))) return rc;
+    // async: the flag is not waited for; every kernel below obeys it on the device instead
+    if ((rc = e->async_mode ? enqueue_flag_copy(e, d_result) : mxopt_read_norm_result(ctx, d_result, &h))) return rc;
   }
-  if (h.nonfinite) {  // engine.rs:571-633: skip the whole micro-batch, touch nothing
-    MXOPT_DEBUG("GRPO engine: NaN/Inf gradient, micro-batch skipped (%llu so far)",
-                (unsigned long long)e->nan_gradient_count + 1);
-    e->nan_gradient_count += 1;
-    e->consecutive_nan_count += 1;
-    if (e->nan_gradient_count >= max_nan(e)) {
-      fill_metrics(e, out, 0, 1);
-      return fail(ctx, MXOPT_ERR_FAILURE,
-                  "Training stopped: exceeded maximum NaN gradient count (" + std::to_string(e->nan_gradient_count) +
-                      "/" + std::to_string(max_nan(e)) + ")");
-    }
-    if (e->consecutive_nan_count >= emergency_threshold(e)) e->needs_emergency_save = true;
-    e->step += 1;
-    fill_metrics(e, out, 0, 1);
-    return MXOPT_OK;
-  }
+  if (h.nonfinite) return grpo_skipped(e, out);  // engine.rs:571-633: skip the whole micro-batch, touch nothing
   e->consecutive_nan_count = 0;  // engine.rs:660
   if (!e->have_acc)
     for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
@@ -374,6 +463,7 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
           for (size_t j = 0; j < e->held.size(); ++j)
             scales[j] = e->held_result[j] >= 0 ? &e->d_result[e->held_result[j]].scale : nullptr;
         prep.d_scale = nullptr;
+        prep = guarded(e, prep);
         rc = mxopt_sgd_plain_with_pending_list_each(ctx, t, e->cfg.learning_rate / (double)N, 0.0, &prep, scales,
                                                     e->held_is_sum ? 1 : 0);
         (void)mxopt_table_set_pending(t, 0, nullptr, 0);
@@ -422,6 +512,8 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
       acc_only.push_back(r);
     }
     mxopt_table* t = nullptr;
+    prep = guarded(e, prep);
+    const mxopt_grad_prep only_guard = guarded(e, no_prep());
     if (!pending.empty()) {
       if ((rc = cached_table(ctx, pending, &t)) || (rc = mxopt_sgd_plain_with_pending(ctx, t, lr, 0.0, &prep, 0))) return rc;
     }
@@ -429,7 +521,9 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
       if ((rc = cached_table(ctx, direct, &t)) || (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, &prep))) return rc;
     }
     if (!acc_only.empty()) {
-      if ((rc = cached_table(ctx, acc_only, &t)) || (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, nullptr))) return rc;
+      if ((rc = cached_table(ctx, acc_only, &t)) ||
+          (rc = mxopt_sgd_plain(ctx, t, lr, 0.0, e->async_skip ? &only_guard : nullptr)))
+        return rc;
     }
     end_cycle(e);
     e->step += 1;
@@ -455,14 +549,15 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     if (rows.empty()) continue;
     mxopt_table* t = nullptr;
     if ((rc = cached_table(ctx, rows, &t))) return rc;
-    if ((rc = mxopt_accumulate_transformed(ctx, t, pass == 0, &prep))) return rc;
+    const mxopt_grad_prep gp = guarded(e, prep);
+    if ((rc = mxopt_accumulate_transformed(ctx, t, pass == 0, &gp))) return rc;
   }
   e->have_acc = true;
   e->micro_step += 1;
 
   int applied = 0;
   if (e->micro_step >= N) {  // engine.rs:666-692, with AdamW on the averaged sum in place of apply_gradients
-    mxopt_grad_prep ap = no_prep();
+    mxopt_grad_prep ap = guarded(e, no_prep());
     ap.has_pre_mul = 1;
     ap.pre_mul = (float)(1.0 / (double)N);
     if ((rc = apply_accumulated(e, e->cfg.learning_rate, 0.0, ap))) return rc;
@@ -809,6 +904,8 @@ void mxopt_engine_free(mxopt_engine* e) {
   for (Slot& s : e->slots)
     state_free(e->ctx, s.acc);
   if (e->d_result) (void)hipFree(e->d_result);
+  if (e->h_pinned) (void)hipHostFree(e->h_pinned);
+  if (e->copied) (void)hipEventDestroy(e->copied);
   if (e->adamw) mxopt_optimizer_free(e->adamw);
   delete e;
 }
@@ -816,10 +913,53 @@ void mxopt_engine_free(mxopt_engine* e) {
 int mxopt_engine_micro_batch(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads,
                              mxopt_engine_metrics* out) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_micro_batch: null engine");
+  int rc = settle(e, nullptr);
+  if (rc) return rc;
   std::vector<size_t> idx;
-  int rc = resolve(e, n, names, grads, &idx);
+  rc = resolve(e, n, names, grads, &idx);
   if (rc) return rc;
   return e->cfg.kind == MXOPT_ENGINE_GRPO ? grpo_micro_batch(e, idx, grads, out) : sft_micro_batch(e, idx, grads, out);
+}
+
+int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads) {
+  const char* op = "mxopt_engine_micro_batch_async";
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null engine");
+  mxopt_ctx* ctx = e->ctx;
+  if (e->cfg.kind != MXOPT_ENGINE_GRPO || e->cfg.apply != MXOPT_ENGINE_APPLY_SGD)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                std::string(op) + ": only the GRPO engine with the plain-SGD apply reads a flag back per micro-batch; "
+                                  "the other modes do not block as they are");
+  int rc = settle(e, nullptr);  // the previous micro-batch's flag has long arrived; a skip is booked now
+  if (rc) return rc;
+  std::vector<size_t> idx;
+  if ((rc = resolve(e, n, names, grads, &idx))) return rc;
+  if (!e->h_pinned) {
+    DeviceGuard guard(ctx->device);
+    HIP_TRY(ctx, hipHostMalloc((void**)&e->h_pinned, sizeof(mxopt_norm_result), hipHostMallocDefault));
+    HIP_TRY(ctx, hipEventCreateWithFlags(&e->copied, hipEventDisableTiming));
+  }
+  mxopt_engine::Book before = take_book(e);
+  e->async_mode = true;
+  e->async_skip = nullptr;
+  e->async_enqueued = false;
+  mxopt_engine_metrics m;
+  rc = grpo_micro_batch(e, idx, grads, &m);
+  const bool enqueued = e->async_enqueued;
+  e->async_mode = false;
+  e->async_skip = nullptr;
+  e->async_enqueued = false;
+  if (rc) return rc;
+  if (enqueued) {
+    e->pending = true;
+    e->pending_applied = m.gradients_applied;
+    e->before = std::move(before);
+  }
+  return MXOPT_OK;
+}
+
+int mxopt_engine_settle(mxopt_engine* e, mxopt_engine_metrics* out) {
+  if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_settle: null engine");
+  return settle(e, out);
 }
 
 int mxopt_engine_flush_gradients(mxopt_engine* e, int* flushed, mxopt_engine_metrics* out) {
@@ -827,6 +967,7 @@ int mxopt_engine_flush_gradients(mxopt_engine* e, int* flushed, mxopt_engine_met
   if (e->cfg.kind != MXOPT_ENGINE_SFT)
     return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "mxopt_engine_flush_gradients: only the SFT engine flushes");
   if (flushed) *flushed = 0;
+  { int rc0 = settle(e, nullptr); if (rc0) return rc0; }
   if (e->micro_step == 0 || !e->have_acc) {  // sft/engine.rs:469-472
     fill_metrics(e, out, 0, 0);
     return MXOPT_OK;
@@ -844,6 +985,7 @@ int mxopt_engine_flush_gradients(mxopt_engine* e, int* flushed, mxopt_engine_met
 
 int mxopt_engine_report_nonfinite_loss(mxopt_engine* e, mxopt_engine_metrics* out) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_report_nonfinite_loss: null engine");
+  { int rc0 = settle(e, nullptr); if (rc0) return rc0; }
   e->nan_gradient_count += 1;
   e->consecutive_nan_count += 1;
   if (e->consecutive_nan_count >= emergency_threshold(e)) e->needs_emergency_save = true;  // sft/engine.rs:228-235
@@ -856,18 +998,28 @@ int mxopt_engine_report_nonfinite_loss(mxopt_engine* e, mxopt_engine_metrics* ou
 
 int mxopt_engine_get_metrics(const mxopt_engine* e, mxopt_engine_metrics* out) {
   if (!e || !out) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_get_metrics: null argument");
+  if (e->pending) {  // the counters are only final once the last async micro-batch's flag has been seen
+    int rc = settle(const_cast<mxopt_engine*>(e), nullptr);
+    if (rc) return rc;
+  }
   fill_metrics(e, out, 0, 0);
   return MXOPT_OK;
 }
 
 int mxopt_engine_clear_emergency_save_flag(mxopt_engine* e) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_clear_emergency_save_flag: null engine");
+  { int rc0 = settle(e, nullptr); if (rc0) return rc0; }
   e->needs_emergency_save = false;
   return MXOPT_OK;
 }
 
 int mxopt_engine_reset(mxopt_engine* e) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_reset: null engine");
+  if (e->pending) {  // whatever the flag says, everything is forgotten below
+    DeviceGuard guard(e->ctx->device);
+    (void)hipEventSynchronize(e->copied);
+    e->pending = false;
+  }
   for (Slot& s : e->slots) s.in_acc = false;
   e->have_acc = false;
   e->held.clear();

@@ -56,6 +56,8 @@ bool launch_rmsprop_list(int pd, int gd, int od, int xd, const Launch& L, const 
 bool launch_sumsq_list(int gd, int xd, const Launch& L, const DevPrep& prep, double* partial_sum);
 bool launch_synth(int od, void* out, uint64_t n, uint64_t seed, uint64_t first_index, int dist, float a, float b,
                   uint32_t grid, hipStream_t stream);
+// *host_mapped_dst = *d_src by a one-lane kernel (dst: pinned host memory, visible to the device).
+void launch_mirror_result(hipStream_t stream, const mxopt_norm_result* d_src, mxopt_norm_result* host_mapped_dst);
 // Address, on `device` (which must be the current device), of the library's fixed array of
 // kStaticPartials float64 partial sums: every GPU holds its own copy at its own address.
 constexpr uint32_t kStaticPartials = MXOPT_STATIC_NORM_WORKGROUPS;

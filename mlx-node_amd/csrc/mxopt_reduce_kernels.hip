@@ -298,6 +298,17 @@ void launch_norm_finish(hipStream_t stream, const double* partial_sum, uint32_t 
                      has_max, clip_mode, d_out);
 }
 
+// One result of the second pass copied into pinned host memory by a kernel (a 40-byte store over the
+// bus instead of a copy command): the engines' asynchronous micro-batch call looks at it later.
+__global__ void mirror_result_kernel(const mxopt_norm_result* __restrict__ src, mxopt_norm_result* __restrict__ dst) {
+  *dst = *src;
+  __threadfence_system();
+}
+
+void launch_mirror_result(hipStream_t stream, const mxopt_norm_result* d_src, mxopt_norm_result* host_mapped_dst) {
+  hipLaunchKernelGGL(mirror_result_kernel, dim3(1), dim3(1), 0, stream, d_src, host_mapped_dst);
+}
+
 // ------------------------------------------------------------------------------------
 // Partial sums that need no allocation: a fixed array in the code object's own device memory, one
 // copy per GPU, for callers that may not allocate (mxopt_global_norm_static).  On the host the

@@ -231,6 +231,8 @@ SIGNATURES.update({
                                    C.POINTER(C.c_void_p)]),
     "mxopt_engine_free": (None, [C.c_void_p]),
     "mxopt_engine_micro_batch": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA, _PM]),
+    "mxopt_engine_micro_batch_async": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), _PA]),
+    "mxopt_engine_settle": (C.c_int, [C.c_void_p, _PM]),
     "mxopt_engine_flush_gradients": (C.c_int, [C.c_void_p, _PI, _PM]),
     "mxopt_engine_report_nonfinite_loss": (C.c_int, [C.c_void_p, _PM]),
     "mxopt_engine_get_metrics": (C.c_int, [C.c_void_p, _PM]),

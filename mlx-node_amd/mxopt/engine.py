@@ -72,6 +72,27 @@ class _EngineOptimizerSide:
             self._held = []
         return m
 
+    def micro_batch_async(self, gradients: Dict[str, torch.Tensor]) -> None:
+        """micro_batch without the host synchronisation (GRPO, plain-SGD apply): the validity flag stays on the
+        device; settle() -- or the next call of any kind -- books a skipped micro-batch afterwards."""
+        names = list(gradients)
+        cnames = (C.c_char_p * max(len(names), 1))(*[s.encode() for s in names])
+        arrs = (L.Array * max(len(names), 1))()
+        for i, nm in enumerate(names):
+            arrs[i] = _arr(gradients[nm])
+        # the kernels read the gradients after this returns: they stay alive until the call after next has settled them
+        self._async_keep = [getattr(self, "_async_keep", [None, None])[1], list(gradients.values())]
+        if self.defers:
+            self._held.append(list(gradients.values()))
+        self._check(self.lib.mxopt_engine_micro_batch_async(self.handle, len(names), cnames, arrs))
+
+    def settle(self) -> L.EngineMetrics:
+        m = L.EngineMetrics()
+        self._check(self.lib.mxopt_engine_settle(self.handle, C.byref(m)))
+        if self.defers and (m.gradients_applied or m.micro_step == 0):
+            self._held = []
+        return m
+
     def metrics(self) -> L.EngineMetrics:
         m = L.EngineMetrics()
         self._check(self.lib.mxopt_engine_get_metrics(self.handle, C.byref(m)))
