@@ -332,7 +332,9 @@ int mxopt_sgd_plain_with_pending(mxopt_ctx* ctx, const mxopt_table* t, double le
  * tensor.g is the first addend: the first micro-batch, or a float32 buffer that already holds
  * earlier ones (more micro-batches than MXOPT_MAX_PENDING + 1).  The pending streams x0.. all have
  * one dtype; tensor.g has that dtype or float32.  The caller keeps every stream alive and unchanged
- * until the update has run.  No counterpart in the reference (it materialises every sum). */
+ * until the update has RUN, i.e. until the work the call enqueued on the context's stream has
+ * completed (the call returning only means it is enqueued), or orders any reuse of that memory after
+ * it on the same stream.  No counterpart in the reference (it materialises every sum). */
 #define MXOPT_MAX_PENDING 7
 
 /* Attach k (0..MXOPT_MAX_PENDING; 0 detaches) pending streams to every row of the table:

@@ -56,8 +56,10 @@ typedef struct mxopt_engine_config {
                                           each micro-batch's gradients lie and the update adds them in
                                           registers (float32, arrival order: the numbers of the float32
                                           buffer, bit for bit).  The caller keeps every gradient buffer of
-                                          a cycle alive and unchanged until the call that applies them
-                                          (or flush_gradients / reset) has returned.  With more than
+                                          a cycle alive and unchanged until the work that the applying call
+                                          (or flush_gradients / reset) enqueued on the context's stream has
+                                          completed -- the call returning is not enough: it only enqueues --
+                                          or orders any reuse of the memory after it on that stream.  With more than
                                           MXOPT_MAX_PENDING + 1 micro-batches in a cycle the oldest ones
                                           are added into a float32 buffer as the later ones arrive (their
                                           buffers are free again after that call); the last

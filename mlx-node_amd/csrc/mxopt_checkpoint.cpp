@@ -167,15 +167,22 @@ int save_state_file(mxopt_ctx* ctx, const char* path, const char* optimizer, int
 
   DeviceGuard guard(ctx->device);
   Staging stage;
+  // Any failure from here on closes and removes the half-written temporary file.
+  auto abandon = [&](int code) {
+    if (file.f) { std::fclose(file.f); file.f = nullptr; }
+    std::remove(tmp.c_str());
+    return code;
+  };
   int rc = stage.ensure(ctx);
-  if (rc) return rc;
+  if (rc) return abandon(rc);
   for (const CheckpointTensor* t : order) {
     const char* src = (const char*)t->device;
     uint64_t left = t->n * sizeof(float);
     while (ok && left) {
       const size_t now = (size_t)std::min<uint64_t>(left, kStageBytes);
-      HIP_TRY(ctx, hipMemcpyAsync(stage.host, src, now, hipMemcpyDeviceToHost, ctx->stream));
-      HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+      hipError_t err = hipMemcpyAsync(stage.host, src, now, hipMemcpyDeviceToHost, ctx->stream);
+      if (err == hipSuccess) err = hipStreamSynchronize(ctx->stream);
+      if (err != hipSuccess) return abandon(hip_fail(ctx, err, "save_file: copying state to the host"));
       ok = std::fwrite(stage.host, 1, now, file.f) == now;
       src += now;
       left -= now;

@@ -413,15 +413,20 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
   if (n && (!param_names || !params || !grads || !outs)) return fail(ctx, MXOPT_ERR_INVALID_ARG, "update_many: null argument");
   std::vector<StateEntry*> states;
   Hp hp;
+  const int64_t step_before = opt->step;  // prepare_many counts the calls; a refused update must not
   int rc = prepare_many(opt, n, param_names, params, grads, outs, prep, &states, &hp);
-  if (rc) return rc;
-  switch (opt->kind) {
-    case Kind::Adam:
-    case Kind::AdamW: rc = mxopt_adam(ctx, opt->many_table, &hp.adam, prep); break;
-    case Kind::Sgd: rc = mxopt_sgd(ctx, opt->many_table, &hp.sgd, prep); break;
-    case Kind::Rmsprop: rc = mxopt_rmsprop(ctx, opt->many_table, &hp.rms, prep); break;
+  if (!rc) {
+    switch (opt->kind) {
+      case Kind::Adam:
+      case Kind::AdamW: rc = mxopt_adam(ctx, opt->many_table, &hp.adam, prep); break;
+      case Kind::Sgd: rc = mxopt_sgd(ctx, opt->many_table, &hp.sgd, prep); break;
+      case Kind::Rmsprop: rc = mxopt_rmsprop(ctx, opt->many_table, &hp.rms, prep); break;
+    }
   }
-  if (rc) return rc;
+  if (rc) {
+    opt->step = step_before;  // nothing was launched: later bias corrections see the count as it was
+    return rc;
+  }
   if (opt->kind == Kind::Sgd && opt->momentum != 0.0)
     for (StateEntry* st : states) st->has_velocity = true;
   return MXOPT_OK;
@@ -511,7 +516,10 @@ int mxopt_optimizer_update_many_accumulated(mxopt_optimizer* opt, size_t n, cons
   std::vector<StateEntry*> states;
   Hp hp;
   int rc = prepare_many(opt, n, param_names, params, grads, outs, prep, &states, &hp);
-  if (rc) return rc;
+  if (rc) {
+    opt->step = step_before;
+    return rc;
+  }
   std::vector<const void*> streams((k - 1) * n);
   for (size_t j = 1; j < k; ++j)
     for (size_t i = 0; i < n; ++i) streams[(j - 1) * n + i] = grads[j * n + i].data;
@@ -770,7 +778,9 @@ int mxopt_accumulate_gradients(mxopt_ctx* ctx, size_t n, const mxopt_array* acc,
   if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "accumulate_gradients: null context");
   if (n == 0) return MXOPT_OK;
   if (!acc || !new_grads || !outs) return fail(ctx, MXOPT_ERR_INVALID_ARG, "accumulate_gradients: null argument");
-  std::vector<mxopt_tensor> first_rows, add_rows;
+  // widen_rows: a 16-bit running sum meets a gradient of another dtype.  `acc.add(new)` promotes such a
+  // pair to float32 (models/qwen3/model.rs:2227): out = widen(acc), exact, then out += new.
+  std::vector<mxopt_tensor> first_rows, add_rows, widen_rows;
   for (size_t i = 0; i < n; ++i) {
     int rc;
     if ((rc = check_array(ctx, &new_grads[i], "accumulate_gradients: new gradient"))) return rc;
@@ -785,21 +795,31 @@ int mxopt_accumulate_gradients(mxopt_ctx* ctx, size_t n, const mxopt_array* acc,
       continue;
     }
     if (acc[i].n != new_grads[i].n) return fail(ctx, MXOPT_ERR_INVALID_ARG, "accumulate_gradients: shapes differ");
-    if (acc[i].dtype != outs[i].dtype)
-      return fail(ctx, MXOPT_ERR_INVALID_ARG, "accumulate_gradients: output dtype must equal the accumulator's");
-    if (acc[i].data != outs[i].data) {  // out of place: read the running sum from a separate buffer
+    const int promoted = acc[i].dtype == new_grads[i].dtype ? acc[i].dtype : MXOPT_F32;  // MLX promote_types
+    if (outs[i].dtype != promoted)
+      return fail(ctx, MXOPT_ERR_INVALID_ARG,
+                  "accumulate_gradients: the output takes the promoted dtype of accumulator and gradient "
+                  "(their own when equal, float32 otherwise)");
+    if (acc[i].dtype != promoted) {  // 16-bit sum, other gradient dtype, float32 result
+      if (acc[i].data == outs[i].data)
+        return fail(ctx, MXOPT_ERR_INVALID_ARG, "accumulate_gradients: a 16-bit accumulator cannot hold the float32 sum in place");
+      mxopt_tensor w = blank_tensor();
+      w.g = acc[i].data; w.g_dtype = (uint8_t)acc[i].dtype; w.n = acc[i].n;
+      w.g_out = outs[i].data; w.g_out_dtype = (uint8_t)outs[i].dtype;
+      widen_rows.push_back(w);
+    } else if (acc[i].data != outs[i].data) {  // out of place: read the running sum from a separate buffer
       r.p = acc[i].data;
       r.p_dtype = (uint8_t)acc[i].dtype;
     }
     add_rows.push_back(r);
   }
-  for (int pass = 0; pass < 2; ++pass) {
-    std::vector<mxopt_tensor>& rows = pass == 0 ? first_rows : add_rows;
+  for (int pass = 0; pass < 3; ++pass) {  // copies of new names, widened running sums, then the additions
+    std::vector<mxopt_tensor>& rows = pass == 0 ? first_rows : pass == 1 ? widen_rows : add_rows;
     if (rows.empty()) continue;
     mxopt_table* t = nullptr;
     int rc = cached_table(ctx, rows, &t);
     if (rc) return rc;
-    if ((rc = mxopt_accumulate(ctx, t, pass == 0, nullptr, -1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, nullptr))) return rc;
+    if ((rc = mxopt_accumulate(ctx, t, pass < 2, nullptr, -1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, nullptr))) return rc;
   }
   return MXOPT_OK;
 }

@@ -47,6 +47,15 @@ class _EngineOptimizerSide:
             self.lib.mxopt_engine_free(self.handle)
         self.handle = None
 
+    def _release_held(self) -> None:
+        """The applying call has been enqueued, not finished: tell torch's allocator that the cycle's gradient
+        tensors are still in use on the context's stream before dropping the references to them."""
+        for tensors in self._held:
+            for t in tensors:
+                if t.is_cuda:
+                    t.record_stream(self.ctx.stream)
+        self._held = []
+
     def _check(self, rc: int) -> None:
         if rc == L.OK:
             return
@@ -69,7 +78,7 @@ class _EngineOptimizerSide:
             self._held.append(list(gradients.values()))
         self._check(self.lib.mxopt_engine_micro_batch(self.handle, len(names), cnames, arrs, C.byref(m)))
         if m.gradients_applied or m.micro_step == 0:
-            self._held = []
+            self._release_held()
         return m
 
     def micro_batch_async(self, gradients: Dict[str, torch.Tensor]) -> None:
@@ -90,7 +99,7 @@ class _EngineOptimizerSide:
         m = L.EngineMetrics()
         self._check(self.lib.mxopt_engine_settle(self.handle, C.byref(m)))
         if self.defers and (m.gradients_applied or m.micro_step == 0):
-            self._held = []
+            self._release_held()
         return m
 
     def metrics(self) -> L.EngineMetrics:
@@ -119,7 +128,7 @@ class _EngineOptimizerSide:
 
     def reset(self) -> None:
         self._check(self.lib.mxopt_engine_reset(self.handle))
-        self._held = []
+        self._release_held()
 
     def save_optimizer_state(self, path) -> None:
         self._check(self.lib.mxopt_engine_save_optimizer_state(self.handle, str(path).encode()))

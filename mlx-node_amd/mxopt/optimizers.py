@@ -294,9 +294,6 @@ def accumulate_gradients(accumulated_gradients: Dict[str, torch.Tensor], new_gra
     acc = [accumulated_gradients.get(k) for k in names]
     outs = [torch.empty_like(g, dtype=_promote(a, g)) if a is not None else torch.empty_like(g)
             for a, g in zip(acc, new)]
-    for k, a, o in zip(names, acc, outs):
-        if a is not None and a.dtype != o.dtype:
-            raise L.InvalidArg(L.ERR_INVALID_ARG, f"'{k}': a 16-bit accumulator cannot take a float32 gradient")
     L.check(ctx.lib.mxopt_accumulate_gradients(ctx.handle, len(names), _arrs(acc), _arrs(new), _arrs(outs)),
             ctx.handle)
     result = dict(zip(names, outs))

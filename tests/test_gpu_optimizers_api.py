@@ -272,6 +272,58 @@ def test_accumulate_gradients(mx):
     assert set(out) == {"a", "b"} and vals(out["b"])[0] == 2 and vals(out["a"])[0] == 2
 
 
+def test_accumulate_gradients_promotes_mixed_dtypes(mx):
+    """models/qwen3/model.rs:2227 is `acc.add(new)`: operands of different dtypes give a float32 sum (MLX
+    promote_types), equal 16-bit dtypes stay 16-bit.  Every pairing against the oracle, ragged sizes."""
+    import torch
+    rng = np.random.default_rng(29)
+    for n in (1, 4097, 100003):
+        a32, g32 = rng.normal(0, 1e-2, n).astype(F), rng.normal(0, 1e-2, n).astype(F)
+        forms = {"f32": lambda x: x, "bf16": O.f32_to_bf16, "f16": lambda x: x.astype(np.float16)}
+        for ka, fa in forms.items():
+            for kg, fg in forms.items():
+                a, g = fa(a32), fg(g32)
+                out = mx.accumulate_gradients({"w": to_dev(a)}, {"w": to_dev(g)})["w"]
+                s = O.as_f32(a) + O.as_f32(g)
+                if ka == kg:
+                    want = forms[ka](s) if ka != "f16" else s.astype(np.float16)
+                    assert out.dtype == {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[ka]
+                else:
+                    want = s
+                    assert out.dtype == torch.float32, (ka, kg)
+                assert_bit_equal(to_host(out), want, f"{ka} + {kg}, n={n}")
+    # the C entry point refuses an output that is not the promoted dtype
+    ctx = mx.default_context()
+    import mxopt.optimizers as MO
+    a, g = to_dev(O.f32_to_bf16(a32)), to_dev(g32)
+    bad = torch.empty(len(g32), dtype=torch.bfloat16, device="cuda")
+    rc = ctx.lib.mxopt_accumulate_gradients(ctx.handle, 1, MO._arrs([a]), MO._arrs([g]), MO._arrs([bad]))
+    assert rc == mx._lib.ERR_INVALID_ARG and b"promoted dtype" in ctx.lib.mxopt_last_error(ctx.handle)
+
+
+def test_a_refused_update_many_leaves_the_call_counter_alone(mx):
+    """adam.rs:73 counts update_single calls; an update_many that is refused launches nothing and must not
+    shift later bias corrections."""
+    ps, gs = rand_lists(31)
+    names = [f"p{i}" for i in range(len(ps))]
+    opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+    ref = O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+    dp, dg = [to_dev(p) for p in ps], [to_dev(g) for g in gs]
+    opt.update_many(names, dp, dg, outs=dp)
+    assert opt.step == len(ps)
+    wrong = list(dg)
+    wrong[-1] = to_dev(np.zeros(len(gs[-1]) + 1, F))          # the last pair does not match: refused as a whole
+    with pytest.raises(ValueError):
+        opt.update_many(names, dp, wrong, outs=dp)
+    assert opt.step == len(ps)
+    opt.update_many(names, dp, dg, outs=dp)
+    cur = list(ps)
+    for _ in range(2):
+        cur = [ref.update_single(nm, p, g) for nm, p, g in zip(names, cur, gs)]
+    for i, p in enumerate(dp):
+        assert_bit_equal(to_host(p), cur[i], f"p{i} after a refused call in between")
+
+
 # ---- __test__/training/basic-training.test.ts:95-128 ----------------------------------------------
 
 def test_apply_gradients_closed_form(mx):
