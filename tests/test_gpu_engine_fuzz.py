@@ -1,6 +1,6 @@
 """Random call sequences against both engines' optimizer side: micro-batches with all or some of the
 names, poisoned micro-batches (GRPO), flushes and NaN-loss reports (SFT), resets -- with and without
-an accumulation buffer, plain-SGD and AdamW apply, bf16 and float32.  After every call parameters
+an accumulation buffer, plain-SGD and AdamW apply, bf16 and float32, the GRPO call blocking or asynchronous.  After every call parameters
 (bit for bit), counters and flags must equal the oracle's.  Derandomised; MXOPT_PROPERTY_EXAMPLES=<n>
 draws n fresh random sequences instead."""
 import math
@@ -60,8 +60,10 @@ def both(what, dev_call, ref_call, mx):
 @given(kind=st.sampled_from(["grpo", "sft"]), bf16=st.booleans(), apply=st.sampled_from(["sgd", "adamw"]),
        n_acc=st.sampled_from([1, 2, 3, 5, 9]), defer=st.booleans(), acc_f32=st.booleans(),
        clip_norm=st.sampled_from([None, 0.5]), clip_value=st.sampled_from([None, 0.003]),
-       wd=st.sampled_from([0.0, 0.01]), ops=st.lists(OPS, min_size=1, max_size=22), seed=st.integers(0, 2 ** 31))
-def test_random_engine_sequences(mx, kind, bf16, apply, n_acc, defer, acc_f32, clip_norm, clip_value, wd, ops, seed):
+       wd=st.sampled_from([0.0, 0.01]), ops=st.lists(OPS, min_size=1, max_size=22), seed=st.integers(0, 2 ** 31),
+       use_async=st.booleans())
+def test_random_engine_sequences(mx, kind, bf16, apply, n_acc, defer, acc_f32, clip_norm, clip_value, wd, ops, seed,
+                                 use_async):
     rng = np.random.default_rng(seed)
     if kind == "grpo" and defer:
         apply = "sgd"
@@ -108,7 +110,16 @@ def test_random_engine_sequences(mx, kind, bf16, apply, n_acc, defer, acc_f32, c
                     return ref.micro_batch(g)
                 return ref.micro_batch(g, norm_sumsq=m.grad_sumsq) if (measured and boundary) else ref.micro_batch(g)
 
-            m = both(what, lambda: dev.micro_batch({k: to_dev(g) for k, g in grads.items()}), ref_call, mx)
+            # GRPO with the plain-SGD apply also through the call that does not wait for the validity flag: booked as
+            # valid, kernels guarded on the device, put right by settle()
+            if use_async and kind == "grpo" and apply == "sgd":
+                def dev_call(grads=grads):
+                    dev.micro_batch_async({k: to_dev(g) for k, g in grads.items()})
+                    return dev.settle()
+            else:
+                def dev_call(grads=grads):
+                    return dev.micro_batch({k: to_dev(g) for k, g in grads.items()})
+            m = both(what, dev_call, ref_call, mx)
             if m is not None and kind == "grpo":
                 assert bool(m.skipped) == poisoned
         elif op == "flush":
