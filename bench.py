@@ -202,7 +202,7 @@ class Workload:
         _, views = self._carve(dtype)
         self._next_stream = getattr(self, "_next_stream", 0) + 1
         mx = self.mx
-        self._fill(views, self._next_stream, mx.SYNTH_NORMAL_OUTLIERS if outliers else mx.SYNTH_NORMAL, std, 100.0)
+        self._fill(views, self._next_stream, mx.SYNTH_GAUSSIAN_OUTLIERS if outliers else mx.SYNTH_GAUSSIAN, std, 100.0)
         return views
 
     def _zeros_list(self):
@@ -641,8 +641,8 @@ def cpu_baseline_cfg1_full():
     oc = B.load()
     sizes = [numel(shape) for _, shape in param_list(QWEN3["0.6B"])]
     key = lambda stream, i: mxopt.synthetic_key(Workload.SEED, 1, 0, stream, i)
-    ps = [oc.fill_synthetic(n, "f32", key(1, i), 0, 0.02) for i, n in enumerate(sizes)]
-    gs = [oc.fill_synthetic(n, "f32", key(2, i), 0, 1e-3) for i, n in enumerate(sizes)]
+    ps = [oc.fill_synthetic(n, "f32", key(1, i), 3, 0.02) for i, n in enumerate(sizes)]      # 3 = MXOPT_SYNTH_GAUSSIAN
+    gs = [oc.fill_synthetic(n, "f32", key(2, i), 3, 1e-3) for i, n in enumerate(sizes)]
     ms = [np.zeros(n, np.float32) for n in sizes]
     vs = [np.zeros(n, np.float32) for n in sizes]
     a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01)
@@ -768,8 +768,8 @@ def main():
               "note": "; ".join(x for x in (wl.note,
                                             "the gradient buffers are generated once and reused by every step (their values do "
                                             "not change the traffic)",
-                                            "'normal' inputs are the sum of four 16-bit uniforms: exact standard deviation, "
-                                            "|x| <= 3.46 sigma") if x),
+                                            "'normal' inputs come from the generator's Gaussian mode (quantile table, tails to "
+                                            "6.3 sigma)") if x),
               "scale": args.scale, "alloc": args.alloc, "placement": placement}
     dtype = wl.dtype
     wl.close()

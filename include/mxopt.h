@@ -439,11 +439,19 @@ int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first
  *                               mean 0, standard deviation a, bell shaped, |x| <= 3.46 a
  *   MXOPT_SYNTH_NORMAL_OUTLIERS the same, and on average every 100th element (second hash % 100 == 0) times f32(b)
  *   MXOPT_SYNTH_UNIFORM         f32(top 24 bits) * f32((b - a) / 2^24) + f32(a): uniform on [a, b)
+ *   MXOPT_SYNTH_GAUSSIAN        normal with standard deviation a and true tails: bit 63 of the hash is the sign,
+ *                               bits 31..62 a uniform u that stands for the two-sided tail probability
+ *                               (u + 0.5) / 2^32 of |x|; u is split like a floating-point number (leading zeros:
+ *                               octave, next 5 bits: sub-interval, 16 more bits: linear interpolation) into a
+ *                               committed 32 x 33 table of float32 quantiles, so |x| reaches 6.3 a with the same
+ *                               relative resolution everywhere; then * f32(a)
+ *   MXOPT_SYNTH_GAUSSIAN_OUTLIERS  the same, and on average every 100th element times f32(b)
  * then rounded once to out's dtype.  Only integer arithmetic, exact conversions and at most two rounded
- * float32 operations: a host program regenerates any slice bit for bit (as the CPU checker in this
+ * float32 operations (three and a table look-up for the Gaussian modes): a host program regenerates any slice bit for bit (as the CPU checker in this
  * repository does), so inputs never have to be copied or read back to compare results at full size.
  * No counterpart in the reference (its tests build inputs on the host). */
-enum { MXOPT_SYNTH_NORMAL = 0, MXOPT_SYNTH_NORMAL_OUTLIERS = 1, MXOPT_SYNTH_UNIFORM = 2 };
+enum { MXOPT_SYNTH_NORMAL = 0, MXOPT_SYNTH_NORMAL_OUTLIERS = 1, MXOPT_SYNTH_UNIFORM = 2, MXOPT_SYNTH_GAUSSIAN = 3,
+       MXOPT_SYNTH_GAUSSIAN_OUTLIERS = 4 };
 int mxopt_fill_synthetic(mxopt_ctx* ctx, void* out, uint64_t n, int dtype, uint64_t seed, uint64_t first_index,
                          int distribution, double a, double b);
 /* The stream key used by this repository's benchmark and tests:

@@ -909,6 +909,11 @@ int mxopt_fill_synthetic(mxopt_ctx* ctx, void* out, uint64_t n, int dtype, uint6
       fa = (float)((b - a) / 16777216.0);
       fb = (float)a;
       break;
+    case MXOPT_SYNTH_GAUSSIAN:
+    case MXOPT_SYNTH_GAUSSIAN_OUTLIERS:
+      fa = (float)a;
+      fb = (float)b;
+      break;
     default:
       return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_fill_synthetic: unknown distribution");
   }

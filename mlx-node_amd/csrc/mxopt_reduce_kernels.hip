@@ -3,6 +3,7 @@
 #include <mutex>
 
 #include "mxopt_kernels_common.h"
+#include "mxopt_gauss_table.h"
 
 namespace mxopt {
 
@@ -262,6 +263,22 @@ __device__ __forceinline__ uint64_t synth_hash(uint64_t seed, uint64_t idx) {
   return z ^ (z >> 31);
 }
 
+// |x| of a standard normal by its two-sided tail probability, a 32-bit uniform split like a floating-point
+// number: leading zeros pick the octave (row), the next 5 bits the sub-interval, 16 more bits interpolate.
+static __device__ const float kGaussQuantile[MXOPT_GAUSS_ROWS][MXOPT_GAUSS_COLS] = {MXOPT_GAUSS_TABLE};
+
+__device__ __forceinline__ float synth_gauss_magnitude(uint32_t u) {
+  if (u == 0u) u = 1u;
+  const int k = __clz((int)u);
+  const uint32_t v = u << k;
+  const uint32_t j = (v >> 26) & 31u;
+  const float f = (float)((v >> 10) & 0xffffu) * 0x1p-16f;  // exact
+  const float t0 = kGaussQuantile[k][j];
+  const float d = kGaussQuantile[k][j + 1] - t0;
+  const float step = d * f;
+  return t0 + step;
+}
+
 template <int OD>
 __global__ __launch_bounds__(kThreads) void synth_kernel(void* __restrict__ out, uint64_t n, uint64_t seed,
                                                          uint64_t first_index, int dist, float a, float b) {
@@ -271,6 +288,12 @@ __global__ __launch_bounds__(kThreads) void synth_kernel(void* __restrict__ out,
     if (dist == MXOPT_SYNTH_UNIFORM) {
       x = (float)(uint32_t)(z >> 40) * a;   // a = (hi - lo) / 2^24, b = lo
       x = x + b;
+    } else if (dist == MXOPT_SYNTH_GAUSSIAN || dist == MXOPT_SYNTH_GAUSSIAN_OUTLIERS) {
+      const float mag = synth_gauss_magnitude((uint32_t)(z >> 31));
+      x = (z >> 63) ? -mag : mag;
+      x = x * a;                             // a = sigma
+      if (dist == MXOPT_SYNTH_GAUSSIAN_OUTLIERS && synth_hash(seed ^ 0xA5A5A5A5A5A5A5A5ull, first_index + i) % 100ull == 0ull)
+        x = x * b;
     } else {
       // sum of four 16-bit uniforms, centred: a bell shape on [-131070, 131070] with an exactly known variance
       const int32_t sum = (int32_t)((z & 0xffffu) + ((z >> 16) & 0xffffu) + ((z >> 32) & 0xffffu) + (z >> 48)) - 131070;

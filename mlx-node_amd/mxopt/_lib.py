@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(os.path.dirname(HERE), "libmxopt.so")
 F32, I32, F16, BF16, U32 = 0, 1, 2, 3, 4
 OK, ERR_INVALID_ARG, ERR_FAILURE, ERR_HIP, ERR_OOM = 0, 1, 2, 3, 4
 TF_FIRST = 0x1
-SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM = 0, 1, 2
+SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM, SYNTH_GAUSSIAN, SYNTH_GAUSSIAN_OUTLIERS = 0, 1, 2, 3, 4
 CLIP_ALWAYS_MULTIPLY, CLIP_IF_ABOVE = 0, 1
 CHUNK_ELEMS = 4096
 MAX_PENDING = 7

@@ -75,9 +75,27 @@ static inline uint64_t synth_hash(uint64_t seed, uint64_t idx) {
   return z ^ (z >> 31);
 }
 
+/* The quantile table of the Gaussian modes is the one the device code compiles. */
+#include "mxopt_gauss_table.h"
+static const float gauss_quantile[MXOPT_GAUSS_ROWS][MXOPT_GAUSS_COLS] = {MXOPT_GAUSS_TABLE};
+
+static inline float synth_gauss_magnitude(uint32_t u) {
+  if (u == 0u) u = 1u;
+  const int k = __builtin_clz(u);
+  const uint32_t v = u << k;
+  const uint32_t j = (v >> 26) & 31u;
+  const float f = (float)((v >> 10) & 0xffffu) * 0x1p-16f;
+  const float t0 = gauss_quantile[k][j];
+  const float d = gauss_quantile[k][j + 1] - t0;
+  const float step = d * f;
+  return t0 + step;
+}
+
 void oracle_fill_synthetic(void* out, int dtype, size_t n, uint64_t seed, uint64_t first_index, int dist, double a,
                            double b) {
-  const float fa = dist == 2 ? (float)((b - a) / 16777216.0) : (float)(a / sqrt((65536.0 * 65536.0 - 1.0) / 3.0));
+  const int gauss = dist == 3 || dist == 4;
+  const float fa = dist == 2 ? (float)((b - a) / 16777216.0)
+                             : gauss ? (float)a : (float)(a / sqrt((65536.0 * 65536.0 - 1.0) / 3.0));
   const float fb = dist == 2 ? (float)a : (float)b;
 #pragma omp parallel for schedule(static)
   for (size_t i = 0; i < n; ++i) {
@@ -86,6 +104,11 @@ void oracle_fill_synthetic(void* out, int dtype, size_t n, uint64_t seed, uint64
     if (dist == 2) {
       x = (float)(uint32_t)(z >> 40) * fa;
       x = x + fb;
+    } else if (gauss) {
+      const float mag = synth_gauss_magnitude((uint32_t)(z >> 31));
+      x = (z >> 63) ? -mag : mag;
+      x = x * fa;
+      if (dist == 4 && synth_hash(seed ^ 0xA5A5A5A5A5A5A5A5ull, first_index + i) % 100ull == 0ull) x = x * fb;
     } else {
       const int32_t sum = (int32_t)((z & 0xffffu) + ((z >> 16) & 0xffffu) + ((z >> 32) & 0xffffu) + (z >> 48)) - 131070;
       x = (float)sum * fa;

@@ -648,7 +648,37 @@ class SFTEngineOptimizerSide(_EngineBase):
 # --------------------------------------------------------------------------
 
 _M64 = (1 << 64) - 1
-SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM = 0, 1, 2
+SYNTH_NORMAL, SYNTH_NORMAL_OUTLIERS, SYNTH_UNIFORM, SYNTH_GAUSSIAN, SYNTH_GAUSSIAN_OUTLIERS = 0, 1, 2, 3, 4
+_GAUSS_TABLE: Optional[np.ndarray] = None
+
+
+def gauss_quantile_table() -> np.ndarray:
+    """The 32 x 33 float32 quantile table of the Gaussian modes, read from the header the device code
+    compiles (mlx-node_amd/csrc/mxopt_gauss_table.h: hexadecimal literals, exact)."""
+    global _GAUSS_TABLE
+    if _GAUSS_TABLE is None:
+        import os
+        import re
+        path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "mlx-node_amd", "csrc",
+                            "mxopt_gauss_table.h")
+        vals = [float.fromhex(h) for h in re.findall(r"(-?0x[0-9a-f.]+p[+-]\d+)f", open(path).read())]
+        _GAUSS_TABLE = np.array(vals, dtype=np.float64).astype(F32).reshape(32, 33)
+    return _GAUSS_TABLE
+
+
+def _gauss_magnitude(u: np.ndarray) -> np.ndarray:
+    """|x| for the 32-bit tail code u (see MXOPT_SYNTH_GAUSSIAN in include/mxopt.h): three float32 ops."""
+    t = gauss_quantile_table()
+    u = np.where(u == 0, 1, u).astype(np.uint64)
+    _, e = np.frexp(u.astype(np.float64))            # u in [2^(e-1), 2^e): exact for 32-bit integers
+    k = (32 - e).astype(np.int64)                     # leading zeros
+    v = (u << k.astype(np.uint64)) & np.uint64(0xFFFFFFFF)
+    j = ((v >> np.uint64(26)) & np.uint64(31)).astype(np.int64)
+    f = ((v >> np.uint64(10)) & np.uint64(0xFFFF)).astype(F32) * F32(2.0 ** -16)
+    t0 = t[k, j]
+    d = t[k, j + 1] - t0
+    step = d * f
+    return t0 + step
 
 
 def _splitmix_finish(z: np.ndarray) -> np.ndarray:
@@ -678,6 +708,13 @@ def synthetic(n: int, dtype: str, seed: int, distribution: int = SYNTH_NORMAL, a
     if distribution == SYNTH_UNIFORM:
         x = (z >> np.uint64(40)).astype(F32) * _f32((b - a) / 16777216.0)
         x = x + _f32(a)
+    elif distribution in (SYNTH_GAUSSIAN, SYNTH_GAUSSIAN_OUTLIERS):
+        mag = _gauss_magnitude((z >> np.uint64(31)) & np.uint64(0xFFFFFFFF))
+        x = np.where((z >> np.uint64(63)) != 0, -mag, mag).astype(F32)
+        x = x * _f32(a)
+        if distribution == SYNTH_GAUSSIAN_OUTLIERS:
+            hit = synthetic_hash(seed ^ 0xA5A5A5A5A5A5A5A5, idx) % np.uint64(100) == np.uint64(0)
+            x = np.where(hit, x * _f32(b), x).astype(F32)
     else:
         m = np.uint64(0xFFFF)
         total = ((z & m) + ((z >> np.uint64(16)) & m) + ((z >> np.uint64(32)) & m) + (z >> np.uint64(48))).astype(np.int64)

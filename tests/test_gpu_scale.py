@@ -170,10 +170,12 @@ def test_config1_bias_corrected_per_call_step_count(oracle_c):
 # config 2
 # ---------------------------------------------------------------------------------------
 
-def test_config2_full_size_every_element(oracle_c):
+@pytest.mark.parametrize("tails", ["bell", "gaussian"])
+def test_config2_full_size_every_element(oracle_c, tails):
     """Inputs come from the library's counter-based generator on the device and are regenerated on the
     host by the oracle's twin of it: nothing is copied to the device, every one of 1.72 G elements of
-    p, m and v is compared after each of two steps."""
+    p, m and v is compared after each of two steps.  Once with the four-uniform bell (|x| <= 3.46 sigma),
+    once with the Gaussian mode, whose tails reach 6 sigma before the x100 outliers multiply them."""
     import torch
     import mxopt as mx
     _, sizes = qwen_sizes("1.7B")
@@ -187,11 +189,13 @@ def test_config2_full_size_every_element(oracle_c):
     dv = [torch.zeros(s, device="cuda") for s in sizes]
     ctx = mx.Context()
     SEED, CFG = 0x5EED0001, 2
+    PLAIN, SPIKED = ((O.SYNTH_NORMAL, O.SYNTH_NORMAL_OUTLIERS) if tails == "bell"
+                     else (O.SYNTH_GAUSSIAN, O.SYNTH_GAUSSIAN_OUTLIERS))
     p_ref = np.empty(n, np.uint16)
     for i in range(nt):
         key = mx.synthetic_key(SEED, CFG, 0, 0, i)
-        ctx.fill_synthetic(dp[i], key, mx.SYNTH_NORMAL, 0.02)
-        p_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, O.SYNTH_NORMAL, 0.02)
+        ctx.fill_synthetic(dp[i], key, PLAIN, 0.02)
+        p_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, PLAIN, 0.02)
     t_g = ctx.table([mx.TensorSpec(g=g) for g in dg])
     t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp, dg, dm, dv)])
     hp = mx.adam_hp(5e-6, 0.9, 0.999, 1e-8, 0.01)
@@ -204,8 +208,10 @@ def test_config2_full_size_every_element(oracle_c):
     for step in range(2):
         for i in range(nt):                     # fresh gradients each step: 1 % of the elements x100
             key = mx.synthetic_key(SEED, CFG, step + 1, 1, i)
-            ctx.fill_synthetic(dg[i], key, mx.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0)
-            g_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0)
+            ctx.fill_synthetic(dg[i], key, SPIKED, 1e-3, 100.0)
+            g_ref[offs[i]:offs[i + 1]] = oracle_c.fill_synthetic(sizes[i], "bf16", key, SPIKED, 1e-3, 100.0)
+        top = float(O.bf16_to_f32(g_ref[:50_000_000]).__abs__().max())
+        assert (top > 0.45) if tails == "gaussian" else (top <= 0.347)     # 100 x 4.5 sigma and more, or capped at 100 x 3.46 sigma
         ctx.global_norm(t_g, res, max_norm=1.0)
         ctx.adam(t_upd, hp, mx.make_prep(scale=res))
         r = ctx.read_norm_result(res)

@@ -10,7 +10,8 @@ from gpu_util import assert_bit_equal, to_host
 
 
 @pytest.mark.parametrize("dist,a,b", [(O.SYNTH_NORMAL, 1e-3, 0.0), (O.SYNTH_NORMAL_OUTLIERS, 1e-3, 100.0),
-                                      (O.SYNTH_UNIFORM, 0.9, 1.1), (O.SYNTH_NORMAL, 0.02, 0.0)])
+                                      (O.SYNTH_UNIFORM, 0.9, 1.1), (O.SYNTH_NORMAL, 0.02, 0.0),
+                                      (O.SYNTH_GAUSSIAN, 1e-3, 0.0), (O.SYNTH_GAUSSIAN_OUTLIERS, 0.02, 100.0)])
 @pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
 def test_device_fill_equals_the_oracle(dist, a, b, dt):
     import torch
