@@ -3,7 +3,10 @@
  *   cabi_demo            known-answer checks through the optimizer objects (the reference's own
  *                        closed forms: __test__/core/optimizers.test.ts:151-203, 324-351) and the
  *                        engine entry points (with and without an accumulation buffer), then a timing of updateSingle-per-tensor against
- *                        one update_many call over the Qwen3-0.6B parameter list.
+ *                        one update_many call over the Qwen3-0.6B parameter list; before that the
+ *                        region-interleaved pool (moments taken from it, the bare probes on its memory and on
+ *                        plain memory), the global norm that allocates nothing, and the GRPO engine's call
+ *                        that does not wait for the validity flag.
  * Prints "PASS" lines and one "TIMING" line; exits non-zero on the first mismatch.
  */
 #define _POSIX_C_SOURCE 200809L
@@ -188,6 +191,122 @@ static void long_cycle(void) {
   }
 }
 
+/* The start-up utilities and the two entry points for hosts with constraints: a pool whose memory alternates
+ * between the device's physical regions, optimizer state taken from it, the probes that show what that is
+ * worth, mxopt_global_norm_static against mxopt_global_norm, and the asynchronous GRPO micro-batch call with a
+ * NaN micro-batch in the middle of a cycle. */
+static double probe_gbps(int kind, void* a, void* b, void* c, void* d, uint64_t n, double streams) {
+  CHECK_MX(mxopt_probe_stream(ctx, kind, a, b, c, d, n));
+  CHECK_MX(mxopt_synchronize(ctx));
+  const double t0 = now_ms();
+  for (int i = 0; i < 5; ++i) CHECK_MX(mxopt_probe_stream(ctx, kind, a, b, c, d, n));
+  CHECK_MX(mxopt_synchronize(ctx));
+  return streams * (double)n * 4.0 / 1e9 / ((now_ms() - t0) / 5.0 * 1e-3);
+}
+
+static void pool_and_friends(void) {
+  const uint64_t n = (uint64_t)1 << 28;  /* 1 GiB per stream */
+  void* plain[4];
+  for (int i = 0; i < 4; ++i) CHECK_HIP(hipMalloc(&plain[i], n * 4));
+  const double plain_mix = probe_gbps(MXOPT_PROBE_MIX43, plain[0], plain[1], plain[2], plain[3], n, 7.0);
+  for (int i = 0; i < 4; ++i) CHECK_HIP(hipFree(plain[i]));
+
+  mxopt_hbm_pool* pool = NULL;
+  CHECK_MX(mxopt_hbm_pool_create(ctx, (size_t)6 << 30, 0, 0, &pool));
+  mxopt_hbm_pool_info info;
+  CHECK_MX(mxopt_hbm_pool_get_info(pool, &info));
+  void* arena[4];
+  for (int i = 0; i < 4; ++i) CHECK_MX(mxopt_hbm_pool_alloc(pool, n * 4, &arena[i]));
+  const double arena_mix = probe_gbps(MXOPT_PROBE_MIX43, arena[0], arena[1], arena[2], arena[3], n, 7.0);
+  printf("POOL regions=%d chunk_mib=%llu setup_s=%.2f (create %.2f, scan %.2f) probes=%d same_region_gbps=%.0f cross_region_gbps=%.0f "
+         "mix43_plain_gbps=%.0f mix43_arena_gbps=%.0f\n", info.regions, (unsigned long long)(info.chunk_bytes >> 20),
+         info.setup_seconds, info.create_seconds, info.scan_seconds, info.probes, info.probe_same_region_gbps, info.probe_cross_region_gbps, plain_mix, arena_mix);
+  for (int i = 0; i < 4; ++i) {
+    if (!mxopt_hbm_pool_owns(pool, arena[i])) { fprintf(stderr, "FAIL pool does not own its allocation\n"); exit(1); }
+    CHECK_MX(mxopt_hbm_pool_free(pool, arena[i]));
+  }
+
+  /* moments from the pool: AdamW, lr 0.1, zero state, no decay -> first step moves every weight by lr * g / (|g| + eps) ... */
+  CHECK_MX(mxopt_set_state_pool(ctx, pool));
+  const float p0[3] = {1.0f, 2.0f, 3.0f}, g0[3] = {0.5f, -0.25f, 0.125f};
+  float *dp = to_device(p0, 3), *dg = to_device(g0, 3), *m = NULL, *v = NULL;
+  const mxopt_array ap = {dp, 3, MXOPT_F32}, ag = {dg, 3, MXOPT_F32};
+  const double lr = 0.1, wd = 0.0, b1 = 0.9, b2 = 0.999, eps = 1e-8;
+  const int bias = 1;
+  mxopt_optimizer* opt = NULL;
+  CHECK_MX(mxopt_adamw_new(ctx, &lr, &b1, &b2, &eps, &wd, &bias, &opt));
+  CHECK_MX(mxopt_optimizer_update_single(opt, "w", &ap, &ag, &ap));
+  uint64_t cnt = 0;
+  int hv = 0;
+  CHECK_MX(mxopt_optimizer_state(opt, "w", &m, &v, &cnt, &hv));
+  if (!mxopt_hbm_pool_owns(pool, m) || !mxopt_hbm_pool_owns(pool, v)) { fprintf(stderr, "FAIL moments are not in the pool\n"); exit(1); }
+  /* ... with bias correction m_hat = g, v_hat = g^2: p - lr * sign(g) up to eps */
+  const double want[3] = {1.0 - 0.1, 2.0 + 0.1, 3.0 - 0.1};
+  expect_close("AdamW with its moments in the region-interleaved pool", dp, want, 3, 1e-6);
+  mxopt_optimizer_free(opt);
+  CHECK_MX(mxopt_set_state_pool(ctx, NULL));
+
+  /* the norm that allocates nothing against the one that sizes a buffer on first use: same bits */
+  enum { NN = 100003 };
+  float* hg = malloc(NN * sizeof *hg);
+  for (int i = 0; i < NN; ++i) hg[i] = (float)((i * 2654435761u) % 2001u) * 1e-3f - 1.0f;
+  float* dgn = to_device(hg, NN);
+  mxopt_tensor row;
+  memset(&row, 0, sizeof row);
+  row.g = dgn; row.n = NN; row.g_dtype = MXOPT_F32; row.bc1 = row.bc2 = 1.0f;
+  mxopt_table* t = NULL;
+  CHECK_MX(mxopt_table_build(ctx, &row, 1, &t));
+  mxopt_norm_result *d_res = NULL, a, b;
+  CHECK_HIP(hipMalloc((void**)&d_res, 2 * sizeof *d_res));
+  CHECK_MX(mxopt_global_norm_static(ctx, t, 0, NULL, 1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, &d_res[0]));
+  CHECK_MX(mxopt_global_norm(ctx, t, 0, NULL, 1.0, MXOPT_CLIP_ALWAYS_MULTIPLY, &d_res[1]));
+  CHECK_MX(mxopt_read_norm_result(ctx, &d_res[0], &a));
+  CHECK_MX(mxopt_read_norm_result(ctx, &d_res[1], &b));
+  double exact = 0.0;
+  for (int i = 0; i < NN; ++i) exact += (double)hg[i] * hg[i];
+  if (memcmp(&a, &b, sizeof a) != 0 || fabs(a.sumsq - exact) > 1e-6 * exact) {
+    fprintf(stderr, "FAIL static norm %.17g, allocating norm %.17g, exact %.17g\n", a.sumsq, b.sumsq, exact);
+    exit(1);
+  }
+  printf("PASS mxopt_global_norm_static: bit-identical to mxopt_global_norm, sum of squares %.9g\n", a.sumsq);
+  mxopt_table_destroy(t);
+  CHECK_HIP(hipFree(d_res));
+  CHECK_HIP(hipFree(dgn));
+  free(hg);
+
+  /* GRPO engine, two micro-batches per step, lr 0.5, no clamp or clip in reach: good, NaN (skipped), good
+   * -> p = 1 - 0.5/2 * (0.25 + 0.25) after the third call, the NaN call counted, nothing waited for */
+  mxopt_engine_config cfg;
+  mxopt_engine_config_default(MXOPT_ENGINE_GRPO, &cfg);
+  cfg.gradient_accumulation_steps = 2;
+  cfg.learning_rate = 0.5;
+  cfg.gradient_clip_norm = 1e9;
+  const float one[4] = {1.0f, 1.0f, 1.0f, 1.0f}, good[4] = {0.25f, 0.25f, 0.25f, 0.25f};
+  float bad[4] = {0.25f, 0.25f, 0.25f, 0.25f};
+  bad[2] = NAN;
+  float *w = to_device(one, 4), *dgood = to_device(good, 4), *dbad = to_device(bad, 4);
+  const char* names[1] = {"w"};
+  const mxopt_array aw = {w, 4, MXOPT_F32}, agood = {dgood, 4, MXOPT_F32}, abad = {dbad, 4, MXOPT_F32};
+  mxopt_engine* eng = NULL;
+  CHECK_MX(mxopt_engine_new(ctx, &cfg, 1, names, &aw, &eng));
+  CHECK_MX(mxopt_engine_micro_batch_async(eng, 1, names, &agood));
+  CHECK_MX(mxopt_engine_micro_batch_async(eng, 1, names, &abad));
+  CHECK_MX(mxopt_engine_micro_batch_async(eng, 1, names, &agood));
+  mxopt_engine_metrics em;
+  CHECK_MX(mxopt_engine_settle(eng, &em));
+  if (em.step != 3 || em.nan_gradient_count != 1 || em.micro_step != 0 || !em.gradients_applied) {
+    fprintf(stderr, "FAIL async engine bookkeeping: step %lld nan %llu micro %d applied %d\n", (long long)em.step,
+            (unsigned long long)em.nan_gradient_count, em.micro_step, em.gradients_applied);
+    exit(1);
+  }
+  const double want_w[4] = {0.875, 0.875, 0.875, 0.875};
+  expect_close("GRPO engine, asynchronous micro-batches with a NaN one in the middle of the cycle", w, want_w, 4, 0.0);
+  mxopt_engine_free(eng);
+  CHECK_HIP(hipFree(w)); CHECK_HIP(hipFree(dgood)); CHECK_HIP(hipFree(dbad));
+  CHECK_HIP(hipFree(dp)); CHECK_HIP(hipFree(dg));
+  mxopt_hbm_pool_destroy(pool);
+}
+
 /* Qwen3-0.6B: vocab 151936, hidden 1024, 28 layers, q 2048x1024, k/v 1024x1024, o 1024x2048,
  * gate/up 3072x1024, down 1024x3072, four norm vectors per layer, final norm, tied embedding. */
 static size_t qwen3_06b(size_t* sizes) {
@@ -254,6 +373,7 @@ int main(int argc, char** argv) {
   printf("%s\n", mxopt_version());
   known_answers();
   long_cycle();
+  pool_and_friends();
   if (argc < 2 || strcmp(argv[1], "--no-timing") != 0) timing();
   mxopt_destroy(ctx);
   return 0;

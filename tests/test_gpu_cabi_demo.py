@@ -1,6 +1,7 @@
 """The plain-C host (mlx-node_amd/examples/cabi_demo.c, built by mlx-node_amd/build.py): known answers
 of the reference's own tests through the C ABI with no Python in between, and the cost of the
-updateSingle-per-tensor loop against one update_many call from compiled host code."""
+updateSingle-per-tensor loop against one update_many call from compiled host code; the region-interleaved pool,
+the allocation-free norm and the asynchronous engine call from plain C."""
 import os
 import re
 import subprocess
@@ -18,7 +19,11 @@ def test_plain_c_host_known_answers_and_timing():
     proc = subprocess.run([DEMO], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     passed = [l for l in proc.stdout.splitlines() if l.startswith("PASS")]
-    assert len(passed) == 6, proc.stdout
+    assert len(passed) == 9, proc.stdout
+    pool = re.search(r"POOL regions=(\d+) .* mix43_plain_gbps=(\d+) mix43_arena_gbps=(\d+)", proc.stdout)
+    assert pool and int(pool.group(1)) >= 1, proc.stdout
+    if int(pool.group(1)) >= 2:      # most of the device free: the arena's memory must not be slower than plain memory
+        assert int(pool.group(3)) > 0.97 * int(pool.group(2)), proc.stdout
     m = re.search(r"TIMING tensors=(\d+) elements=(\d+) update_single_loop_ms=([\d.]+) \(host enqueue ([\d.]+)\) "
                   r"update_many_ms=([\d.]+)", proc.stdout)
     assert m, proc.stdout
