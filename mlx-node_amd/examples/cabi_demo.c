@@ -212,7 +212,7 @@ static void pool_and_friends(void) {
   for (int i = 0; i < 4; ++i) CHECK_HIP(hipFree(plain[i]));
 
   mxopt_hbm_pool* pool = NULL;
-  CHECK_MX(mxopt_hbm_pool_create(ctx, (size_t)6 << 30, 0, 0, &pool));
+  CHECK_MX(mxopt_hbm_pool_create(ctx, (size_t)6 << 30, 0, 2, &pool));
   mxopt_hbm_pool_info info;
   CHECK_MX(mxopt_hbm_pool_get_info(pool, &info));
   void* arena[4];

@@ -55,6 +55,24 @@ def test_pool_finds_regions_and_interleaves(mx, pool):
     assert i.probes > 0 and 0 < i.scan_seconds <= i.setup_seconds < 30
 
 
+def test_pool_limited_to_two_regions(mx, ctx, pool):
+    """max_regions = 2: the arena alternates between the two regions with the most free memory only."""
+    small = ctx.hbm_pool(3 * GiB, 0, 2)
+    try:
+        i = small.info()
+        assert i.capacity_bytes == 3 * GiB and i.regions >= 1
+        assert sum(i.region_arena_bytes) == i.capacity_bytes
+        if i.regions >= 2:
+            assert i.probe_cross_region_gbps > 1.07 * i.probe_same_region_gbps
+            assert abs(i.region_arena_bytes[0] - i.region_arena_bytes[1]) <= i.chunk_bytes
+            assert sum(i.region_arena_bytes[2:]) == 0
+        a = small.alloc(3 * GiB)
+        assert small.owns(a) and not pool.owns(a)
+        small.free(a)
+    finally:
+        small.close()
+
+
 def test_pool_allocator_first_fit_coalesces_and_refuses(mx, ctx, pool):
     a = pool.alloc(1000)
     b = pool.alloc(3 * GiB)
