@@ -109,7 +109,8 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * with the device).  Whatever is allocated from the arena has its traffic spread over the regions,
  * whichever streams a kernel combines; this replaces the luck of mxopt_hbm_spread_begin/_end.
  * If all free memory lies in one region (regions == 1 in the info) the arena still works, without
- * the gain.  chunk_bytes = 0: 64 MiB (a power of two in [2 MiB, 1 GiB]).  max_regions = 0: alternate
+ * the gain.  chunk_bytes = 0: 64 MiB (a power of two in [2 MiB, 1 GiB]; the free memory must make at
+ * most 24 000 chunks, i.e. 16 MiB or more on an empty device).  max_regions = 0: alternate
  * between all regions found; 2: between the two with the most free memory (read-only passes lose about
  * 3 % on memory interleaved over two regions and 6 - 10 % over three, read-write passes gain 13 - 20 %
  * either way).  Allocations are 512-byte

@@ -215,7 +215,7 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
   if (want_chunks > avail_chunks)
     return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": " + std::to_string(capacity_bytes >> 20) + " MiB wanted, " +
                                         std::to_string(free_b >> 20) + " MiB free");
-  if (avail_chunks > 60000)  // the driver limits the number of live allocations of a process
+  if (avail_chunks > 24000)  // the driver limits the number of live allocations of a process, and maps fewer still
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": chunk_bytes too small for this much free memory");
 
   // 1. All free memory as physical chunks: memory far from what a small allocation would get can

@@ -199,9 +199,9 @@ static double probe_gbps(int kind, void* a, void* b, void* c, void* d, uint64_t 
   CHECK_MX(mxopt_probe_stream(ctx, kind, a, b, c, d, n));
   CHECK_MX(mxopt_synchronize(ctx));
   const double t0 = now_ms();
-  for (int i = 0; i < 5; ++i) CHECK_MX(mxopt_probe_stream(ctx, kind, a, b, c, d, n));
+  for (int i = 0; i < 10; ++i) CHECK_MX(mxopt_probe_stream(ctx, kind, a, b, c, d, n));
   CHECK_MX(mxopt_synchronize(ctx));
-  return streams * (double)n * 4.0 / 1e9 / ((now_ms() - t0) / 5.0 * 1e-3);
+  return streams * (double)n * 4.0 / 1e9 / ((now_ms() - t0) / 10.0 * 1e-3);
 }
 
 static void pool_and_friends(void) {
