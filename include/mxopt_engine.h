@@ -107,7 +107,7 @@ void mxopt_engine_free(mxopt_engine* e);
 int mxopt_engine_micro_batch(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads,
                              mxopt_engine_metrics* out);
 
-/* mxopt_engine_micro_batch for the GRPO engine (apply = SGD) without its one host synchronisation: the
+/* mxopt_engine_micro_batch for the GRPO engine (either apply mode) without its one host synchronisation: the
  * blocking call reads the validity flag back (32 bytes) before it decides whether to accumulate, where
  * the reference reads every gradient back for the same test (grpo/engine.rs:563-569).  Here the flag
  * stays on the device: the norm pass writes it, every kernel of the call that would change memory
@@ -118,8 +118,11 @@ int mxopt_engine_micro_batch(mxopt_engine* e, size_t n, const char* const* names
  * (NaN counters, emergency flag, `step`).  Results -- parameters, buffers, counters -- are those of the
  * blocking calls.  Two differences in timing: metrics come from mxopt_engine_settle, and the
  * "Training stopped" failure of a micro-batch that reaches max_nan_gradients is returned by the call
- * that settles it.  With defer_accumulation the caller keeps a micro-batch's gradient buffers alive
- * as for the blocking call. */
+ * that settles it.  With apply = ADAMW the optimizer's call counter goes back with the rest; moments
+ * that a skipped first update allocated stay, zero-filled, which is what a later first update starts
+ * from anyway.  With defer_accumulation the caller keeps a micro-batch's gradient buffers alive as for
+ * the blocking call.  The SFT engine is refused: it reads nothing back unless the caller asks for
+ * metrics. */
 int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const* names, const mxopt_array* grads);
 /* Waits for the last async micro-batch's flag (a no-op after a blocking call) and returns the metrics the
  * blocking call would have returned for it.  `out` may be NULL. */

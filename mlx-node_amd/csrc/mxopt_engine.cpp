@@ -63,6 +63,7 @@ struct mxopt_engine {
     int64_t step;
     uint64_t nan_gradient_count;
     uint32_t consecutive_nan_count;
+    int64_t adamw_calls;  // APPLY_ADAMW: the optimizer object's call counter
     std::vector<size_t> held_slots;
     std::vector<std::vector<mxopt_array>> held;
     std::vector<int> held_result;
@@ -85,6 +86,7 @@ mxopt_engine::Book take_book(const mxopt_engine* e) {
   b.have_acc = e->have_acc; b.needs_emergency_save = e->needs_emergency_save; b.held_is_sum = e->held_is_sum;
   b.micro_step = e->micro_step; b.step = e->step; b.nan_gradient_count = e->nan_gradient_count;
   b.consecutive_nan_count = e->consecutive_nan_count;
+  b.adamw_calls = e->adamw ? mxopt_optimizer_step_count(e->adamw) : 0;
   b.held_slots = e->held_slots; b.held = e->held; b.held_result = e->held_result;
   b.in_acc.resize(e->slots.size());
   for (size_t i = 0; i < e->slots.size(); ++i) b.in_acc[i] = e->slots[i].in_acc ? 1 : 0;
@@ -95,6 +97,7 @@ void put_book(mxopt_engine* e, const mxopt_engine::Book& b) {
   e->have_acc = b.have_acc; e->needs_emergency_save = b.needs_emergency_save; e->held_is_sum = b.held_is_sum;
   e->micro_step = b.micro_step; e->step = b.step; e->nan_gradient_count = b.nan_gradient_count;
   e->consecutive_nan_count = b.consecutive_nan_count;
+  if (e->adamw) optimizer_set_step_count(e->adamw, b.adamw_calls);  // the update it counted did nothing on the device
   e->held_slots = b.held_slots; e->held = b.held; e->held_result = b.held_result;
   for (size_t i = 0; i < e->slots.size() && i < b.in_acc.size(); ++i) e->slots[i].in_acc = b.in_acc[i] != 0;
 }
@@ -925,10 +928,10 @@ int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const*
   const char* op = "mxopt_engine_micro_batch_async";
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null engine");
   mxopt_ctx* ctx = e->ctx;
-  if (e->cfg.kind != MXOPT_ENGINE_GRPO || e->cfg.apply != MXOPT_ENGINE_APPLY_SGD)
+  if (e->cfg.kind != MXOPT_ENGINE_GRPO)
     return fail(ctx, MXOPT_ERR_INVALID_ARG,
-                std::string(op) + ": only the GRPO engine with the plain-SGD apply reads a flag back per micro-batch; "
-                                  "the other modes do not block as they are");
+                std::string(op) + ": only the GRPO engine reads a flag back per micro-batch; the SFT engine does not "
+                                  "block as it is");
   int rc = settle(e, nullptr);  // the previous micro-batch's flag has long arrived; a skip is booked now
   if (rc) return rc;
   std::vector<size_t> idx;

@@ -77,5 +77,8 @@ int check_array(mxopt_ctx* ctx, const mxopt_array* a, const char* what, bool all
 // keeps the most recently used few.
 int cached_table(mxopt_ctx* ctx, std::vector<mxopt_tensor>& rows, mxopt_table** out);
 int norm_scratch(mxopt_ctx* ctx, mxopt_norm_result** out);
+// Puts an optimizer's call counter (mxopt_optimizer_step_count) back: for a caller whose conditional
+// update turned out to have been skipped on the device.
+void optimizer_set_step_count(mxopt_optimizer* opt, int64_t calls);
 
 }  // namespace mxopt

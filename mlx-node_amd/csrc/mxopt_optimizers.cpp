@@ -111,6 +111,8 @@ struct mxopt_optimizer {
   mxopt_table* many_table = nullptr;
 };
 
+void mxopt::optimizer_set_step_count(mxopt_optimizer* opt, int64_t calls) { opt->step = calls; }
+
 namespace {
 
 bool is_adam(const mxopt_optimizer* o) { return o->kind == Kind::Adam || o->kind == Kind::AdamW; }

@@ -34,18 +34,20 @@ def poisoned(rng, bf16, it, kind):
 
 
 @pytest.mark.parametrize("bf16", [False, True])
-@pytest.mark.parametrize("defer", [False, True])
+@pytest.mark.parametrize("mode", ["sgd", "sgd-deferred", "adamw"])
 @pytest.mark.parametrize("n_acc", [1, 3])
-def test_async_settled_after_every_micro_batch(mx, bf16, defer, n_acc):
+def test_async_settled_after_every_micro_batch(mx, tmp_path, bf16, mode, n_acc):
     """Every call is settled before the next: the speculative bookkeeping, the guarded kernels and the
     roll-back are exercised, and the device's own sum of squares can be handed to the oracle (clip active)."""
     rng = np.random.default_rng(41 + n_acc)
     params = make_params(rng, bf16)
     dparams = {k: to_dev(v) for k, v in params.items()}
+    defer = mode == "sgd-deferred"
     kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=2.0, gradient_clip_value=0.02,
-              max_nan_gradients=50, emergency_save_threshold=2)
+              max_nan_gradients=50, emergency_save_threshold=2, apply=mode.split("-")[0], weight_decay=0.01)
     dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=defer, **kw)
     ref = O.GRPOEngineOptimizerSide(params, **kw)
+    applied = 0
     for it, kind in enumerate(SCRIPT):
         grads = poisoned(rng, bf16, it, kind)
         dev.micro_batch_async({k: to_dev(g) for k, g in grads.items()})
@@ -57,21 +59,31 @@ def test_async_settled_after_every_micro_batch(mx, bf16, defer, n_acc):
         else:
             r = ref.micro_batch(grads)
         assert (bool(m.skipped), bool(m.gradients_applied), m.step) == (r["skipped"], r["gradients_applied"], r["step"]), it
+        applied += int(r["gradients_applied"])
         check_state(dev, ref, dparams, f"micro-batch {it} ({kind})")
     assert ref.state.nan_gradient_count == 5
+    if mode == "adamw":      # the optimizer object's call counter saw only the updates that took place
+        import ctypes as C
+        path = tmp_path / "state.safetensors"
+        dev.save_optimizer_state(path)
+        kind, step, tensors, elements = C.create_string_buffer(32), C.c_int64(), C.c_uint64(), C.c_uint64()
+        assert mx.load().mxopt_checkpoint_inspect(str(path).encode(), kind, 32, C.byref(step), C.byref(tensors),
+                                                  C.byref(elements)) == 0
+        assert step.value == applied * len(params)
 
 
-@pytest.mark.parametrize("defer", [False, True])
+@pytest.mark.parametrize("mode", ["sgd", "sgd-deferred", "adamw"])
 @pytest.mark.parametrize("n_acc", [2, 4])
-def test_async_pipelined_never_settled_in_between(mx, defer, n_acc):
+def test_async_pipelined_never_settled_in_between(mx, mode, n_acc):
     """No settle between the calls: each call books its predecessor's flag itself.  The clip threshold is out
     of reach (factor exactly 1), so the oracle needs no figure from the device and every call can be left
     unsettled; blocking calls and getters mixed in must settle by themselves."""
     rng = np.random.default_rng(43)
     params = make_params(rng, True)
     dparams = {k: to_dev(v) for k, v in params.items()}
+    defer = mode == "sgd-deferred"
     kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=1e9, gradient_clip_value=0.02,
-              max_nan_gradients=50, emergency_save_threshold=2)
+              max_nan_gradients=50, emergency_save_threshold=2, apply=mode.split("-")[0], weight_decay=0.01)
     dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=defer, **kw)
     ref = O.GRPOEngineOptimizerSide(params, **kw)
     keep = []
@@ -113,9 +125,7 @@ def test_async_training_stopped_surfaces_when_settled(mx):
 def test_async_is_refused_where_nothing_blocks(mx):
     dparams = {"w": to_dev(np.ones(100, F))}
     g = {"w": to_dev(np.zeros(100, F))}
-    with pytest.raises(mx.InvalidArg, match="only the GRPO engine with the plain-SGD apply"):
+    with pytest.raises(mx.InvalidArg, match="only the GRPO engine reads a flag back"):
         mx.SFTEngineOptimizerSide(dparams).micro_batch_async(g)
-    with pytest.raises(mx.InvalidArg, match="only the GRPO engine with the plain-SGD apply"):
-        mx.GRPOEngineOptimizerSide(dparams, apply="adamw").micro_batch_async(g)
     dev = mx.GRPOEngineOptimizerSide(dparams)
     assert dev.settle().step == 0             # nothing pending: a no-op

@@ -112,7 +112,7 @@ def test_random_engine_sequences(mx, kind, bf16, apply, n_acc, defer, acc_f32, c
 
             # GRPO with the plain-SGD apply also through the call that does not wait for the validity flag: booked as
             # valid, kernels guarded on the device, put right by settle()
-            if use_async and kind == "grpo" and apply == "sgd":
+            if use_async and kind == "grpo":
                 def dev_call(grads=grads):
                     dev.micro_batch_async({k: to_dev(g) for k, g in grads.items()})
                     return dev.settle()
