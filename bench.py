@@ -731,7 +731,13 @@ def main():
     if args.placement == "pool":
         # the arena takes the free memory but for a margin left to torch's own scratch and the runtime
         free = torch.cuda.mem_get_info()[0]
-        pool = ctx.hbm_pool(free - (8 << 30), args.pool_chunk_mb << 20, args.pool_regions)
+        try:
+            pool = ctx.hbm_pool(free - (8 << 30), args.pool_chunk_mb << 20, args.pool_regions)
+        except mxopt.MxoptError as e:
+            # e.g. another process holds most of the device: measure in plain memory and say so in the line
+            print(f"bench.py: no region-interleaved arena ({e}); buffers come from plain device memory", file=sys.stderr)
+            placement = {"kind": "plain", "arena_refused": str(e)}
+    if pool is not None:
         pool.use_for_state()
         i = pool.info()
         placement = {"kind": "mxopt_hbm_pool", "chunk_mib": i.chunk_bytes >> 20, "regions_found": i.regions,
