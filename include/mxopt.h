@@ -114,7 +114,8 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * between all regions found; 2: between the two with the most free memory (read-only passes lose about
  * 3 % on memory interleaved over two regions and 6 - 10 % over three, read-write passes gain 13 - 20 %
  * either way).  Allocations are 512-byte
- * aligned, first fit, thread-safe; contents are not cleared.  Destroy the pool after everything that
+ * aligned, first fit, thread-safe; contents are not cleared.  A pointer goes back to the pool it came
+ * from whichever pool a context or the hooks point at by then.  Destroy the pool after everything that
  * allocated from it.  No counterpart in the reference (MLX owns its allocator there). */
 #define MXOPT_HBM_MAX_REGIONS 8
 typedef struct mxopt_hbm_pool mxopt_hbm_pool;
@@ -136,7 +137,9 @@ typedef struct mxopt_hbm_pool_info {
 } mxopt_hbm_pool_info;
 int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
                           mxopt_hbm_pool** out);
-void mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool);
+/* Refused (MXOPT_ERR_INVALID_ARG, nothing happens) while allocations from the pool are live: their memory would
+ * be unmapped under whoever still uses it. */
+int mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool);
 int mxopt_hbm_pool_alloc(mxopt_hbm_pool* pool, size_t bytes, void** out);
 int mxopt_hbm_pool_free(mxopt_hbm_pool* pool, void* ptr);
 int mxopt_hbm_pool_owns(const mxopt_hbm_pool* pool, const void* ptr);   /* 1 if ptr lies inside the arena */

@@ -177,6 +177,20 @@ hipMemAccessDesc rw_access(int device) {
   return acc;
 }
 
+// Every live pool of the process: a pointer is given back to the pool it came from, whichever pool a
+// context or the allocator hooks point at by then.
+std::mutex g_pools_mu;
+std::vector<mxopt_hbm_pool*> g_pools;
+std::mutex g_hook_mu;
+mxopt_hbm_pool* g_hook_pool = nullptr;
+
+mxopt_hbm_pool* pool_of(const void* ptr) {
+  std::lock_guard<std::mutex> all(g_pools_mu);
+  for (mxopt_hbm_pool* p : g_pools)
+    if (ptr && (const char*)ptr >= p->base && (const char*)ptr < p->base + p->capacity) return p;
+  return nullptr;
+}
+
 }  // namespace
 
 extern "C" {
@@ -449,12 +463,35 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
   info.probes = probes;
   MXOPT_DEBUG("hbm pool: %zu MiB arena of %zu MiB chunks over %d region(s); probe %.0f GB/s inside one region, %.0f across; %.2f s",
               pool->capacity >> 20, chunk_bytes >> 20, nregions, same_gbps, cross_gbps, info.setup_seconds);
+  {
+    std::lock_guard<std::mutex> all(g_pools_mu);
+    g_pools.push_back(pool);
+  }
   *out = pool;
   return MXOPT_OK;
 }
 
-void mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool) {
-  if (!pool) return;
+int mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool) {
+  if (!pool) return MXOPT_OK;
+  {
+    // Unmapping memory that someone still uses would make their next kernel fault: refuse instead.
+    std::lock_guard<std::mutex> all(g_pools_mu);
+    size_t live = 0, bytes = 0;
+    {
+      std::lock_guard<std::mutex> lock(pool->mu);
+      live = pool->live.size();
+      for (auto& kv : pool->live) bytes += kv.second;
+    }
+    if (live)
+      return fail(pool->ctx, MXOPT_ERR_INVALID_ARG,
+                  "mxopt_hbm_pool_destroy: " + std::to_string(live) + " allocation(s), " + std::to_string(bytes >> 20) +
+                      " MiB, are still live; free them (optimizer and engine objects, the host allocator's segments) first");
+    g_pools.erase(std::remove(g_pools.begin(), g_pools.end(), pool), g_pools.end());
+  }
+  {
+    std::lock_guard<std::mutex> lock(g_hook_mu);
+    if (g_hook_pool == pool) g_hook_pool = nullptr;
+  }
   {
     DeviceGuard guard(pool->ctx->device);
     (void)hipStreamSynchronize(pool->ctx->stream);
@@ -466,6 +503,7 @@ void mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool) {
     if (pool->ctx->state_pool == pool) pool->ctx->state_pool = nullptr;
   }
   delete pool;
+  return MXOPT_OK;
 }
 
 // First fit; NULL when no free range is large enough.
@@ -541,9 +579,6 @@ int mxopt_set_state_pool(mxopt_ctx* ctx, mxopt_hbm_pool* pool) {
 
 // ---- hooks with the signature host allocators plug in (torch's CUDAPluggableAllocator) ------------
 
-static std::mutex g_hook_mu;
-static mxopt_hbm_pool* g_hook_pool = nullptr;
-
 int mxopt_hbm_pool_set_hook_target(mxopt_hbm_pool* pool) {
   std::lock_guard<std::mutex> lock(g_hook_mu);
   g_hook_pool = pool;
@@ -569,12 +604,7 @@ void* mxopt_hbm_pool_hook_alloc(ptrdiff_t size, int device, void* stream) {
 
 void mxopt_hbm_pool_hook_free(void* ptr, ptrdiff_t size, int device, void* stream) {
   (void)size; (void)device; (void)stream;
-  mxopt_hbm_pool* pool;
-  {
-    std::lock_guard<std::mutex> lock(g_hook_mu);
-    pool = g_hook_pool;
-  }
-  if (pool && mxopt_hbm_pool_owns(pool, ptr)) { (void)mxopt_hbm_pool_free(pool, ptr); return; }
+  if (mxopt_hbm_pool* pool = pool_of(ptr)) { (void)mxopt_hbm_pool_free(pool, ptr); return; }
   (void)hipFree(ptr);
 }
 
@@ -591,8 +621,9 @@ hipError_t state_alloc(mxopt_ctx* ctx, void** out, size_t bytes) {
 }
 
 void state_free(mxopt_ctx* ctx, void* ptr) {
+  (void)ctx;
   if (!ptr) return;
-  if (ctx->state_pool && mxopt_hbm_pool_owns(ctx->state_pool, ptr)) { (void)mxopt_hbm_pool_free(ctx->state_pool, ptr); return; }
+  if (mxopt_hbm_pool* pool = pool_of(ptr)) { (void)mxopt_hbm_pool_free(pool, ptr); return; }
   (void)hipFree(ptr);
 }
 

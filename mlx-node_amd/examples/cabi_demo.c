@@ -304,7 +304,7 @@ static void pool_and_friends(void) {
   mxopt_engine_free(eng);
   CHECK_HIP(hipFree(w)); CHECK_HIP(hipFree(dgood)); CHECK_HIP(hipFree(dbad));
   CHECK_HIP(hipFree(dp)); CHECK_HIP(hipFree(dg));
-  mxopt_hbm_pool_destroy(pool);
+  CHECK_MX(mxopt_hbm_pool_destroy(pool));
 }
 
 /* Qwen3-0.6B: vocab 151936, hidden 1024, 28 layers, q 2048x1024, k/v 1024x1024, o 1024x2048,

@@ -106,7 +106,7 @@ SIGNATURES = {
     "mxopt_hbm_spread_begin": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
     "mxopt_hbm_spread_end": (C.c_int, [C.c_void_p]),
     "mxopt_hbm_pool_create": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
-    "mxopt_hbm_pool_destroy": (None, [C.c_void_p]),
+    "mxopt_hbm_pool_destroy": (C.c_int, [C.c_void_p]),
     "mxopt_hbm_pool_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
     "mxopt_hbm_pool_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "mxopt_hbm_pool_owns": (C.c_int, [C.c_void_p, C.c_void_p]),

@@ -334,9 +334,10 @@ class HbmPool:
         return torch.cuda.MemPool(HbmPool._torch_allocator.allocator())
 
     def close(self) -> None:
+        """Raises while anything allocated from the pool is alive (torch tensors and MemPools included)."""
         if self.handle:
-            self.ctx.lib.mxopt_hbm_pool_set_hook_target(None)
-            self.ctx.lib.mxopt_hbm_pool_destroy(self.handle)
+            torch.cuda.empty_cache()     # segments torch only caches go back through the free hook
+            L.check(self.ctx.lib.mxopt_hbm_pool_destroy(self.handle), self.ctx.handle)
             self.handle = C.c_void_p()
 
 

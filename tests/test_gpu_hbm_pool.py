@@ -68,6 +68,9 @@ def test_pool_limited_to_two_regions(mx, ctx, pool):
             assert sum(i.region_arena_bytes[2:]) == 0
         a = small.alloc(3 * GiB)
         assert small.owns(a) and not pool.owns(a)
+        with pytest.raises(mx.InvalidArg, match=r"1 allocation\(s\), 3072 MiB, are still live"):
+            small.close()                     # unmapping under a live allocation is refused
+        assert small.owns(a)
         small.free(a)
     finally:
         small.close()
@@ -144,8 +147,9 @@ def test_optimizer_state_comes_from_the_pool(mx, ctx, pool):
         assert pool.owns(m.value) and pool.owns(v.value) and cnt.value == n
         assert pool.info().used_bytes >= 2 * 4 * n
         assert_bit_equal(to_host(out), O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01).update_single("w", p, g), "AdamW, pooled state")
-        del opt
-        assert pool.info().used_bytes == 0    # the moments went back to the arena
+        ctx.lib.mxopt_set_state_pool(ctx.handle, None)
+        del opt                               # detached meanwhile: the moments still find their way back
+        assert pool.info().used_bytes == 0
     finally:
         ctx.lib.mxopt_set_state_pool(ctx.handle, None)
     opt = mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, ctx=ctx)   # detached again: state from the driver
