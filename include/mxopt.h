@@ -116,7 +116,7 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * either way).  Allocations are 512-byte
  * aligned, first fit, thread-safe; contents are not cleared.  A pointer goes back to the pool it came
  * from whichever pool a context or the hooks point at by then.  Destroy the pool after everything that
- * allocated from it.  No counterpart in the reference (MLX owns its allocator there). */
+ * allocated from it and before its context.  No counterpart in the reference (MLX owns its allocator there). */
 #define MXOPT_HBM_MAX_REGIONS 8
 typedef struct mxopt_hbm_pool mxopt_hbm_pool;
 typedef struct mxopt_hbm_pool_info {
