@@ -72,6 +72,18 @@ struct SumsqChunk {
     return hidden_inf ? __builtin_nanf("") : s32;
   }
 
+  // MODE 2 when nobody asked for the norm: the new sum is stored and nothing is squared.  With 16-bit
+  // gradients the squares (widen, transform, multiply-add per element) cost more instruction issue than
+  // the pass has to spare beside its memory traffic.
+  __device__ __forceinline__ void finish_store_only(const ChunkView& cv, uint32_t tid, bool first) {
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
+      store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+    }
+  }
+
   // Partial or unaligned chunk.
   static __device__ __forceinline__ float slow(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
     const void* X = squared_stream(cv);
@@ -132,6 +144,20 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
   double acc_sum = 0.0;
 
   uint32_t c = blockIdx.x;
+  if (MODE == 2 && partial_sum == nullptr) {  // accumulation only
+    for (; c < nchunks; c += gridDim.x) {
+      const ChunkView cv = locate(T, C, one, c);
+      if (cv.fast) {
+        Chunk k;
+        k.load(cv, tid, first);
+        k.finish_store_only(cv, tid, first);
+      } else {
+        (void)Chunk::slow(cv, pr, tid, first);
+      }
+      if (tid < cv.head) (void)Chunk::one_element(cv, pr, tid, first, 0.0f);
+    }
+    return;
+  }
   for (; c < nchunks; c += gridDim.x) {
     const ChunkView cv = locate(T, C, one, c);
     float s;
