@@ -56,6 +56,25 @@ struct SumsqChunk {
   // Returns this lane's float32 sum of squares over the chunk; stores the new sum in MODE 2.
   __device__ __forceinline__ float finish(const ChunkView& cv, const PrepRegs& pr, uint32_t tid, bool first) {
     float s32 = 0.0f;
+    if ((pr.flags & (kPrepClampPre | kPrepPreMul)) == kPrepClampPre) {
+      // A clamp and nothing else before the norm (the GRPO engine's validity + norm pass).  The flags are
+      // tested once per chunk, not per element, and the raw values' validity costs one multiply-add each:
+      // x * 0 is NaN exactly when x is a NaN or an infinity, which the clamp would have hidden.
+      float poison = 0.0f;
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
+          if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
+          poison = fmaf(x[j][e], 0.0f, poison);
+          const float y = __builtin_amdgcn_fmed3f(x[j][e], pr.pre_lo, pr.pre_hi);
+          s32 = fmaf(y, y, s32);
+        }
+        if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+      }
+      return poison != poison ? __builtin_nanf("") : s32;
+    }
     const bool clamped = (pr.flags & kPrepClampPre) != 0;
     bool hidden_inf = false;
 #pragma unroll
