@@ -71,7 +71,8 @@ const char* mxopt_last_error(const mxopt_ctx* ctx);
  * crates/mlx-sys/src/mlx.cpp:189-209). */
 int mxopt_synchronize(mxopt_ctx* ctx);
 /* Tuning knobs, by name: "grid_blocks_per_cu" (persistent grid = CUs x this),
- * "persistent" (0: one workgroup per chunk for the update kernels), "nontemporal" /
+ * "persistent" (0: one workgroup per chunk for the update kernels), "persistent_accumulate" (1: the
+ * persistent grid also for accumulation passes after the first that take no norm), "nontemporal" /
  * "nontemporal_reduce" (streaming-hint memory instructions in the read-write / read-only kernels). */
 int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value);
 int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);

@@ -200,10 +200,10 @@ static int run_sumsq(mxopt_ctx* ctx, const mxopt_table* t, int mode, int first, 
   }
   size_t offset = 0;
   for (const Group& g : t->groups) {
-    // Reductions need one partial per workgroup, so they keep a bounded grid; so does the
-    // read-modify-write accumulation, which measured faster that way.  Only the first,
-    // write-dominated accumulation pass follows the update kernels' launch policy.
-    Launch L = make_launch(ctx, t, g, want || !(mode == 2 && first) || ctx->persistent != 0);
+    // Reductions need one partial per workgroup, so they keep a bounded grid.  Accumulation passes that
+    // take no norm follow the update kernels' launch policy (one workgroup per chunk: 6.12 against
+    // 6.04 TB/s for acc += g on region-interleaved memory).
+    Launch L = make_launch(ctx, t, g, want || mode != 2 || ctx->persistent != 0 || (ctx->persistent_accumulate != 0 && !first));
     if (mode != 2) L.nontemporal = ctx->nontemporal_reduce;
     const int ad = mode == 0 ? g.gd : g.god;
     MXOPT_DEBUG("%s (reduction mode %d%s): %s, %u chunks in %u workgroups", op, mode, first ? ", first" : "",
@@ -344,6 +344,8 @@ int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
     ctx->nontemporal = value != 0;
   } else if (n == "nontemporal_reduce") {
     ctx->nontemporal_reduce = value != 0;
+  } else if (n == "persistent_accumulate") {
+    ctx->persistent_accumulate = value != 0;
   } else {
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: unknown option " + n);
   }
@@ -357,6 +359,7 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
   else if (n == "persistent") *value = ctx->persistent;
   else if (n == "nontemporal") *value = ctx->nontemporal;
   else if (n == "nontemporal_reduce") *value = ctx->nontemporal_reduce;
+  else if (n == "persistent_accumulate") *value = ctx->persistent_accumulate;
   else if (n == "num_cus") *value = ctx->num_cus;
   else return MXOPT_ERR_INVALID_ARG;
   return MXOPT_OK;

@@ -78,6 +78,7 @@ struct mxopt_ctx {
   int persistent = 0;           // update kernels: 0 = one workgroup per chunk, 1 = bounded grid
   int nontemporal = 0;          // streaming-hint loads/stores in update, transform, accumulate kernels
   int nontemporal_reduce = 1;   // streaming-hint loads in the read-only reduction kernels
+  int persistent_accumulate = 0;  // bounded grid also for accumulation passes that take no norm
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
   size_t partial_cap = 0;
   double* d_static_partials = nullptr;        // this device's copy of the library's fixed partial-sum array
