@@ -174,8 +174,8 @@ def test_config1_bias_corrected_per_call_step_count(oracle_c):
 def test_config2_full_size_every_element(oracle_c, tails):
     """Inputs come from the library's counter-based generator on the device and are regenerated on the
     host by the oracle's twin of it: nothing is copied to the device, every one of 1.72 G elements of
-    p, m and v is compared after each of two steps.  Once with the four-uniform bell (|x| <= 3.46 sigma),
-    once with the Gaussian mode, whose tails reach 6 sigma before the x100 outliers multiply them."""
+    p, m and v is compared after each step.  One step with the four-uniform bell (|x| <= 3.46 sigma), two
+    with the Gaussian mode, whose tails reach 6 sigma before the x100 outliers multiply them."""
     import torch
     import mxopt as mx
     _, sizes = qwen_sizes("1.7B")
@@ -205,7 +205,7 @@ def test_config2_full_size_every_element(oracle_c, tails):
     # a second host trajectory that never sees a device value: the oracle with its OWN clip factor, from the
     # exact float64 sum (optimizers/mod.rs:87-102 -> adamw.rs:84-116)
     own_p, own_m, own_v = p_ref.copy(), np.zeros(n, F), np.zeros(n, F)
-    for step in range(2):
+    for step in range(2 if tails == "gaussian" else 1):
         for i in range(nt):                     # fresh gradients each step: 1 % of the elements x100
             key = mx.synthetic_key(SEED, CFG, step + 1, 1, i)
             ctx.fill_synthetic(dg[i], key, SPIKED, 1e-3, 100.0)
