@@ -45,6 +45,8 @@ TRAFFIC_KERNEL_SOURCES = ["mxopt_kernels.hip", "mxopt_kernels_common.h", "mxopt_
 MEASURED_TRAFFIC_B_PER_ELEM = {("cfg5", 1): 25.91, ("cfg5-deferred", 1): 27.89}
 PROBE_PROFILE = "profiles/probe_streams_pool_and_plain.txt"
 OTHER_CONFIGS = ["cfg1", "cfg2", "cfg3-sgd", "cfg3-rmsprop", "cfg4", "cfg4-flat"]
+# steps each configuration states for itself
+OTHER_CONFIG_STEPS = {"cfg1": 10, "cfg2": 20, "cfg3-sgd": 20, "cfg3-rmsprop": 20, "cfg4": 100, "cfg4-flat": 100}
 
 
 def traffic_profile_is_current():
@@ -78,16 +80,32 @@ def parse_args():
     ap.add_argument("--alloc", default="tensor", choices=["tensor", "slab", "packed"],
                     help="tensor: one device allocation per tensor and stream; slab: one allocation per stream, "
                          "tensors are 512-byte aligned views into it")
-    ap.add_argument("--placement", default="pool", choices=["pool", "spread", "plain"],
-                    help="pool: every buffer comes from a region-interleaved arena (mxopt_hbm_pool_create); spread: the "
-                         "buffers are allocated inside mxopt_hbm_spread_begin/end (their physical pages interleaved with "
-                         "released memory, a matter of luck); plain: wherever the driver puts them")
+    ap.add_argument("--placement", default="pool", choices=["pool", "state-pool", "spread", "plain"],
+                    help="pool: every buffer comes from a region-interleaved arena (mxopt_hbm_pool_create); state-pool: "
+                         "only what the library itself would own (moments, accumulation buffers) comes from the arena, "
+                         "parameters and gradients lie wherever the host's allocator (here torch's) put them -- what a "
+                         "drop-in host sees after mxopt_set_state_pool; spread: the buffers are allocated inside "
+                         "mxopt_hbm_spread_begin/end (their physical pages interleaved with released memory, a matter of "
+                         "luck); plain: wherever the driver puts them")
+    ap.add_argument("--placements", type=int, default=-1,
+                    help="1: the default workload is also measured with --placement plain (in a child process started "
+                         "before this one touches the GPU: the first allocations of a fresh process) and with "
+                         "--placement state-pool, and config.placement carries the three AdamW rates; default: only "
+                         "for cfg5 at full scale on the arena")
+    ap.add_argument("--verify", type=int, default=-1,
+                    help="1: after the timed steps, seeded windows of parameters and moments are recomputed on the host "
+                         "by the C twin of the oracle for exactly the steps that ran and compared bit for bit "
+                         "(`verified` in the line); default: cfg5 only")
     ap.add_argument("--pool-regions", type=int, default=2, help="--placement pool: regions to alternate between (0 = all found)")
     ap.add_argument("--pool-chunk-mb", type=int, default=0, help="--placement pool: chunk size (0 = the library's 64)")
     ap.add_argument("--others", type=int, default=-1,
                     help="1: after the main workload, run BASELINE's configs 1-4 for a few steps each and report them as "
                          "other_configs; default: only when the workload is cfg5 at full scale")
-    ap.add_argument("--others-steps", type=int, default=5)
+    ap.add_argument("--others-steps", type=int, default=0,
+                    help="timed steps of each of the other configurations (0 = what the configuration states: 10, 20, 20, 100)")
+    ap.add_argument("--ceiling", type=int, default=1, help="0: skip the bare probes (roofline.measured_ceiling)")
+    ap.add_argument("--variants", type=int, default=1,
+                    help="cfg5: 0 = skip the same step done the other ways (deferred accumulation, the other --fold-last)")
     ap.add_argument("--spread-block-mb", type=int, default=0, help="--placement spread: block size (0 = the library's 64)")
     ap.add_argument("--spread-keep", type=int, default=0, help="--placement spread: every n-th block is kept (0 = 3)")
     ap.add_argument("--micro", type=int, default=4,
@@ -139,10 +157,12 @@ class Workload:
         self.n = int(sum(self.sizes))
         self.kernel_events = {}     # kernel name -> list of (start, end) events
         self.res = self.ctx.norm_result()
-        if pool is not None:
-            self.mem_pool = pool.torch_pool()     # torch allocates this workload's buffers from the arena
-            window = torch.cuda.use_mem_pool(self.mem_pool)
-        elif args.placement == "spread":
+        self.mem_pool = pool.torch_pool() if pool is not None else None   # torch allocates from the arena through it
+        # state-pool: only moments and accumulation buffers (what the library's own objects allocate through
+        # mxopt_set_state_pool) come from the arena; parameters and gradients are the host's and lie in plain memory
+        self.arena_kinds = (() if pool is None else ("state",) if args.placement == "state-pool"
+                            else ("param", "grad", "state"))
+        if args.placement == "spread":
             window = self.ctx.hbm_spread(args.spread_block_mb << 20, args.spread_keep)
         else:
             window = contextlib.nullcontext()
@@ -150,9 +170,15 @@ class Workload:
             getattr(self, "_setup_" + args.workload.replace("-", "_"))()
             torch.cuda.synchronize()
 
-    def free_bytes(self):
-        """Device memory this workload may still take."""
-        if self.pool is not None:
+    def _window(self, kind):
+        """Where buffers of this kind ("param", "grad", "state") are allocated."""
+        if kind in self.arena_kinds:
+            return self.torch.cuda.use_mem_pool(self.mem_pool)
+        return contextlib.nullcontext()
+
+    def free_bytes(self, kind="state"):
+        """Device memory this workload may still take for buffers of that kind."""
+        if kind in self.arena_kinds:
             i = self.pool.info()
             return i.capacity_bytes - i.used_bytes
         return self.torch.cuda.mem_get_info()[0]
@@ -180,33 +206,35 @@ class Workload:
         for i, v in enumerate(views):
             self.ctx.fill_synthetic(v, self.mx.synthetic_key(self.SEED, cfg, 0, stream_id, i), dist, a, b)
 
-    def _zeros(self, n):
-        return self.torch.zeros(n, dtype=self.torch.float32, device="cuda")
-
     # one list of tensors per stream, either separately allocated or carved out of one slab
-    def _carve(self, dtype):
+    def _carve(self, dtype, kind):
         t = self.torch
         mode = getattr(self.args, "alloc", "tensor")
-        if mode == "tensor":
-            return None, [t.empty(n, dtype=dtype, device="cuda") for n in self.sizes]
-        offs, total = [], 0
-        for n in self.sizes:
-            offs.append(total)
-            # slab: 512 B (bf16) / 1 KiB (f32) alignment; packed: back to back, natural alignment only
-            total += (n + 255) // 256 * 256 if mode == "slab" else n
-        slab = t.empty(max(total, 1), dtype=dtype, device="cuda")
-        return slab, [slab[o:o + n] for o, n in zip(offs, self.sizes)]
+        with self._window(kind):
+            if mode == "tensor":
+                return None, [t.empty(n, dtype=dtype, device="cuda") for n in self.sizes]
+            offs, total = [], 0
+            for n in self.sizes:
+                offs.append(total)
+                # slab: 512 B (bf16) / 1 KiB (f32) alignment; packed: back to back, natural alignment only
+                total += (n + 255) // 256 * 256 if mode == "slab" else n
+            slab = t.empty(max(total, 1), dtype=dtype, device="cuda")
+            return slab, [slab[o:o + n] for o, n in zip(offs, self.sizes)]
 
-    def _randn_list(self, dtype, std, outliers=False):
+    def _randn_list(self, dtype, std, outliers=False, kind="grad"):
         """A list of tensors with bell-shaped values of standard deviation `std` (optionally 1 % x100)."""
-        _, views = self._carve(dtype)
+        _, views = self._carve(dtype, kind)
         self._next_stream = getattr(self, "_next_stream", 0) + 1
         mx = self.mx
-        self._fill(views, self._next_stream, mx.SYNTH_GAUSSIAN_OUTLIERS if outliers else mx.SYNTH_GAUSSIAN, std, 100.0)
+        dist = mx.SYNTH_GAUSSIAN_OUTLIERS if outliers else mx.SYNTH_GAUSSIAN
+        self._fill(views, self._next_stream, dist, std, 100.0)
+        # what a host program needs to regenerate any slice of this stream: (stream id, distribution, a, b)
+        self.stream_specs = getattr(self, "stream_specs", {})
+        self.stream_specs[self._next_stream] = (dist, std, 100.0)
         return views
 
-    def _zeros_list(self):
-        slab, views = self._carve(self.torch.float32)
+    def _zeros_list(self, kind="state"):
+        slab, views = self._carve(self.torch.float32, kind)
         if slab is not None:
             slab.zero_()
         else:
@@ -214,8 +242,8 @@ class Workload:
                 v.zero_()
         return views
 
-    def _empty_list(self, dtype):
-        return self._carve(dtype)[1]
+    def _empty_list(self, dtype, kind="state"):
+        return self._carve(dtype, kind)[1]
 
     def _timed(self, name, fn):
         s = self.torch.cuda.Event(enable_timing=True)
@@ -233,11 +261,12 @@ class Workload:
     def _setup_cfg5(self):
         t, mx = self.torch, self.mx
         bf = t.bfloat16
-        need = self.n * (2 + 8 + 4)
-        free = self.free_bytes()
         self.n_micro = 4
-        n_gbuf = 4 if free > need + 4 * self.n * 2 + (3 << 30) else 1
-        self.p = self._randn_list(bf, 0.02)
+        if "grad" in self.arena_kinds or not self.arena_kinds:    # everything from one place
+            n_gbuf = 4 if self.free_bytes("grad") > self.n * (2 + 8 + 4) + 4 * self.n * 2 + (3 << 30) else 1
+        else:                                                     # parameters and gradients in plain memory
+            n_gbuf = 4 if self.free_bytes("grad") > self.n * 2 + 4 * self.n * 2 + (3 << 30) else 1
+        self.p = self._randn_list(bf, 0.02, kind="param")
         self.m = self._zeros_list()
         self.v = self._zeros_list()
         self.acc = self._empty_list(t.float32)
@@ -250,12 +279,13 @@ class Workload:
         self.dtype = "f32"
         self.storage = "bf16 parameters and gradients, float32 accumulation buffer and moments"
         self.fold_last = bool(self.args.fold_last)
+        # folded: the update reads the accumulation buffer AND the last micro-batch (24 + 2 B/elem); the last
+        # accumulation pass only measures the norm (6 B/elem): 6 + 10 + 10 + 6 + 26 = 58 B/elem/step.
+        # unfolded: four plain accumulation passes, 6 + 3 * 10 + 24 = 60 B/elem/step
+        last = self.g[(self.n_micro - 1) % n_gbuf]
+        self.t_upd_pending = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=gl, m=m, v=v)
+                                             for p, a, gl, m, v in zip(self.p, self.acc, last, self.m, self.v)])
         if self.fold_last:
-            # the update reads the accumulation buffer AND the last micro-batch (24 + 2 B/elem); the last
-            # accumulation pass only measures the norm (6 B/elem): 6 + 10 + 10 + 6 + 26 = 58 B/elem/step
-            last = self.g[(self.n_micro - 1) % n_gbuf]
-            self.t_upd_pending = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=a, g_out=gl, m=m, v=v)
-                                                 for p, a, gl, m, v in zip(self.p, self.acc, last, self.m, self.v)])
             self.bytes_per_elem = {"accumulate_first": 6, "accumulate": 10, "accumulate_norm_only": 6, "adamw": 26}
             self.step_bytes_per_elem = 6 + 10 * 2 + 6 + 26
         else:
@@ -285,26 +315,48 @@ class Workload:
             one()
         t.cuda.synchronize()
         dt = (time.perf_counter() - t0) / steps
+        self.deferred_steps_done = steps + 1
         return {"value": round(1.0 / dt, 4), "unit": "steps/s", "ms_per_step": round(dt * 1e3, 4),
                 "bytes_per_elem_per_step": 36, "step_hbm_gbps": round(36 * self.n / dt / 1e9, 1),
                 "note": "same buffers and result; the four resident micro-batches are added in registers by the norm "
                         "pass (8 B/elem) and by AdamW (28 B/elem) instead of being accumulated into the float32 buffer"}
 
-    def _step_cfg5(self):
+    def _step_cfg5(self, fold_last=None):
         c = self.ctx
+        fold_last = self.fold_last if fold_last is None else fold_last
         for k in range(self.n_micro):
             tab = self.t_acc[k % len(self.t_acc)]
             last = k == self.n_micro - 1
-            if last and self.fold_last:
+            if last and fold_last:
                 self._timed("accumulate_norm_only", lambda: c.accumulate_norm_only(tab, self.res, max_norm=1.0))
                 continue
             name = "accumulate_first" if k == 0 else ("accumulate_sumsq" if last else "accumulate")
             self._timed(name, lambda: c.accumulate(tab, first=(k == 0), out=self.res if last else None,
                                                    max_norm=1.0))
-        if self.fold_last:
+        if fold_last:
             self._timed("adamw", lambda: c.adam_with_pending(self.t_upd_pending, self.hp, self.prep))
         else:
             self._timed("adamw", lambda: c.adam(self.t_upd, self.hp, self.prep))
+
+    def other_fold_variant(self, steps):
+        """Config 5 on the same buffers with the other --fold-last setting (same result, 60 instead of 58 B/elem
+        or the reverse)."""
+        t = self.torch
+        fold = not self.fold_last
+        bpe = 58 if fold else 60
+        self._step_cfg5(fold)
+        t.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self._step_cfg5(fold)
+        t.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        self.other_fold_steps_done = steps + 1
+        return {"fold_last": int(fold), "value": round(1.0 / dt, 4), "unit": "steps/s", "ms_per_step": round(dt * 1e3, 4),
+                "bytes_per_elem_per_step": bpe, "step_hbm_gbps": round(bpe * self.n / dt / 1e9, 1),
+                "note": ("four plain accumulation passes (6 + 3 x 10 B/elem), the last carrying the sum of squares, and "
+                         "AdamW from the buffer alone (24 B/elem): the step as counted at 60 B/elem") if not fold else
+                        "the last micro-batch only measured (6 B/elem) and added again inside AdamW (26 B/elem)"}
 
     # -- cfg5 without its accumulation buffer: the four micro-batches stay resident and are summed in
     #    registers, in arrival order, by the norm pass (8 B/elem) and by the update (18 + 10 B/elem)
@@ -312,7 +364,7 @@ class Workload:
         t, mx = self.torch, self.mx
         bf = t.bfloat16
         self.n_micro = self.args.micro
-        self.p = self._randn_list(bf, 0.02)
+        self.p = self._randn_list(bf, 0.02, kind="param")
         self.m = self._zeros_list()
         self.v = self._zeros_list()
         self.g = [self._randn_list(bf, 1e-3) for _ in range(self.n_micro)]
@@ -337,7 +389,7 @@ class Workload:
     # -- cfg1: fp32 AdamW
     def _setup_cfg1(self):
         t, mx = self.torch, self.mx
-        self.p = self._randn_list(t.float32, 0.02)
+        self.p = self._randn_list(t.float32, 0.02, kind="param")
         self.g = self._randn_list(t.float32, 1e-3)
         self.m = self._zeros_list()
         self.v = self._zeros_list()
@@ -379,10 +431,10 @@ class Workload:
         t, mx = self.torch, self.mx
         bf = t.bfloat16
         if uniform_p:
-            self.p = self._carve(bf)[1]
+            self.p = self._carve(bf, "param")[1]
             self._fill(self.p, 100, mx.SYNTH_UNIFORM, 0.9, 1.1)
         else:
-            self.p = self._randn_list(bf, 0.02)
+            self.p = self._randn_list(bf, 0.02, kind="param")
         self.g = self._randn_list(bf, gstd, outliers=self.args.workload == "cfg2")   # cfg2: 1 % of the elements x100
         self.m = self._zeros_list()
         self.v = self._zeros_list()
@@ -404,6 +456,45 @@ class Workload:
 
     def _setup_cfg4(self):
         self._setup_cfg2(lr=1e-3, wd=0.0, gstd=1e-2, uniform_p=True)
+        self.graph_variant = self._graph_variant   # config 4 exists to show launch overhead: also timed from a HIP graph
+
+    def _graph_variant(self, steps):
+        """The same step (norm pass, its one-workgroup second pass, AdamW) on a side stream, eager and replayed
+        from a HIP graph: three launches whose gaps are a measurable part of a 0.4 ms step."""
+        t, mx = self.torch, self.mx
+        s = t.cuda.Stream()
+        ctx = mx.Context(stream=s)
+        res = ctx.norm_result()
+        t_g = ctx.table([mx.TensorSpec(g=g) for g in self.g])
+        t_upd = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v)
+                           for p, g, m, v in zip(self.p, self.g, self.m, self.v)])
+        prep = mx.make_prep(scale=res)
+
+        def one():
+            ctx.global_norm(t_g, res, max_norm=1.0)
+            ctx.adam(t_upd, self.hp, prep)
+        t.cuda.synchronize()
+        with t.cuda.stream(s):
+            one()                                   # warm-up: the partial-sum buffer exists before the capture
+            s.synchronize()
+            graph = t.cuda.CUDAGraph()
+            with t.cuda.graph(graph, stream=s):
+                one()
+            out = {}
+            for name, fn in (("eager_ms_per_step", one), ("graph_ms_per_step", graph.replay)):
+                for _ in range(3):
+                    fn()
+                s.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                s.synchronize()
+                out[name] = round((time.perf_counter() - t0) * 1e3 / steps, 4)
+        out["graph_step_hbm_gbps"] = round(self.step_bytes_per_elem * self.n / (out["graph_ms_per_step"] * 1e-3) / 1e9, 1)
+        out["what"] = "mxopt_global_norm + mxopt_adam captured once on a side stream and replayed; same buffers"
+        del graph
+        t_g.close(); t_upd.close(); ctx.close()
+        return out
 
     _step_cfg4 = _step_cfg2
     _setup_cfg4_flat = _setup_cfg4
@@ -412,7 +503,7 @@ class Workload:
     # -- cfg3: fp32 SGD / RMSprop
     def _setup_cfg3(self):
         t, mx = self.torch, self.mx
-        self.p = self._randn_list(t.float32, 0.02)
+        self.p = self._randn_list(t.float32, 0.02, kind="param")
         self.g = self._randn_list(t.float32, 1e-3)
         self.v = self._zeros_list()
         self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v)
@@ -446,7 +537,7 @@ class Workload:
         t, mx = self.torch, self.mx
         bf = t.bfloat16
         self.names = [name for name, _ in param_list(QWEN3["8B"])]
-        self.p = self._randn_list(bf, 0.02)
+        self.p = self._randn_list(bf, 0.02, kind="param")
         self.g = self._randn_list(bf, 1e-3)
         params = dict(zip(self.names, self.p))
         self.n_micro = N = self.args.micro
@@ -519,7 +610,8 @@ class Workload:
     def _setup_copy(self):
         t, mx = self.torch, self.mx
         self.g = self._randn_list(t.float32, 1.0)
-        self.o = [t.empty_like(g) for g in self.g]
+        with self._window("grad"):
+            self.o = [t.empty_like(g) for g in self.g]
         self.t_copy = self.ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(self.g, self.o)])
         self.dtype = "f32"
         self.bytes_per_elem = {"copy": 8}
@@ -534,7 +626,8 @@ class Workload:
     #    ceilings of a read-only, a write-only, a copy and a 4-read/3-write pass on this memory
     def _setup_probes(self):
         t = self.torch
-        self.streams = [t.zeros(self.n, dtype=t.float32, device="cuda") for _ in range(4)]
+        with self._window("param"):
+            self.streams = [t.zeros(self.n, dtype=t.float32, device="cuda") for _ in range(4)]
         self.dtype = "u32"
         self.bytes_per_elem = {"probe_read": 4, "probe_write": 4, "probe_copy": 8, "probe_mix43": 28}
         self.step_bytes_per_elem = 44
@@ -550,6 +643,103 @@ class Workload:
 
     def step(self):
         getattr(self, "_step_" + self.args.workload.replace("-", "_"))()
+        self.steps_done = getattr(self, "steps_done", 0) + 1
+
+
+# ----------------------------------------------------------------------------------------
+# Self-check of the timed configuration (outside the timed region; the oracle is the checker only)
+# ----------------------------------------------------------------------------------------
+
+def verify_cfg5(wl, segments, window=256 * 1024, n_large=12):
+    """Recomputes, on the host, seeded windows of config 5's parameters and moments for exactly the optimizer
+    steps that ran on the device, and compares them bit for bit with what the device holds now.
+
+    The inputs are regenerated from the generator's host twin (no device value is read for them), pushed through
+    the C twin of the oracle -- four float32 accumulations in arrival order, AdamW on the clipped sum, bf16
+    write-back -- once per step.  `segments` is [(steps, clip factor)]: the factor is the device's own (checked
+    here against the reference's float32 scalar chain on the device's sum of squares, and the norm against a
+    float64 reduction by torch over the device buffers at rel 1e-5).  Windows: every tensor of at most 64 Ki
+    elements in full, and head, tail and an odd interior offset of `n_large` large tensors spread over the list
+    (the largest among them)."""
+    import math
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import mxopt_oracle as O
+    import oracle_c_binding as B
+    torch, mx = wl.torch, wl.mx
+    oc = B.load()
+    t0 = time.perf_counter()
+    sizes, cfg = wl.sizes, wl.CONFIG_ID[wl.args.workload]
+    n_gbuf = len(wl.g)
+
+    def host(stream, i, dtype, off, length):
+        dist, a, b = wl.stream_specs[stream]
+        return oc.fill_synthetic(length, dtype, mx.synthetic_key(wl.SEED, cfg, 0, stream, i), dist, a, b, first_index=off)
+
+    def bits(t):
+        t = t.cpu().contiguous()
+        return (t.view(torch.int16).numpy().view(np.uint16) if t.dtype == torch.bfloat16
+                else t.numpy().view(np.uint32))
+
+    large = [i for i, n in enumerate(sizes) if n > 65536]
+    picked = sorted(set([large[(len(large) - 1) * k // (n_large - 1)] for k in range(n_large)] +
+                        [max(range(len(sizes)), key=lambda i: sizes[i])]))
+    windows = [(i, 0, n) for i, n in enumerate(sizes) if 0 < n <= 65536]
+    for i in picked:
+        n, w = sizes[i], min(window, sizes[i])
+        mid = (n // 2) | 1                       # an odd element offset: not 16-byte aligned in any stream
+        for off in sorted({0, min(mid, n - w), n - w}):
+            windows.append((i, off, w))
+
+    # the norm the device took, against an independent float64 reduction of the same device buffers
+    total_t = torch.zeros((), dtype=torch.float64, device="cuda")
+    piece = 1 << 26
+    for i, n in enumerate(sizes):
+        for s in range(0, n, piece):
+            e = min(n, s + piece)
+            x = wl.g[0][i][s:e].float()
+            for k in range(1, wl.n_micro):
+                x += wl.g[k % n_gbuf][i][s:e].float()
+            total_t += x.double().square_().sum()
+    total = float(total_t)
+    norm_rel = 0.0
+    factor_ok = True
+    for _, scale, sumsq in segments:
+        norm_rel = max(norm_rel, abs(math.sqrt(sumsq) - math.sqrt(total)) / math.sqrt(total))
+        _, want = O.norm_scale_c1(sumsq, 1.0)
+        factor_ok = factor_ok and np.float32(scale) == want
+
+    elements = mismatches = 0
+    first_bad = None
+    for i, off, w in windows:
+        p = host(1, i, "bf16", off, w)
+        gs = [host(2 + (k % n_gbuf), i, "bf16", off, w) for k in range(wl.n_micro)]
+        m, v = np.zeros(w, np.float32), np.zeros(w, np.float32)
+        acc = np.empty(w, np.float32)
+        for k, g in enumerate(gs):
+            oc.accumulate_f32(acc, g, k == 0)
+        for steps, scale, _ in segments:
+            args = B.adam_args(5e-6, 0.9, 0.999, 1e-8, 0.01, scale=float(scale))
+            for _ in range(steps):
+                p = oc.f32_to_bf16(oc.adam(p, acc, m, v, args, fused=True))
+        for name, want, got in (("p", p, bits(wl.p[i][off:off + w])), ("m", m.view(np.uint32), bits(wl.m[i][off:off + w])),
+                                ("v", v.view(np.uint32), bits(wl.v[i][off:off + w]))):
+            bad = int(np.count_nonzero(want.view(got.dtype) != got))
+            mismatches += bad
+            if bad and first_bad is None:
+                first_bad = f"{name} of tensor {i} at offset {off}"
+        elements += 3 * w
+    ok = mismatches == 0 and factor_ok and norm_rel <= 1e-5
+    out = {"windows": len(windows), "elements": elements, "bit_exact": mismatches == 0,
+           "optimizer_steps_checked": sum(s for s, _, _ in segments),
+           "clip_factor_is_reference_chain_on_device_sum": bool(factor_ok),
+           "norm_rel_err_vs_torch_float64": float(f"{norm_rel:.3g}"), "ok": bool(ok),
+           "seconds": round(time.perf_counter() - t0, 2),
+           "what": "p, m, v windows recomputed by the C twin of the oracle from regenerated inputs for every step "
+                   "this process ran (warm-up, timed, and the deferred variant's), compared bit for bit"}
+    if first_bad:
+        out["first_mismatch"] = first_bad
+    return out
 
 
 # ----------------------------------------------------------------------------------------
@@ -560,13 +750,28 @@ def cpu_baseline(args, n_total):
     import numpy as np
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle_c_binding as B
+    import mxopt
     oc = B.load()
     S = int(min(args.cpu_sample, n_total))
-    rng = np.random.default_rng(1)
     w = args.workload
     f32 = np.float32
-    p32 = (rng.standard_normal(S, dtype=f32) * f32(0.02))
-    g32 = (rng.standard_normal(S, dtype=f32) * f32(1e-3))
+    cfg = Workload.CONFIG_ID[w]
+    GAUSS, GAUSS_OUT, UNIFORM = mxopt.SYNTH_GAUSSIAN, mxopt.SYNTH_GAUSSIAN_OUTLIERS, mxopt.SYNTH_UNIFORM
+
+    def gen(stream, dtype, dist, a, b=100.0):
+        """The first S elements of stream `stream` as the device workload holds them, tensor after tensor
+        (the library generator's host twin; same keys as Workload._fill)."""
+        sizes, _ = tensor_sizes(args)
+        out = np.empty(S, np.uint16 if dtype == "bf16" else f32)
+        pos = 0
+        for i, n in enumerate(sizes):
+            if pos >= S:
+                break
+            take = min(n, S - pos)
+            out[pos:pos + take] = oc.fill_synthetic(take, dtype, mxopt.synthetic_key(Workload.SEED, cfg, 0, stream, i), dist, a, b)
+            pos += take
+        return out
+
     m, v = np.zeros(S, f32), np.zeros(S, f32)
 
     def timeit(fn, reps=2):
@@ -579,16 +784,22 @@ def cpu_baseline(args, n_total):
 
     fused_s = None
     if w in ("cfg5", "cfg5-deferred", "cfg2", "cfg4", "cfg4-flat"):
-        p, g = oc.f32_to_bf16(p32), oc.f32_to_bf16(g32)
-        del p32, g32
+        five = w in ("cfg5", "cfg5-deferred")
+        if w in ("cfg4", "cfg4-flat"):
+            p = gen(100, "bf16", UNIFORM, 0.9, 1.1)
+            gs = [gen(1, "bf16", GAUSS, 1e-2)]
+        else:
+            p = gen(1, "bf16", GAUSS, 0.02)
+            gs = ([gen(2 + k, "bf16", GAUSS, 1e-3) for k in range(4)] if five
+                  else [gen(2, "bf16", GAUSS_OUT, 1e-3)])
         acc = np.empty(S, f32)
-        lr, wd = (5e-6, 0.01) if w != "cfg4" else (1e-3, 0.0)
+        lr, wd = (5e-6, 0.01) if w not in ("cfg4", "cfg4-flat") else (1e-3, 0.0)
 
         def step(fused):
-            src = g
-            if w in ("cfg5", "cfg5-deferred"):
+            src = gs[0]
+            if five:
                 for k in range(4):
-                    oc.accumulate_f32(acc, g, k == 0)
+                    oc.accumulate_f32(acc, gs[k], k == 0)
                 src = acc
             sumsq = oc.sumsq(src)
             scale = float(min(np.float32(1.0) / (np.float32(np.sqrt(sumsq)) + np.float32(1e-6)), np.float32(1.0)))
@@ -596,15 +807,17 @@ def cpu_baseline(args, n_total):
             out = oc.adam(p, src, m, v, a, fused=fused)
             oc.f32_to_bf16(out)     # parameters are kept in bf16
         what = ("4x accumulate + sumsq + scale + AdamW as 13 separate float32 passes (adamw.rs:84-116) + bf16 cast"
-                if w in ("cfg5", "cfg5-deferred") else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
+                if five else "sumsq + scale + AdamW as 13 separate float32 passes + bf16 cast")
         t_unfused = timeit(lambda: step(False))
         fused_s = timeit(lambda: step(True))
     elif w.startswith("cfg1"):
+        p32, g32 = gen(1, "f32", GAUSS, 0.02), gen(2, "f32", GAUSS, 1e-3)
         a = B.adam_args(1e-3, 0.9, 0.999, 1e-8, 0.01)
         t_unfused = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=False))
         fused_s = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=True))
         what = "AdamW as 13 separate float32 passes (adamw.rs:84-116)"
     elif w == "cfg3-sgd":
+        p32, g32 = gen(1, "f32", GAUSS, 0.02), gen(2, "f32", GAUSS, 1e-3)
         fl = lambda x: float(np.float32(x))
         a = B.SgdArgs(lr=fl(1e-4), momentum=fl(0.9), one_minus_damp=1.0, wd=fl(1e-4), has_wd=1, has_momentum=1,
                       nesterov=0, first=0)
@@ -612,6 +825,7 @@ def cpu_baseline(args, n_total):
         fused_s = timeit(lambda: oc.sgd(p32, g32, v, a, fused=True))
         what = "SGD+momentum+L2 as 7 separate float32 passes (sgd.rs:86-140)"
     else:
+        p32, g32 = gen(1, "f32", GAUSS, 0.02), gen(2, "f32", GAUSS, 1e-3)
         fl = lambda x: float(np.float32(x))
         a = B.RmspropArgs(lr=fl(1e-4), alpha=fl(0.99), one_minus_alpha=fl(1.0 - 0.99), eps=fl(1e-8), wd=0.0, has_wd=0)
         t_unfused = timeit(lambda: oc.rmsprop(p32, g32, v, a, fused=False))
@@ -621,8 +835,9 @@ def cpu_baseline(args, n_total):
     scale_up = n_total / S
     return {
         "value": 1.0 / (t_unfused * scale_up), "unit": "steps/s", "cores": oc.num_threads(), "kind": "port",
-        "sample": f"{S} of {n_total} elements, one flat tensor, best of 2; {what}; scaled per element "
-                  f"to the full list (sample step {t_unfused * 1e3:.1f} ms)",
+        "sample": f"the first {S} of {n_total} elements of the workload's own streams (the library generator's host "
+                  f"twin regenerates what the device holds: same seed, keys and distributions), one flat tensor, best "
+                  f"of 2; {what}; scaled per element to the full list (sample step {t_unfused * 1e3:.1f} ms)",
         "fused_single_pass_value": (1.0 / (fused_s * scale_up)) if fused_s else None,
     }
 
@@ -711,10 +926,41 @@ def measured_ceiling(args, torch, mx, ctx, pool):
             "profile": PROBE_PROFILE}
 
 
+def child_leg(args, placement, steps=5, warmup=2):
+    """The same workload in a child process with another placement; returns what its line says about the step and
+    the dominant kernel.  Run before this process touches the GPU, the child's allocations are the first of a
+    fresh process: one compact physical run, which is what `plain` means on a freshly started host."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--workload", args.workload, "--placement", placement,
+           "--steps", str(steps), "--warmup", str(warmup), "--cpu-sample", "0", "--others", "0", "--placements", "0",
+           "--verify", "0", "--ceiling", "0", "--variants", "0", "--fold-last", str(args.fold_last),
+           "--scale", str(args.scale), "--alloc", args.alloc]
+    try:
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
+        d = json.loads(line)
+        k = d["kernels"][d["roofline"]["kernel"]]
+        return {"ms_per_step": d["ms_per_step"], "dominant_kernel_gbps": k["gbps"], "dominant_kernel_ms": k["avg_ms"],
+                "step_hbm_gbps": d["step_hbm_gbps"], "steps": steps}
+    except Exception as e:  # the leg is a side figure: its failure must not take the headline with it
+        return {"error": f"{type(e).__name__}: {e}"[:300]}
+
+
+def leg_summary(r, wl, steps):
+    d = r["kernels"][wl.dominant]
+    return {"ms_per_step": round(r["ms_per_step"], 4), "dominant_kernel_gbps": d["gbps"], "dominant_kernel_ms": d["avg_ms"],
+            "step_hbm_gbps": round(r["step_gbps"], 1), "steps": steps}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
+    full_default = args.workload == "cfg5" and args.scale == 1.0
+    three_placements = args.placement == "pool" and (args.placements == 1 or (args.placements == -1 and full_default))
+    # before anything here touches the GPU: the plain leg wants to be the first allocations of a fresh process
+    plain_leg = child_leg(args, "plain") if three_placements else None
+
     import torch
     import mxopt
 
@@ -728,11 +974,17 @@ def main():
         ctx.set_option(k, int(v))
     pool = None
     placement = "plain"
-    if args.placement == "pool":
-        # the arena takes the free memory but for a margin left to torch's own scratch and the runtime
+    sizes, _ = tensor_sizes(args)
+    if args.placement in ("pool", "state-pool"):
+        # the arena takes the free memory but for a margin left to torch's own scratch and the runtime -- and, when
+        # the state-pool leg follows (or is the placement asked for), for the parameters and gradients that leg
+        # keeps in plain memory
         free = torch.cuda.mem_get_info()[0]
+        host_side = 0
+        if three_placements or args.placement == "state-pool":
+            host_side = sum(sizes) * 2 * 5 + (4 << 30) if args.workload == "cfg5" else free // 2
         try:
-            pool = ctx.hbm_pool(free - (8 << 30), args.pool_chunk_mb << 20, args.pool_regions)
+            pool = ctx.hbm_pool(free - (8 << 30) - host_side, args.pool_chunk_mb << 20, args.pool_regions)
         except mxopt.MxoptError as e:
             # e.g. another process holds most of the device: measure in plain memory and say so in the line
             print(f"bench.py: no region-interleaved arena ({e}); buffers come from plain device memory", file=sys.stderr)
@@ -740,7 +992,10 @@ def main():
     if pool is not None:
         pool.use_for_state()
         i = pool.info()
-        placement = {"kind": "mxopt_hbm_pool", "chunk_mib": i.chunk_bytes >> 20, "regions_found": i.regions,
+        placement = {"kind": "mxopt_hbm_pool" if args.placement == "pool" else
+                             "moments and accumulation buffers from mxopt_hbm_pool (mxopt_set_state_pool); parameters and "
+                             "gradients in plain device memory",
+                     "chunk_mib": i.chunk_bytes >> 20, "regions_found": i.regions,
                      "regions_used": min(args.pool_regions, i.regions) if args.pool_regions else i.regions,
                      "arena_gib": round(i.capacity_bytes / 2**30, 1),
                      "region_free_gib": [round(x / 2**30, 1) for x in i.region_free_bytes[:i.regions]],
@@ -767,7 +1022,24 @@ def main():
                 "kernel": wl.dominant, "algorithmic_bytes_per_launch": dom["bytes_per_elem"] * n,
                 "avg_launch_ms": dom["avg_ms"]}
 
-    deferred = wl.deferred_variant(args.steps) if args.workload == "cfg5" else None
+    # config 5 only: the same buffers stepped two other ways (every one a full optimizer step with the same
+    # result), then the self-check over all steps this process made
+    deferred = unfolded = verified = None
+    if args.workload == "cfg5":
+        segments = []
+
+        def book(steps):
+            h = ctx.read_norm_result(wl.res)
+            segments.append((steps, h.scale, h.sumsq))
+        book(wl.steps_done)
+        if args.variants:
+            deferred = wl.deferred_variant(args.steps)
+            if deferred:
+                book(wl.deferred_steps_done)
+            unfolded = wl.other_fold_variant(args.steps)
+            book(wl.other_fold_steps_done)
+        if args.verify == 1 or (args.verify == -1 and args.scale == 1.0):
+            verified = verify_cfg5(wl, segments)
     config = {"workload": f"{args.workload}: {wl.list_name}", "tensors": len(wl.sizes), "elements": n,
               "bytes_per_elem_per_step": wl.step_bytes_per_elem,
               "storage": getattr(wl, "storage", "float32 everywhere"),
@@ -778,29 +1050,51 @@ def main():
                                             "6.3 sigma)") if x),
               "scale": args.scale, "alloc": args.alloc, "placement": placement}
     dtype = wl.dtype
+    main_leg = leg_summary(r, wl, args.steps)
     wl.close()
 
-    full_default = args.workload == "cfg5" and args.scale == 1.0
-    if args.workload not in ("probes", "copy"):
+    if args.ceiling and args.workload not in ("probes", "copy"):
         roofline["measured_ceiling"] = measured_ceiling(args, torch, mxopt, ctx, pool)
         roofline["frac_of_measured_ceiling"] = round(dom["gbps"] / roofline["measured_ceiling"]["mix43_gbps"], 4)
+
+    if three_placements and pool is not None:
+        # what a drop-in host sees: its own allocator keeps parameters and gradients, the library's pool only
+        # moments and accumulation buffers
+        a = with_workload(args, args.workload)
+        a.placement = "state-pool"
+        w3 = Workload(a, torch, mxopt, ctx, pool)
+        state_pool_leg = leg_summary(measure(w3, 5, 2), w3, 5)
+        w3.close()
+        placement["legs"] = {
+            "arena (every buffer from the pool; the headline)": main_leg,
+            "state_pool (moments and accumulation buffers from the pool, parameters and gradients from torch's allocator)":
+                state_pool_leg,
+            "plain (torch's allocator for everything; child process run first, so the first allocations of a fresh process)":
+                plain_leg}
+        placement["adamw_gbps"] = {"arena": main_leg["dominant_kernel_gbps"],
+                                   "state_pool": state_pool_leg["dominant_kernel_gbps"],
+                                   "plain": (plain_leg or {}).get("dominant_kernel_gbps")}
 
     others = None
     if args.others == 1 or (args.others == -1 and full_default):
         others = {}
         for name in OTHER_CONFIGS:
             a = with_workload(args, name)
+            a.placement = "pool" if pool is not None else "plain"
+            steps2 = args.others_steps or OTHER_CONFIG_STEPS[name]
             w2 = Workload(a, torch, mxopt, ctx, pool)
-            r2 = measure(w2, args.others_steps, 2)
+            r2 = measure(w2, steps2, 2)
             d2 = r2["kernels"][w2.dominant]
             others[name] = {"list": w2.list_name, "tensors": len(w2.sizes), "elements": w2.n,
-                            "steps": args.others_steps, "steps_per_s": round(r2["steps_per_s"], 3),
+                            "steps": steps2, "steps_per_s": round(r2["steps_per_s"], 3),
                             "ms_per_step": round(r2["ms_per_step"], 4),
                             "bytes_per_elem_per_step": w2.step_bytes_per_elem,
                             "step_hbm_gbps": round(r2["step_gbps"], 1),
                             "dominant_kernel": w2.dominant, "dominant_kernel_ms": d2["avg_ms"],
                             "dominant_kernel_gbps": d2["gbps"], "frac": round(d2["gbps"] / HBM_PEAK_GBPS, 4),
                             "kernels": r2["kernels"]}
+            if hasattr(w2, "graph_variant"):
+                others[name]["hip_graph"] = w2.graph_variant(steps2)
             w2.close()
         if args.cpu_sample > 0:
             others["cfg1"]["cpu_baseline"] = cpu_baseline_cfg1_full()
@@ -821,11 +1115,17 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
+    if verified:
+        out["verified"] = verified
+    if unfolded:
+        out["other_fold"] = unfolded
     if deferred:
         out["deferred_accumulation"] = deferred
     if others:
         out["other_configs"] = others
     print(json.dumps(out))
+    if verified and not verified["ok"]:
+        sys.exit("bench.py: the timed configuration failed its own check (see `verified` in the line above)")
 
 
 if __name__ == "__main__":

@@ -44,18 +44,31 @@ def _run(cmd, verbose):
         print(err)
 
 
-def build(verbose: bool = False) -> str:
+def _headers_mtime() -> float:
+    dirs = [CSRC, os.path.join(ROOT, "include")]
+    return max(os.path.getmtime(os.path.join(d, f)) for d in dirs for f in os.listdir(d) if f.endswith(".h"))
+
+
+def build(verbose: bool = False, incremental: bool = False) -> str:
     """Every translation unit is compiled by its own hipcc process (they are independent and the three
-    kernel files take about as long as each other), then linked."""
+    kernel files take about as long as each other), then linked.  incremental: a unit whose object file is
+    newer than its source and than every header is not compiled again (for edit-compile loops; the default
+    compiles everything)."""
     from concurrent.futures import ThreadPoolExecutor
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     os.makedirs(OBJ_DIR, exist_ok=True)
-    jobs = []
+    jobs, objs = [], []
+    newest_header = _headers_mtime() if incremental else 0.0
     for s in SOURCES:
         obj = os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o")
-        jobs.append(([hipcc] + FLAGS + ["-x", "hip", "-c", os.path.join(CSRC, s), "-o", obj], obj))
-    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+        objs.append(obj)
+        src = os.path.join(CSRC, s)
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header):
+            continue
+        jobs.append(([hipcc] + FLAGS + ["-x", "hip", "-c", src, "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(max(len(jobs), 1), os.cpu_count() or 1, 8)) as pool:
         list(pool.map(lambda j: _run(j[0], verbose), jobs))
+    jobs = [(None, o) for o in objs]
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + [obj for _, obj in jobs] + ["-o", LIB + ".tmp"], verbose)
     os.replace(LIB + ".tmp", LIB)
     build_demo(verbose)
@@ -132,4 +145,4 @@ if __name__ == "__main__":
     if "--sanitize" in sys.argv:
         print(build_sanitized(verbose=True))
     else:
-        print(build(verbose=True))
+        print(build(verbose=True, incremental="--incremental" in sys.argv))

@@ -72,6 +72,7 @@ struct mxopt_engine {
   bool async_mode = false;                            // inside an async call
   const uint64_t* async_skip = nullptr;            // ... the device flag its kernels obey
   bool async_enqueued = false;                        // ... a flag copy was enqueued
+  Book* async_book = nullptr;                         // ... the bookkeeping to go back to (the caller's local)
   bool pending = false;
   int pending_applied = 0;
   Book before;
@@ -315,7 +316,9 @@ int defer_spill(mxopt_engine* e) {
     int rc = cached_table(ctx, rows, &t);
     if (rc) return rc;
     if (grpo) {
-      mxopt_grad_prep prep = guarded(e, grpo_clamp(e));
+      // Not guarded by the arriving micro-batch's validity flag: the two entries that move were accepted by
+      // earlier calls, and their sum is the same whatever the new micro-batch turns out to hold.
+      mxopt_grad_prep prep = grpo_clamp(e);
       if (e->cfg.has_gradient_clip_norm) prep.d_scale = &e->d_result[e->held_result[j]].scale;
       rc = mxopt_accumulate_transformed(ctx, t, j == 0, &prep);
     } else {
@@ -333,6 +336,11 @@ int defer_spill(mxopt_engine* e) {
   e->held_result[0] = -1;
   e->held.erase(e->held.begin() + 1);
   e->held_result.erase(e->held_result.begin() + 1);
+  if (e->async_book) {  // the spill stays whatever the arriving micro-batch's flag says: the caller's buffers are free
+    e->async_book->held = e->held;
+    e->async_book->held_result = e->held_result;
+    e->async_book->held_is_sum = true;
+  }
   return MXOPT_OK;
 }
 
@@ -945,13 +953,31 @@ int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const*
   e->async_mode = true;
   e->async_skip = nullptr;
   e->async_enqueued = false;
+  e->async_book = &before;
   mxopt_engine_metrics m;
   rc = grpo_micro_batch(e, idx, grads, &m);
   const bool enqueued = e->async_enqueued;
   e->async_mode = false;
   e->async_skip = nullptr;
   e->async_enqueued = false;
-  if (rc) return rc;
+  e->async_book = nullptr;
+  if (rc) {
+    // The call failed after its validity flag was asked for (a later check or a HIP error): the bookkeeping
+    // goes back to where it was, and a micro-batch that held a NaN/Inf is still booked as the skip the
+    // blocking call would have returned before it ever reached the failing step.
+    if (enqueued) {
+      const std::string why = ctx->err;
+      put_book(e, before);
+      bool bad = false;
+      {
+        DeviceGuard guard(ctx->device);
+        bad = hipEventSynchronize(e->copied) == hipSuccess && e->h_pinned->nonfinite != 0;
+      }
+      if (bad) (void)grpo_skipped(e, nullptr);
+      ctx->err = why;
+    }
+    return rc;
+  }
   if (enqueued) {
     e->pending = true;
     e->pending_applied = m.gradients_applied;
@@ -1041,12 +1067,17 @@ int mxopt_engine_reset(mxopt_engine* e) {
 int mxopt_engine_save_optimizer_state(mxopt_engine* e, const char* path) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_save_optimizer_state: null engine");
   if (!e->adamw) return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "this engine applies plain SGD: there is no optimizer state");
+  // An async micro-batch that is still unsettled has advanced the AdamW call counter as if it were valid:
+  // the file must hold the counter of the updates the device really made.
+  { int rc0 = settle(e, nullptr); if (rc0) return rc0; }
   return mxopt_optimizer_save_file(e->adamw, path);
 }
 
 int mxopt_engine_load_optimizer_state(mxopt_engine* e, const char* path) {
   if (!e) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_engine_load_optimizer_state: null engine");
   if (!e->adamw) return fail(e->ctx, MXOPT_ERR_INVALID_ARG, "this engine applies plain SGD: there is no optimizer state");
+  // Settled first: a later settle would otherwise write the counter of before the pending call over the loaded one.
+  { int rc0 = settle(e, nullptr); if (rc0) return rc0; }
   return mxopt_optimizer_load_file(e->adamw, path);
 }
 

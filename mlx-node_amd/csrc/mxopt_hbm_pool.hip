@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <cstdio>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -360,6 +361,12 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
         k = k2;
       }
       HIP_TRY(ctx, hipMemUnmap(va_ref, kSlabChunksBytes));
+      if (log_level() >= 2) {
+        std::string line = "hbm pool scan: reference slab " + std::to_string(ref) + ", threshold " + std::to_string((int)thr) + ":";
+        for (size_t k = 0; k < others.size(); ++k)
+          if (probed[k]) line += " " + std::to_string(others[k]) + "=" + std::to_string((int)rate[others[k]]);
+        std::fprintf(stderr, "mxopt: %s\n", line.c_str());  // longer than log_line's buffer
+      }
       if (abs_thr == 0.0) { abs_thr = thr; same_gbps = lo; cross_gbps = hi; }
       std::vector<int> rest;
       bool same = true;

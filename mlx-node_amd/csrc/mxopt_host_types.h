@@ -53,6 +53,11 @@ struct DevPrep {  // kernel argument
   uint32_t flags;
 };
 
+// True when a gradient stage runs before the optimizer's own ops: its result is float32 whatever g's dtype.
+inline bool prep_promotes(const DevPrep& prep) {
+  return (prep.flags & (kPrepPreMul | kPrepClampPre | kPrepClampPost)) != 0 || prep.d_scale != nullptr;
+}
+
 // Deferred accumulation with kPrepEachStream: the clip factor of tensor.g and of each pending stream
 // (device scalars; all NULL = no factor).
 struct StreamScales {

@@ -244,11 +244,6 @@ static bool adam_g2_for_pd(int od, int g2d, const Launch& L, const AdamMath& mat
   return false;
 }
 
-// True when a gradient stage runs before the optimizer's own ops: its result is float32 whatever g's dtype.
-static bool prep_promotes(const DevPrep& prep) {
-  return (prep.flags & (kPrepPreMul | kPrepClampPre | kPrepClampPost)) != 0 || prep.d_scale != nullptr;
-}
-
 bool launch_adam(int pd, int gd, int od, int g2d, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
   if (g2d < 0) return dispatch_update(pd, gd, od, L, AdamMath{hp, prep_promotes(prep) ? MXOPT_F32 : gd}, prep);
   if (gd != MXOPT_F32) return false;

@@ -103,10 +103,13 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
 
 bool launch_adam_list(int pd, int gd, int od, int xd, const Launch& L, const mxopt_adam_hp& hp, const DevPrep& prep) {
   if (od != pd) return false;
+  // With no pending stream and no stage in front, the gradient reaches the square as it came: a 16-bit
+  // tensor whose square is 16-bit too (as in launch_adam); any add or stage makes it float32 first.
+  const AdamMath math{hp, (L.npending == 0 && !prep_promotes(prep)) ? gd : MXOPT_F32};
   switch (pd) {
-    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, AdamMath{hp}, prep);
-    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, AdamMath{hp}, prep);
-    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, AdamMath{hp}, prep);
+    case MXOPT_F32: return update_list_for_pd<MXOPT_F32>(gd, xd, L, math, prep);
+    case MXOPT_BF16: return update_list_for_pd<MXOPT_BF16>(gd, xd, L, math, prep);
+    case MXOPT_F16: return update_list_for_pd<MXOPT_F16>(gd, xd, L, math, prep);
   }
   return false;
 }

@@ -405,3 +405,54 @@ def test_optimizer_object_steps_over_unsummed_micro_batches(mx, ctx, kind, which
     opt.update_many_accumulated([], [], [[] for _ in range(10)])   # an empty list is a no-op for any k
     if which == "adamw":
         assert opt.step == 5 * len(names)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("which", ["adamw", "rmsprop"])
+def test_lone_16bit_gradient_keeps_its_dtype_in_the_square(mx, ctx, kind, which):
+    """One micro-batch, no clip, no stage: the gradient reaches the optimizer as it came, so its square is a
+    16-bit tensor (mlx.cpp:2016-2020 through adamw.rs:92 / rmsprop.rs:80).  The deferred kernels with no
+    pending stream, update_many_accumulated with one micro-batch, update_many and the table kernel all have to
+    agree with update_single of the oracle on that."""
+    sizes = [5, 4096, 4099, 70001]
+    names = [f"w{i}" for i in range(len(sizes))]
+    ps = lists(71, sizes, kind, 0.02)
+    gs = [cast(g, kind) for g in lists(72, sizes, "f32", 3e-2)]   # large enough for the 16-bit rounding of g*g to show in v
+    make = {"adamw": (lambda: mx.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01, ctx=ctx), lambda: O.AdamW(1e-3, 0.9, 0.999, 1e-8, 0.01)),
+            "rmsprop": (lambda: mx.RMSprop(1e-2, 0.95, 1e-8, 0.0, ctx=ctx), lambda: O.RMSprop(1e-2, 0.95, 1e-8, 0.0))}[which]
+    ref = make[1]()
+    want_p = [cast(ref.update_single(n, p, g), kind) for n, p, g in zip(names, ps, gs)]
+    want_v = [ref.state[n][1] if which == "adamw" else ref.state[n] for n in names]
+    # the float32 square would give another v: the case has to be able to tell the two apart
+    wide = make[1]()
+    for n, p, g in zip(names, ps, gs):
+        wide.update_single(n, p, O.as_f32(g))
+    assert any(not np.array_equal((wide.state[n][1] if which == "adamw" else wide.state[n]), w) for n, w in zip(names, want_v))
+
+    # 1. optimizer object, one un-summed micro-batch
+    opt = make[0]()
+    dp = [to_dev(p) for p in ps]
+    opt.update_many_accumulated(names, dp, [[to_dev(g) for g in gs]])
+    for i, n in enumerate(names):
+        assert_bit_equal(to_host(dp[i]), want_p[i], f"update_many_accumulated p {n}")
+        assert_bit_equal(to_host(opt.state(n)[1]), want_v[i], f"update_many_accumulated v {n}")
+    # 2. the same through update_many
+    opt2 = make[0]()
+    dp2 = [to_dev(p) for p in ps]
+    opt2.update_many(names, dp2, [to_dev(g) for g in gs], outs=dp2)
+    for i, n in enumerate(names):
+        assert_bit_equal(to_host(dp2[i]), want_p[i], f"update_many p {n}")
+        assert_bit_equal(to_host(opt2.state(n)[1]), want_v[i], f"update_many v {n}")
+    # 3. the bare list kernel with no pending stream against the bare table kernel
+    dp3, dg3 = [to_dev(p) for p in ps], [to_dev(g) for g in gs]
+    dm3, dv3 = ([to_dev(np.zeros(n, F)) for n in sizes] for _ in range(2))
+    table = ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, m=m, v=v) for p, g, m, v in zip(dp3, dg3, dm3, dv3)])
+    table.set_pending([])
+    if which == "adamw":
+        ctx.adam_with_pending_list(table, mx.adam_hp(1e-3, 0.9, 0.999, 1e-8, 0.01))
+    else:
+        ctx.rmsprop_with_pending_list(table, mx.rmsprop_hp(1e-2, 0.95, 1e-8, 0.0))
+    for i, n in enumerate(names):
+        assert_bit_equal(to_host(dp3[i]), want_p[i], f"list kernel p {n}")
+        assert_bit_equal(to_host(dv3[i]), want_v[i], f"list kernel v {n}")
+    table.close()

@@ -129,3 +129,117 @@ def test_async_is_refused_where_nothing_blocks(mx):
         mx.SFTEngineOptimizerSide(dparams).micro_batch_async(g)
     dev = mx.GRPOEngineOptimizerSide(dparams)
     assert dev.settle().step == 0             # nothing pending: a no-op
+
+
+def _inspect_step(mx, path):
+    import ctypes as C
+    kind, step, tensors, elements = C.create_string_buffer(32), C.c_int64(), C.c_uint64(), C.c_uint64()
+    assert mx.load().mxopt_checkpoint_inspect(str(path).encode(), kind, 32, C.byref(step), C.byref(tensors),
+                                              C.byref(elements)) == 0
+    return step.value
+
+
+def test_save_and_load_settle_a_pending_micro_batch_first(mx, tmp_path):
+    """AdamW apply, one micro-batch per step.  A NaN micro-batch that is still unsettled has advanced the call
+    counter speculatively: a checkpoint written then must hold the counter of the updates that took place, and a
+    checkpoint loaded then must not be overwritten by the roll-back that follows."""
+    rng = np.random.default_rng(47)
+    params = make_params(rng, True)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=1, gradient_clip_norm=1e9, gradient_clip_value=0.02,
+              max_nan_gradients=50, emergency_save_threshold=2, apply="adamw", weight_decay=0.01)
+    dev = mx.GRPOEngineOptimizerSide(dparams, **kw)
+    ref = O.GRPOEngineOptimizerSide(params, **kw)
+    n = len(params)
+    keep = []
+
+    def call(kind, it):
+        grads = poisoned(rng, True, it, kind)
+        dg = {k: to_dev(g) for k, g in grads.items()}
+        keep.append(dg)
+        dev.micro_batch_async(dg)
+        ref.micro_batch(grads)
+
+    call("ok", 0)
+    first = tmp_path / "first.safetensors"
+    dev.save_optimizer_state(first)                   # settles the valid call: one update per parameter
+    assert _inspect_step(mx, first) == n
+    call("ok", 1)
+    call("nan", 2)                                    # unsettled; the counter stands at 3n speculatively
+    second = tmp_path / "second.safetensors"
+    dev.save_optimizer_state(second)
+    assert _inspect_step(mx, second) == 2 * n
+    check_state(dev, ref, dparams, "after the save")
+    call("inf", 3)                                    # unsettled again
+    dev.load_optimizer_state(first)                   # the skip is booked first, then the file's counter stands
+    third = tmp_path / "third.safetensors"
+    dev.save_optimizer_state(third)
+    assert _inspect_step(mx, third) == n
+    m = dev.metrics()
+    assert (m.step, m.nan_gradient_count) == (ref.state.step, ref.state.nan_gradient_count) == (4, 2)
+
+
+def test_spill_is_not_undone_by_an_invalid_arrival(mx):
+    """Deferred accumulation with more micro-batches than streams, asynchronous calls: the arrival that makes the
+    two oldest micro-batches move into the float32 buffers holds a NaN.  The move is made whatever that flag says,
+    so the caller may reuse those two buffers straight away, as after a blocking call."""
+    import torch
+    rng = np.random.default_rng(53)
+    params = make_params(rng, True)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    n_acc = 11
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=n_acc, gradient_clip_norm=1e9, gradient_clip_value=0.02,
+              max_nan_gradients=50, emergency_save_threshold=3)
+    dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
+    ref = O.GRPOEngineOptimizerSide(params, **kw)
+    script = ["ok"] * (mx.MAX_PENDING + 1) + ["nan"] + ["ok"] * (n_acc - mx.MAX_PENDING - 1)
+    sent = []
+    for it, kind in enumerate(script):
+        grads = poisoned(rng, True, it, kind)
+        dg = {k: to_dev(g) for k, g in grads.items()}
+        sent.append(dg)
+        dev.micro_batch_async(dg)
+        ref.micro_batch(grads)
+        if kind == "nan":
+            torch.cuda.synchronize()
+            for old in sent[:2]:                      # "free again after that call"
+                for t in old.values():
+                    t.fill_(float("nan"))
+    m = dev.settle()
+    assert m.gradients_applied and m.step == ref.state.step
+    check_state(dev, ref, dparams, "end of the cycle")
+
+
+@pytest.mark.parametrize("kind", ["ok", "nan"])
+def test_async_call_that_fails_after_its_flag_was_requested(mx, kind):
+    """Deferred accumulation refuses a micro-batch whose names differ from the cycle's -- after the norm pass and
+    the flag copy were enqueued.  The bookkeeping goes back to where it was; if the refused micro-batch also held
+    a NaN it is booked as the skip the blocking call would have returned before it reached that check."""
+    rng = np.random.default_rng(59)
+    params = make_params(rng, False)
+    dparams = {k: to_dev(v) for k, v in params.items()}
+    kw = dict(learning_rate=0.05, gradient_accumulation_steps=3, gradient_clip_norm=1e9, gradient_clip_value=0.02,
+              max_nan_gradients=50, emergency_save_threshold=3)
+    dev = mx.GRPOEngineOptimizerSide(dparams, defer_accumulation=True, **kw)
+    ref = O.GRPOEngineOptimizerSide(params, **kw)
+    g0 = make_grads(rng, False, 0.01)
+    d0 = {k: to_dev(g) for k, g in g0.items()}
+    dev.micro_batch_async(d0)
+    ref.micro_batch(g0)
+    sub = poisoned(rng, False, 1, kind)
+    del sub["ln"]
+    dsub = {k: to_dev(g) for k, g in sub.items()}
+    with pytest.raises(mx.InvalidArg, match="same gradient names"):
+        dev.micro_batch_async(dsub)
+    if kind == "nan":
+        ref.micro_batch(sub)                          # a skip: the raw values are tested before anything else
+    check_state(dev, ref, dparams, "after the refused call")
+    for it in (2, 3):                                 # the cycle goes on as if the refused call had not been made
+        g = make_grads(rng, False, 0.01)
+        dg = {k: to_dev(v) for k, v in g.items()}
+        d0[f"keep{it}"] = dg
+        dev.micro_batch_async(dg)
+        ref.micro_batch(g)
+    m = dev.settle()
+    assert m.gradients_applied
+    check_state(dev, ref, dparams, "end of the cycle")

@@ -272,3 +272,46 @@ def test_coefficients_are_f64_then_f32():  # mlx.cpp:531-535 with adamw.rs:88,94
     ad = O.Adam()
     ad.update_single("p", arr(0), g)
     assert ad.state["p"][1][0] == (g * g)[0] * O._f32(1.0 - 0.999)
+
+
+# ---- compositions that no reference test runs: hand-derived closed forms ----
+
+def test_clip_grad_value_and_norm_closed_form():  # optimizers/mod.rs:174-226
+    """Clamp to +-clip_value first (:188-192), the norm is taken of the CLAMPED values (:196-205), the factor is
+    min(max / (n + 1e-6), 1) in float32 (:207-213) and every clamped tensor is multiplied by it (:219-226).
+    [3, -4, 0.5] clamped to +-1 is [1, -1, 0.5]: n = sqrt(2.25) = 1.5, so with max 1 the factor is 1/(1.5+1e-6).
+    A factor taken of the raw values would be 1/sqrt(25.25); scaling before clamping would give [0.6, -0.8, 0.1]."""
+    g = {"a": arr(3, -4), "b": arr(0.5)}
+    out = O.GradientUtils.clip_grad_value_and_norm(g, 1.0, 1.0)
+    s = F(1.0) / (F(1.5) + F(1e-6))
+    assert np.array_equal(out["a"], arr(1, -1) * s) and np.array_equal(out["b"], arr(0.5) * s)
+    assert abs(float(out["a"][0]) - 2.0 / 3.0) < 1e-6
+    # norm below the maximum: the factor is min(...) = exactly 1, the clamped values come back unchanged
+    out = O.GradientUtils.clip_grad_value_and_norm(g, 1.0, 10.0)
+    assert np.array_equal(out["a"], arr(1, -1)) and np.array_equal(out["b"], arr(0.5))
+    # max_norm = None (:195, :222-224): the clamped values themselves, no multiply
+    out = O.GradientUtils.clip_grad_value_and_norm(g, 2.5, None)
+    assert np.array_equal(out["a"], arr(2.5, -2.5)) and np.array_equal(out["b"], arr(0.5))
+    assert O.GradientUtils.clip_grad_value_and_norm({}, 1.0, 1.0) == {}   # :179-181
+    # the result is float32 whatever the input (clip with float32 bounds promotes bf16)
+    out = O.GradientUtils.clip_grad_value_and_norm({"h": O.f32_to_bf16(arr(3, -4, 0.5))}, 1.0, 1.0)
+    assert out["h"].dtype == np.float32 and np.array_equal(out["h"], arr(1, -1, 0.5) * s)
+
+
+def test_clip_gradients_by_value_one_sided_bounds():  # gradients/mod.rs:299-312 over mlx.cpp:469-481
+    """Every tensor of the list is clamped on its own; a non-finite bound is 'no bound' on that side
+    (std::isfinite, mlx.cpp:473-478), so (-inf, 1) only caps and (0, +inf) only floors."""
+    gs = [arr(-5, -0.5, 0.5, 5), arr(7), arr()]
+    out = O.clip_gradients_by_value(gs, -1.0, 1.0)
+    assert [o.tolist() for o in out] == [[-1, -0.5, 0.5, 1], [1], []]
+    out = O.clip_gradients_by_value(gs, -math.inf, 1.0)
+    assert [o.tolist() for o in out] == [[-5, -0.5, 0.5, 1], [1], []]
+    out = O.clip_gradients_by_value(gs, 0.0, math.inf)
+    assert [o.tolist() for o in out] == [[0, 0, 0.5, 5], [7], []]
+    out = O.clip_gradients_by_value(gs, math.nan, math.nan)        # neither bound is finite: untouched
+    assert [o.tolist() for o in out] == [[-5, -0.5, 0.5, 5], [7], []]
+    # the bounds are cast to float32 before the comparison (static_cast<float>, :474, :477): 0.1 is not
+    # representable, and a value between float32(0.1) and the float64 0.1 is capped to float32(0.1)
+    out = O.clip_gradients_by_value([arr(0.2)], -1.0, 0.1)
+    assert out[0][0] == F(0.1) and float(out[0][0]) != 0.1
+    assert O.clip_gradients_by_value([], -1.0, 1.0) == []
