@@ -627,10 +627,14 @@ class Workload:
     def _setup_probes(self):
         t = self.torch
         with self._window("param"):
-            self.streams = [t.zeros(self.n, dtype=t.float32, device="cuda") for _ in range(4)]
+            self.streams = [t.zeros(self.n, dtype=t.float32, device="cuda") for _ in range(5)]
+        # the deferred update's mix: four 2-byte gradient streams and a 2-byte parameter (halves of two of the
+        # buffers, viewed as bf16), two 4-byte moments
+        halves = [h for s in (self.streams[1], self.streams[4]) for h in s.view(t.bfloat16).chunk(2)]
+        self.list_streams = (self.streams[0].view(t.bfloat16)[:self.n], self.streams[2], self.streams[3], halves)
         self.dtype = "u32"
-        self.bytes_per_elem = {"probe_read": 4, "probe_write": 4, "probe_copy": 8, "probe_mix43": 28}
-        self.step_bytes_per_elem = 44
+        self.bytes_per_elem = {"probe_read": 4, "probe_write": 4, "probe_copy": 8, "probe_mix43": 28, "probe_list4": 28}
+        self.step_bytes_per_elem = 72
         self.dominant = "probe_mix43"
         self.note = "bare kernels: no table, no tails, no arithmetic; mix43 = float32 AdamW's four read and three write streams"
 
@@ -639,7 +643,9 @@ class Workload:
         self._timed("probe_read", lambda: c.probe_stream(mx.PROBE_READ, s[0]))
         self._timed("probe_write", lambda: c.probe_stream(mx.PROBE_WRITE, s[1]))
         self._timed("probe_copy", lambda: c.probe_stream(mx.PROBE_COPY, s[0], s[1]))
-        self._timed("probe_mix43", lambda: c.probe_stream(mx.PROBE_MIX43, *s))
+        self._timed("probe_mix43", lambda: c.probe_stream(mx.PROBE_MIX43, *s[:4]))
+        p16, m, v, gs = self.list_streams
+        self._timed("probe_list4", lambda: c.probe_list(p16, m, v, gs))
 
     def step(self):
         getattr(self, "_step_" + self.args.workload.replace("-", "_"))()
@@ -921,8 +927,10 @@ def measured_ceiling(args, torch, mx, ctx, pool):
     k = r["kernels"]
     return {"mix43_gbps": k["probe_mix43"]["gbps"], "copy_gbps": k["probe_copy"]["gbps"],
             "read_gbps": k["probe_read"]["gbps"], "write_gbps": k["probe_write"]["gbps"],
-            "what": "bare float32 streaming kernels (no table, no arithmetic) over 4 GiB per stream from the same "
-                    "allocator, measured in this run; mix43 = 4 read + 3 write streams in place",
+            "list4_gbps": k["probe_list4"]["gbps"],
+            "what": "bare streaming kernels (no table, no arithmetic) over 4 GiB per float32 stream from the same "
+                    "allocator, measured in this run; mix43 = 4 read + 3 write streams in place; list4 = the deferred "
+                    "update's mix: four 2-byte gradient streams and a 2-byte parameter, two 4-byte moments, 28 B/elem",
             "profile": PROBE_PROFILE}
 
 

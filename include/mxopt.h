@@ -165,6 +165,10 @@ void mxopt_hbm_pool_hook_free(void* ptr, ptrdiff_t size, int device, void* strea
  * (MIX43 is float32 AdamW's byte mix, 28 B/elem.)  One launch on the context's stream. */
 enum { MXOPT_PROBE_READ = 0, MXOPT_PROBE_WRITE = 1, MXOPT_PROBE_COPY = 2, MXOPT_PROBE_MIX43 = 3 };
 int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n_elems);
+/* The byte mix of the update over k un-summed 16-bit micro-batches (mxopt_adam_with_pending_list) without its
+ * arithmetic: g[0..k) and p are 2-byte streams of n_elems elements, m and v 4-byte ones; p, m and v are
+ * rewritten in place (2k + 20 B/elem).  k in [1, 8], n_elems a positive multiple of 4096. */
+int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k, uint64_t n_elems);
 
 /* ---- tensor table ------------------------------------------------------------------
  * One descriptor per tensor.  Which fields a kernel reads is listed at that kernel;
@@ -216,10 +220,14 @@ typedef struct mxopt_norm_result {
   double   norm;      /* sqrt(sumsq)                                                */
   float    norm_f32;  /* (float)norm: what clip_grad_norm_with_norm returns          */
   float    scale;     /* clip factor, see mxopt_clip_mode                           */
-  uint64_t nonfinite; /* 1 when the sum of squares is not finite (a NaN/Inf element, or
-                         squares beyond float32 range) or when prep's clamp_pre met a raw
-                         +-Inf (which the clamp would have hidden), else 0: the engines'
-                         validity checks (grpo/engine.rs:563-569, :1692-1698)          */
+  uint64_t nonfinite; /* 0: every element finite.  1: some element is a NaN or an infinity -- the
+                         engines' per-element validity check (grpo/engine.rs:563-569), also under
+                         prep's clamp_pre, which would have hidden a raw +-Inf; sumsq, norm and
+                         scale are NaN then.  2: every element is finite but their squares left
+                         float32 range: sumsq and norm are +Inf and scale 0, which is what the
+                         reference's own float32 chain makes of such gradients
+                         (optimizers/mod.rs:78-96); kernels told to skip on this flag look at
+                         bit 0 only and still run                                           */
 } mxopt_norm_result;
 
 /* How `scale` is derived from the norm. */
@@ -244,9 +252,10 @@ typedef struct mxopt_grad_prep {
   int          has_clamp_pre;  float pre_lo, pre_hi;    /* mlx clip, mlx.cpp:469-481        */
   const float* d_scale;        /* device scalar (e.g. &norm_result->scale); NULL = none    */
   int          has_clamp_post; float post_lo, post_hi;
-  /* Device counter (e.g. &norm_result->nonfinite); when it is non-zero the update / transform
-   * kernel changes nothing: the engines' "any NaN/Inf gradient => skip the whole step" policy
-   * (grpo/engine.rs:561-607, sft/engine.rs:221-258) without a host round trip.  NULL = never skip. */
+  /* Device flag word (e.g. &norm_result->nonfinite); when its bit 0 is set -- some gradient element was a
+   * NaN or an infinity -- the update / transform kernel changes nothing: the engines' "any NaN/Inf
+   * gradient => skip the whole step" policy (grpo/engine.rs:561-607, sft/engine.rs:221-258) without a
+   * host round trip.  NULL = never skip. */
   const uint64_t* d_skip_if_nonzero;
 } mxopt_grad_prep;
 

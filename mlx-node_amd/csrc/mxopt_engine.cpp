@@ -415,7 +415,7 @@ int settle(mxopt_engine* e, mxopt_engine_metrics* out) {
   }
   e->pending = false;
   const mxopt_norm_result h = *e->h_pinned;
-  if (h.nonfinite) {
+  if (h.nonfinite & 1u) {  // bit 0: an invalid element; the kernels looked at the same bit
     put_book(e, e->before);
     return grpo_skipped(e, out);
   }
@@ -449,7 +449,7 @@ int grpo_micro_batch(mxopt_engine* e, const std::vector<size_t>& idx, const mxop
     // async: the flag is not waited for; every kernel below obeys it on the device instead
     if ((rc = e->async_mode ? enqueue_flag_copy(e, d_result) : mxopt_read_norm_result(ctx, d_result, &h))) return rc;
   }
-  if (h.nonfinite) return grpo_skipped(e, out);  // engine.rs:571-633: skip the whole micro-batch, touch nothing
+  if (h.nonfinite & 1u) return grpo_skipped(e, out);  // engine.rs:571-633: skip the whole micro-batch, touch nothing
   e->consecutive_nan_count = 0;  // engine.rs:660
   if (!e->have_acc)
     for (Slot& s : e->slots) s.in_acc = false;  // also after a call that failed half way
@@ -971,7 +971,7 @@ int mxopt_engine_micro_batch_async(mxopt_engine* e, size_t n, const char* const*
       bool bad = false;
       {
         DeviceGuard guard(ctx->device);
-        bad = hipEventSynchronize(e->copied) == hipSuccess && e->h_pinned->nonfinite != 0;
+        bad = hipEventSynchronize(e->copied) == hipSuccess && (e->h_pinned->nonfinite & 1u) != 0;
       }
       if (bad) (void)grpo_skipped(e, nullptr);
       ctx->err = why;

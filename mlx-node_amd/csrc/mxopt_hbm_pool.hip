@@ -90,6 +90,58 @@ __global__ __launch_bounds__(kProbeThreads) void probe_mix43_kernel(pu32x4* __re
   }
 }
 
+// The byte mix of the update over un-summed 16-bit micro-batches (deferred accumulation) without its
+// arithmetic: per element K + 1 two-byte reads (the gradient streams and the parameter), two four-byte
+// reads (the moments); the parameter and the moments are written back in place.  One workgroup per
+// 4096-element tile, every load of the tile issued before the first store, as in the update kernels.
+template <int K>
+__global__ __launch_bounds__(kProbeThreads) void probe_list_kernel(pu32x4* __restrict__ p, pu32x4* __restrict__ m,
+                                                                  pu32x4* __restrict__ v,
+                                                                  const pu32x4* __restrict__ g0, const pu32x4* __restrict__ g1,
+                                                                  const pu32x4* __restrict__ g2, const pu32x4* __restrict__ g3,
+                                                                  const pu32x4* __restrict__ g4, const pu32x4* __restrict__ g5,
+                                                                  const pu32x4* __restrict__ g6, const pu32x4* __restrict__ g7,
+                                                                  uint32_t ntiles) {
+  constexpr int U = 2;  // groups of 8 elements per lane: 2 x 256 x 8 = 4096 elements per tile
+  const pu32x4* gs[8] = {g0, g1, g2, g3, g4, g5, g6, g7};
+  for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t b16 = (size_t)t * (kProbeThreads * U) + threadIdx.x;      // 16-byte pieces of a 2-byte stream
+    const size_t b32 = (size_t)t * (kProbeThreads * U * 2) + threadIdx.x;  // ... of a 4-byte stream
+    pu32x4 rg[K][U], rp[U], rm[U][2], rv[U][2];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) rg[k][j] = gs[k][b16 + j * kProbeThreads];
+      rp[j] = p[b16 + j * kProbeThreads];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        rm[j][h] = m[b32 + (2 * j + h) * kProbeThreads];
+        rv[j][h] = v[b32 + (2 * j + h) * kProbeThreads];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      pu32x4 s = rg[0][j];
+#pragma unroll
+      for (int k = 1; k < K; ++k) s += rg[k][j];
+      p[b16 + j * kProbeThreads] = rp[j] ^ s;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        m[b32 + (2 * j + h) * kProbeThreads] = rm[j][h] + s;
+        v[b32 + (2 * j + h) * kProbeThreads] = rv[j][h] ^ (s >> 1);
+      }
+    }
+  }
+}
+
+template <int K>
+static void launch_probe_list_k(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, uint32_t ntiles) {
+  const pu32x4* q[8];
+  for (int k = 0; k < 8; ++k) q[k] = (const pu32x4*)g[k < K ? k : 0];
+  hipLaunchKernelGGL(probe_list_kernel<K>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)p, (pu32x4*)m,
+                     (pu32x4*)v, q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], ntiles);
+}
+
 static int launch_probe(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n) {
   const uint32_t ntiles = (uint32_t)(n / kProbeTileElems);
   const uint32_t bounded = (uint32_t)std::min<uint64_t>(ntiles, (uint64_t)ctx->num_cus * 16u);
@@ -207,6 +259,32 @@ int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void
       return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: buffers must be non-NULL and 16-byte aligned");
   DeviceGuard guard(ctx->device);
   return launch_probe(ctx, kind, a, b, c, d, n_elems);
+}
+
+int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k, uint64_t n_elems) {
+  const char* op = "mxopt_probe_list";
+  if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null context");
+  if (n_elems == 0 || n_elems % 4096 != 0 || n_elems / 4096 > 0xffffffffull)
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": n_elems must be a positive multiple of 4096");
+  if (k < 1 || k > 8 || !g) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": 1 to 8 gradient streams");
+  const void* ptrs[11] = {p, m, v};
+  for (int i = 0; i < k; ++i) ptrs[3 + i] = g[i];
+  for (int i = 0; i < 3 + k; ++i)
+    if (!ptrs[i] || (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": buffers must be non-NULL and 16-byte aligned");
+  DeviceGuard guard(ctx->device);
+  const uint32_t ntiles = (uint32_t)(n_elems / 4096);
+  switch (k) {
+    case 1: launch_probe_list_k<1>(ctx, p, m, v, g, ntiles); break;
+    case 2: launch_probe_list_k<2>(ctx, p, m, v, g, ntiles); break;
+    case 3: launch_probe_list_k<3>(ctx, p, m, v, g, ntiles); break;
+    case 4: launch_probe_list_k<4>(ctx, p, m, v, g, ntiles); break;
+    case 5: launch_probe_list_k<5>(ctx, p, m, v, g, ntiles); break;
+    case 6: launch_probe_list_k<6>(ctx, p, m, v, g, ntiles); break;
+    case 7: launch_probe_list_k<7>(ctx, p, m, v, g, ntiles); break;
+    default: launch_probe_list_k<8>(ctx, p, m, v, g, ntiles); break;
+  }
+  return check_launch(ctx, op);
 }
 
 int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,

@@ -164,8 +164,10 @@ __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, con
 
 // The engines skip the whole step when any gradient element is NaN/Inf (grpo/engine.rs:561-607):
 // with a counter from the norm pass the update kernels honour that without a host round trip.
+// Bit 0 of mxopt_norm_result.nonfinite is "some element was a NaN or an infinity"; bit 1 (finite elements
+// whose squares overflowed) does not stop a step: the reference clips such gradients to zero and goes on.
 __device__ __forceinline__ bool skip_requested(const DevPrep& prep) {
-  return prep.d_skip_if_nonzero != nullptr && *prep.d_skip_if_nonzero != 0ull;
+  return prep.d_skip_if_nonzero != nullptr && (*prep.d_skip_if_nonzero & 1ull) != 0ull;
 }
 
 // A value clamp would turn +-Inf into a finite bound and hide it from the sum-based validity
@@ -175,8 +177,8 @@ __device__ __forceinline__ bool skip_requested(const DevPrep& prep) {
 // a NaN or an infinity (its partial is poisoned afterwards), so the clamp itself can be a single
 // median-of-three that does not care about NaN.
 __device__ __forceinline__ float norm_value(const PrepRegs& pr, float x, bool clamped, bool& bad) {
-  if (!clamped) return prep_pre(pr, x);
   bad |= !__builtin_isfinite(x);
+  if (!clamped) return prep_pre(pr, x);
   if (pr.flags & kPrepPreMul) x = x * pr.pre_mul;
   return __builtin_amdgcn_fmed3f(x, pr.pre_lo, pr.pre_hi);
 }

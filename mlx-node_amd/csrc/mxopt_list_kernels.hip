@@ -22,8 +22,15 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
     const ChunkView cv = locate(T, C, one, c);
     const PendingStreams<KMAX> ps = pending_of<KMAX>(X, ntensors, cv.tensor, kx);
     const void* G = cv.t.g;
-    float s32 = 0.0f;
+    float s32 = 0.0f, poison = 0.0f;
     bool bad = false;
+    // Full chunks: validity of the sum costs one multiply-add per element (s * 0 is NaN exactly for a NaN or an
+    // infinity); under a clamp the lane's partial is poisoned afterwards, so the clamp need not care about NaN.
+    auto fast_value = [&](float s) {
+      poison = fmaf(s, 0.0f, poison);
+      if (pr.flags & kPrepPreMul) s = s * pr.pre_mul;
+      return clamped ? __builtin_amdgcn_fmed3f(s, pr.pre_lo, pr.pre_hi) : s;
+    };
     auto one_element = [&](uint64_t off) {
       const float y = norm_value(pr, pending_sum_element<GD, XD, KMAX>(G, ps, kx, off), clamped, bad);
       s32 = fmaf(y, y, s32);
@@ -43,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
 #pragma unroll
           for (int k = 0; k < KMAX; ++k)
             if (k < kx) s = s + x[k][e];
-          const float y = norm_value(pr, s, clamped, bad);
+          const float y = fast_value(s);
           s32 = fmaf(y, y, s32);
         }
       }
@@ -65,7 +72,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
 #pragma unroll
           for (int k = 0; k < KMAX; ++k)
             if (k < kx) s = s + x[k][j][e];
-          const float y = norm_value(pr, s, clamped, bad);
+          const float y = fast_value(s);
           s32 = fmaf(y, y, s32);
         }
       }
@@ -93,7 +100,7 @@ __global__ __launch_bounds__(kThreads) void sumsq_list_kernel(const DevTensor* _
     }
     if (tid < cv.head) one_element(tid);
     // As in sumsq_kernel: float32 inside a chunk, float64 across chunks; a hidden NaN/Inf poisons the partial.
-    acc_sum += (double)(bad ? __builtin_nanf("") : s32);
+    acc_sum += (double)((bad || poison != poison) ? __builtin_nanf("") : s32);
   }
 
   unsigned long long unused = 0;

@@ -1,6 +1,7 @@
 // mxopt kernels for gfx950, part 2: global-norm reduction (optionally fused with gradient accumulation)
 // and the synthetic-data generator.
 #include <mutex>
+#include <type_traits>
 
 #include "mxopt_kernels_common.h"
 #include "mxopt_gauss_table.h"
@@ -75,7 +76,27 @@ struct SumsqChunk {
       }
       return poison != poison ? __builtin_nanf("") : s32;
     }
-    const bool clamped = (pr.flags & kPrepClampPre) != 0;
+    // No clamp: x * 0 is NaN exactly for a NaN or an infinity, so one multiply-add per element tells an
+    // invalid element (the partial becomes NaN) from squares of finite elements that overflow float32 (+Inf).
+    if (!(pr.flags & kPrepClampPre)) {
+      float poison = 0.0f;
+      auto body = [&](auto with_mul) {  // the stage flag is tested once per chunk, not per element
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
+            if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
+            poison = fmaf(x[j][e], 0.0f, poison);
+            const float y = decltype(with_mul)::value ? x[j][e] * pr.pre_mul : x[j][e];
+            s32 = fmaf(y, y, s32);
+          }
+          if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
+        }
+      };
+      if (pr.flags & kPrepPreMul) body(std::true_type{}); else body(std::false_type{});
+      return poison != poison ? __builtin_nanf("") : s32;
+    }
     bool hidden_inf = false;
 #pragma unroll
     for (int j = 0; j < U; ++j) {
@@ -83,7 +104,7 @@ struct SumsqChunk {
       for (int e = 0; e < E; ++e) {
         if (MODE == 2) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], first);
         if (MODE == 3) x[j][e] = accumulate_op<AD, GD>(x[j][e], g[j][e], false);
-        const float y = norm_value(pr, x[j][e], clamped, hidden_inf);
+        const float y = norm_value(pr, x[j][e], true, hidden_inf);
         s32 = fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, NT>(cv.t.g_out, cv.start + (uint64_t)(j * kThreads + tid) * E, x[j]);
@@ -110,6 +131,7 @@ struct SumsqChunk {
     void* A = cv.t.g_out;
     float s32 = 0.0f;
     const bool clamped = (pr.flags & kPrepClampPre) != 0;
+    bool bad = false;
     const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;
     for (uint32_t q = tid; q < ngroups; q += kThreads) {
       const uint64_t off = cv.start + (uint64_t)q * E;
@@ -125,12 +147,12 @@ struct SumsqChunk {
       for (int e = 0; e < E; ++e) {
         if (MODE == 2) x[e] = accumulate_op<AD, GD>(x[e], g[e], first);
         if (MODE == 3) x[e] = accumulate_op<AD, GD>(x[e], g[e], false);
-        bool bad = false;
         const float y = norm_value(pr, x[e], clamped, bad);
-        s32 = bad ? __builtin_nanf("") : fmaf(y, y, s32);
+        s32 = fmaf(y, y, s32);
       }
       if (MODE == 2) store_group<AD, E, false>(A, off, x);
     }
+    if (bad) s32 = __builtin_nanf("");
     for (uint32_t i = ngroups * E + tid; i < cv.len; i += kThreads) s32 = one_element(cv, pr, cv.start + i, first, s32);
     return s32;
   }
@@ -177,8 +199,14 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
     }
     return;
   }
+  // The descriptor of the workgroup's next chunk (two dependent table reads) is fetched while the current
+  // chunk's data is under way: with thousands of small tensors every trip would otherwise wait three memory
+  // round trips in a row.
+  ChunkView ahead{};
+  if (c < nchunks) ahead = locate(T, C, one, c);
   for (; c < nchunks; c += gridDim.x) {
-    const ChunkView cv = locate(T, C, one, c);
+    const ChunkView cv = ahead;
+    if (c + gridDim.x < nchunks) ahead = locate(T, C, one, c + gridDim.x);
     float s;
     if (MODE < 2 && AD != MXOPT_F32 && cv.fast && pr.flags == 0) {
       // 16-bit values squared as they are: one packed dot product per pair (v_dot2_f32_bf16 / v_dot2_f32_f16)
@@ -190,6 +218,8 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
 #pragma unroll
       for (int j = 0; j < 2; ++j) r[j] = NT ? __builtin_nontemporal_load(q + j * kThreads) : q[j * kThreads];
       s = 0.0f;
+      // validity: a pair times (0, 0) is NaN exactly when one of the two is a NaN or an infinity
+      float poison = 0.0f;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const uint32_t w[4] = {r[j].x, r[j].y, r[j].z, r[j].w};
@@ -198,12 +228,15 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
           if (AD == MXOPT_BF16) {
             const bf16x2_t v = __builtin_bit_cast(bf16x2_t, w[e]);
             s = __builtin_amdgcn_fdot2_f32_bf16(v, v, s, false);
+            poison = __builtin_amdgcn_fdot2_f32_bf16(v, __builtin_bit_cast(bf16x2_t, 0u), poison, false);
           } else {
             const f16x2_t v = __builtin_bit_cast(f16x2_t, w[e]);
             s = __builtin_amdgcn_fdot2(v, v, s, false);
+            poison = __builtin_amdgcn_fdot2(v, __builtin_bit_cast(f16x2_t, 0u), poison, false);
           }
         }
       }
+      if (poison != poison) s = __builtin_nanf("");
     } else if (cv.fast) {
       Chunk k;
       k.load(cv, tid, first);
@@ -213,8 +246,8 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
     }
     if (tid < cv.head) s = Chunk::one_element(cv, pr, tid, first, s);
     // A lane's float32 partial covers <= 16 squares of one chunk; chunks are combined in float64.
-    // A NaN/Inf element (or squares that overflow float32) makes the partial, and so the total,
-    // non-finite: that is the validity check (the reference's sum-based one, grpo/engine.rs:1692-1698).
+    // A NaN/Inf element makes the partial, and so the total, NaN: the engines' validity check
+    // (grpo/engine.rs:563-569).  Squares of finite elements that overflow float32 make it +Inf instead.
     acc_sum += (double)s;
   }
 
@@ -254,7 +287,9 @@ __global__ __launch_bounds__(kThreads) void norm_finish_kernel(const double* __r
     out->norm = norm;
     out->norm_f32 = norm32;
     out->scale = scale;
-    out->nonfinite = (sumsq - sumsq == 0.0) ? 0ull : 1ull;  // x - x is 0 exactly for finite x only
+    // NaN: some element was a NaN or an infinity (1).  +Inf: every element was finite and their squares left
+    // float32 range (2): the reference goes on with a clip factor of 0 there, and so does `scale` above.
+    out->nonfinite = (sumsq != sumsq) ? 1ull : (sumsq - sumsq == 0.0) ? 0ull : 2ull;
   }
 }
 

@@ -116,6 +116,7 @@ SIGNATURES = {
     "mxopt_hbm_pool_hook_alloc": (C.c_void_p, [C.c_ssize_t, C.c_int, C.c_void_p]),
     "mxopt_hbm_pool_hook_free": (None, [C.c_void_p, C.c_ssize_t, C.c_int, C.c_void_p]),
     "mxopt_probe_stream": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64]),
+    "mxopt_probe_list": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_uint64]),
     "mxopt_table_set_pending": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_void_p), C.c_int]),
     "mxopt_norm_with_pending_list": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(GradPrep), C.c_double, C.c_int,
                                                C.c_void_p]),

@@ -736,3 +736,64 @@ def test_subnormal_intermediates(mx, ctx, kind):
             assert (np.abs(v_ref[v_ref != 0]) < np.finfo(F).tiny).any()        # the test does reach subnormals
         dp.copy_(do)
     table.close()
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("where", ["full chunk", "last chunk", "head"])
+@pytest.mark.parametrize("path", ["norm", "accumulate", "norm_only", "list"])
+def test_validity_flag_tells_invalid_elements_from_overflowing_squares(mx, ctx, bf16, where, path):
+    """Without a clamp the flag is the engines' per-element test (grpo/engine.rs:563-569): bit 0 says "some
+    element is a NaN or an infinity".  A finite 1e20 is a valid gradient whose square leaves float32 range: the
+    reference's own sum of squares becomes +Inf there, its clip factor 0 (optimizers/mod.rs:87-96), and the step
+    is taken with zeroed gradients -- so the flag reads 2, the factor 0, and a kernel told to skip on the flag
+    still runs.  A real infinity reads 1 and the kernel does nothing."""
+    import torch
+    sizes = [3 * 4096 + 100, 300]
+    _, gs = make_lists(90, sizes=sizes, bf16=bf16, outliers=False)
+    shift = 1 if where == "head" else 0          # a one-element shift: the vector path runs behind a peeled head
+    at = {"full chunk": 4096 + 77, "last chunk": 3 * 4096 + 50, "head": 0}[where]
+
+    def put(value):
+        out = [g.copy() for g in gs]
+        if bf16:
+            out[0][at] = O.f32_to_bf16(np.array([value], F))[0]
+        else:
+            out[0][at] = value
+        return out
+
+    def flag_of(grads):
+        shift_g = shift * (7 if bf16 else 3)     # 14 / 12 bytes in: every stream of the row is aligned again one element later
+        dg = [to_dev(g, shift_g) for g in grads]
+        res = ctx.norm_result()
+        if path == "norm":
+            t = ctx.table([mx.TensorSpec(g=g) for g in dg])
+            ctx.global_norm(t, res, max_norm=1.0)
+        elif path == "list":
+            dz = [to_dev(np.zeros_like(g), shift_g) for g in grads]
+            t = ctx.table([mx.TensorSpec(g=z) for z in dz])
+            t.set_pending([dg])
+            ctx.norm_with_pending_list(t, res, max_norm=1.0)
+        else:
+            da = [to_dev(np.zeros(g.size, F), shift * 3) for g in grads]
+            t = ctx.table([mx.TensorSpec(g=g, g_out=a) for g, a in zip(dg, da)])
+            if path == "accumulate":
+                ctx.accumulate(t, first=False, out=res, max_norm=1.0)
+            else:
+                ctx.accumulate_norm_only(t, res, max_norm=1.0)
+        r = ctx.read_norm_result(res)
+        # what a kernel that obeys the flag does afterwards
+        dst = [torch.full((g.size,), 7.0, device="cuda") for g in grads]
+        tt = ctx.table([mx.TensorSpec(g=g, g_out=o) for g, o in zip(dg, dst)])
+        ctx.grad_transform(tt, mx.make_prep(scale=res, skip_if_nonfinite=res))
+        ran = bool((dst[1] != 7.0).any())
+        t.close(); tt.close()
+        return r, ran, dst
+
+    r, ran, _ = flag_of(put(0.001))
+    assert r.nonfinite == 0 and ran
+    r, ran, dst = flag_of(put(1e20))
+    assert r.nonfinite == 2 and math.isinf(r.sumsq) and r.scale == 0.0 and ran
+    assert float(dst[0].abs().max()) == 0.0 and float(dst[1].abs().max()) == 0.0     # finite gradients times 0
+    for bad in (np.inf, -np.inf, np.nan):
+        r, ran, _ = flag_of(put(bad))
+        assert r.nonfinite == 1 and math.isnan(r.sumsq) and not ran
