@@ -71,6 +71,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg5",
                     choices=["cfg1", "cfg1-update-single", "cfg1-update-many", "cfg2", "cfg3-sgd", "cfg3-rmsprop",
+                             "cfg3-sgd-deferred", "cfg3-rmsprop-deferred",
                              "cfg4", "cfg4-flat", "cfg5", "cfg5-deferred", "copy", "probes", "grpo-engine", "sft-engine"])
     ap.add_argument("--cpu-sample", type=int, default=512 * 1024 * 1024,
                     help="elements of the CPU-baseline sample (0 = skip the CPU leg)")
@@ -127,7 +128,7 @@ def parse_args():
 
 def tensor_sizes(args):
     from mxopt.qwen3_shapes import QWEN3, numel, param_list
-    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg5": "8B", "cfg5-deferred": "8B", "grpo-engine": "8B", "sft-engine": "8B"}.get(args.workload)
+    model = {"cfg1": "0.6B", "cfg1-update-single": "0.6B", "cfg1-update-many": "0.6B", "cfg2": "1.7B", "cfg3-sgd": "4B", "cfg3-rmsprop": "4B", "cfg3-sgd-deferred": "4B", "cfg3-rmsprop-deferred": "4B", "cfg5": "8B", "cfg5-deferred": "8B", "grpo-engine": "8B", "sft-engine": "8B"}.get(args.workload)
     if model:
         sizes = []
         for _, shape in param_list(QWEN3[model]):
@@ -196,6 +197,7 @@ class Workload:
     # -- helpers
     SEED = 0x5EED0001
     CONFIG_ID = {"cfg1": 1, "cfg1-update-single": 1, "cfg1-update-many": 1, "cfg2": 2, "cfg3-sgd": 3, "cfg3-rmsprop": 3,
+                 "cfg3-sgd-deferred": 3, "cfg3-rmsprop-deferred": 3,
                  "cfg4": 4, "cfg4-flat": 4, "cfg5": 5, "cfg5-deferred": 5, "copy": 6, "grpo-engine": 7, "sft-engine": 8,
                  "probes": 9}
 
@@ -530,6 +532,40 @@ class Workload:
     def _step_cfg3_rmsprop(self):
         self._timed("rmsprop", lambda: self.ctx.rmsprop(self.t_upd, self.hp))
 
+    # -- cfg3's optimizers over --micro un-summed float32 micro-batches (deferred accumulation): the norm of the sum
+    #    (4k B/elem, read only) and the update over k + 2 read and 2 write streams (4k + 16 B/elem)
+    def _setup_cfg3_deferred(self, which):
+        t, mx = self.torch, self.mx
+        k = self.n_micro = self.args.micro
+        self.p = self._randn_list(t.float32, 0.02, kind="param")
+        self.g = [self._randn_list(t.float32, 1e-3) for _ in range(k)]
+        self.v = self._zeros_list()
+        self.t_upd = self.ctx.table([mx.TensorSpec(p=p, p_out=p, g=g, v=v) for p, g, v in zip(self.p, self.g[0], self.v)])
+        self.t_upd.set_pending(self.g[1:])
+        self.prep = mx.make_prep(scale=self.res)
+        self.hp = mx.sgd_hp(1e-4, 0.9, 1e-4, 0.0, False) if which == "sgd" else mx.rmsprop_hp(1e-4, 0.99, 1e-8, 0.0)
+        self.dtype = "f32"
+        self.bytes_per_elem = {"norm_of_sum": 4 * k, which: 4 * k + 16}
+        self.step_bytes_per_elem = 8 * k + 16
+        self.dominant = which
+        self.note = f"{k} resident float32 micro-batches summed in registers by the norm pass and by the update; clip 1.0"
+
+    def _setup_cfg3_sgd_deferred(self):
+        self._setup_cfg3_deferred("sgd")
+
+    def _setup_cfg3_rmsprop_deferred(self):
+        self._setup_cfg3_deferred("rmsprop")
+
+    def _step_cfg3_sgd_deferred(self):
+        c = self.ctx
+        self._timed("norm_of_sum", lambda: c.norm_with_pending_list(self.t_upd, self.res, max_norm=1.0))
+        self._timed("sgd", lambda: c.sgd_with_pending_list(self.t_upd, self.hp, self.prep))
+
+    def _step_cfg3_rmsprop_deferred(self):
+        c = self.ctx
+        self._timed("norm_of_sum", lambda: c.norm_with_pending_list(self.t_upd, self.res, max_norm=1.0))
+        self._timed("rmsprop", lambda: c.rmsprop_with_pending_list(self.t_upd, self.hp, self.prep))
+
     # -- the engines' optimizer side (include/mxopt_engine.h) on the 8B list: 4 micro-batches of bf16
     #    gradients per optimizer step, bf16 parameters updated in place by the reference's plain SGD
     def _setup_engine(self, kind):
@@ -822,7 +858,7 @@ def cpu_baseline(args, n_total):
         t_unfused = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=False))
         fused_s = timeit(lambda: oc.adam(p32, g32, m, v, a, fused=True))
         what = "AdamW as 13 separate float32 passes (adamw.rs:84-116)"
-    elif w == "cfg3-sgd":
+    elif w.startswith("cfg3-sgd"):
         p32, g32 = gen(1, "f32", GAUSS, 0.02), gen(2, "f32", GAUSS, 1e-3)
         fl = lambda x: float(np.float32(x))
         a = B.SgdArgs(lr=fl(1e-4), momentum=fl(0.9), one_minus_damp=1.0, wd=fl(1e-4), has_wd=1, has_momentum=1,

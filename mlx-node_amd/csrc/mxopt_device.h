@@ -19,6 +19,19 @@ constexpr int kThreads = 256;
 constexpr int kChunk = kChunkElems;
 constexpr int kElemsPerLane = kChunk / kThreads;  // 16
 
+// Every buffer of a table is device memory, but the kernels only see its address as a number read from
+// the table, so the compiler would fall back to FLAT memory instructions (which probe the LDS and scratch
+// apertures as well); naming the global address space gives global_load / global_store.
+#define MXOPT_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ const MXOPT_GLOBAL T* global_ptr(const void* p) {
+  return (const MXOPT_GLOBAL T*)(uintptr_t)p;
+}
+template <class T>
+__device__ __forceinline__ MXOPT_GLOBAL T* global_ptr(void* p) {
+  return (MXOPT_GLOBAL T*)(uintptr_t)p;
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -51,8 +64,8 @@ template <>
 struct Elem<MXOPT_F32> {
   using T = float;
   static constexpr int kBytes = 4;
-  static __device__ __forceinline__ float load(const void* base, uint64_t i) { return ((const float*)base)[i]; }
-  static __device__ __forceinline__ void store(void* base, uint64_t i, float x) { ((float*)base)[i] = x; }
+  static __device__ __forceinline__ float load(const void* base, uint64_t i) { return global_ptr<float>(base)[i]; }
+  static __device__ __forceinline__ void store(void* base, uint64_t i, float x) { global_ptr<float>(base)[i] = x; }
   static __device__ __forceinline__ float round(float x) { return x; }
 };
 template <>
@@ -63,10 +76,10 @@ struct Elem<MXOPT_BF16> {
   static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_bf16_bits(x); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
   static __device__ __forceinline__ float load(const void* base, uint64_t i) {
-    return unpack(((const uint16_t*)base)[i]);
+    return unpack(global_ptr<uint16_t>(base)[i]);
   }
   static __device__ __forceinline__ void store(void* base, uint64_t i, float x) {
-    ((uint16_t*)base)[i] = (uint16_t)pack(x);
+    global_ptr<uint16_t>(base)[i] = (uint16_t)pack(x);
   }
   static __device__ __forceinline__ float round(float x) { return unpack(pack(x)); }
 };
@@ -78,10 +91,10 @@ struct Elem<MXOPT_F16> {
   static __device__ __forceinline__ uint32_t pack(float x) { return f32_to_f16_bits(x); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack(lo) | (pack(hi) << 16); }
   static __device__ __forceinline__ float load(const void* base, uint64_t i) {
-    return unpack(((const uint16_t*)base)[i]);
+    return unpack(global_ptr<uint16_t>(base)[i]);
   }
   static __device__ __forceinline__ void store(void* base, uint64_t i, float x) {
-    ((uint16_t*)base)[i] = (uint16_t)pack(x);
+    global_ptr<uint16_t>(base)[i] = (uint16_t)pack(x);
   }
   static __device__ __forceinline__ float round(float x) { return unpack(pack(x)); }
 };
@@ -92,14 +105,14 @@ struct Elem<MXOPT_F16> {
 template <int DT, int E, bool NT>
 __device__ __forceinline__ void load_group(const void* base, uint64_t off, float (&x)[E]) {
   if constexpr (DT == MXOPT_F32) {
-    const f32x4* q = (const f32x4*)((const float*)base + off);
+    const MXOPT_GLOBAL f32x4* q = global_ptr<f32x4>((const void*)((const float*)base + off));
 #pragma unroll
     for (int k = 0; k < E / 4; ++k) {
       f32x4 t = NT ? __builtin_nontemporal_load(q + k) : q[k];
       x[4 * k + 0] = t.x; x[4 * k + 1] = t.y; x[4 * k + 2] = t.z; x[4 * k + 3] = t.w;
     }
   } else if constexpr (E == 8) {
-    const u32x4* q = (const u32x4*)((const uint16_t*)base + off);
+    const MXOPT_GLOBAL u32x4* q = global_ptr<u32x4>((const void*)((const uint16_t*)base + off));
     u32x4 t = NT ? __builtin_nontemporal_load(q) : *q;
     uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
@@ -108,7 +121,7 @@ __device__ __forceinline__ void load_group(const void* base, uint64_t off, float
       x[2 * k + 1] = Elem<DT>::unpack(w[k] >> 16);
     }
   } else {
-    const u32x2* q = (const u32x2*)((const uint16_t*)base + off);
+    const MXOPT_GLOBAL u32x2* q = global_ptr<u32x2>((const void*)((const uint16_t*)base + off));
     u32x2 t = NT ? __builtin_nontemporal_load(q) : *q;
     x[0] = Elem<DT>::unpack(t.x & 0xffffu); x[1] = Elem<DT>::unpack(t.x >> 16);
     x[2] = Elem<DT>::unpack(t.y & 0xffffu); x[3] = Elem<DT>::unpack(t.y >> 16);
@@ -118,7 +131,7 @@ __device__ __forceinline__ void load_group(const void* base, uint64_t off, float
 template <int DT, int E, bool NT>
 __device__ __forceinline__ void store_group(void* base, uint64_t off, const float (&x)[E]) {
   if constexpr (DT == MXOPT_F32) {
-    f32x4* q = (f32x4*)((float*)base + off);
+    MXOPT_GLOBAL f32x4* q = global_ptr<f32x4>((void*)((float*)base + off));
 #pragma unroll
     for (int k = 0; k < E / 4; ++k) {
       f32x4 t = {x[4 * k + 0], x[4 * k + 1], x[4 * k + 2], x[4 * k + 3]};
@@ -130,13 +143,13 @@ __device__ __forceinline__ void store_group(void* base, uint64_t off, const floa
     t.y = Elem<DT>::pack2(x[2], x[3]);
     t.z = Elem<DT>::pack2(x[4], x[5]);
     t.w = Elem<DT>::pack2(x[6], x[7]);
-    u32x4* q = (u32x4*)((uint16_t*)base + off);
+    MXOPT_GLOBAL u32x4* q = global_ptr<u32x4>((void*)((uint16_t*)base + off));
     if (NT) __builtin_nontemporal_store(t, q); else *q = t;
   } else {
     u32x2 t;
     t.x = Elem<DT>::pack2(x[0], x[1]);
     t.y = Elem<DT>::pack2(x[2], x[3]);
-    u32x2* q = (u32x2*)((uint16_t*)base + off);
+    MXOPT_GLOBAL u32x2* q = global_ptr<u32x2>((void*)((uint16_t*)base + off));
     if (NT) __builtin_nontemporal_store(t, q); else *q = t;
   }
 }
@@ -145,6 +158,13 @@ __device__ __forceinline__ void store_group(void* base, uint64_t off, const floa
 
 __device__ __forceinline__ float clamp_keep_nan(float g, float lo, float hi) {
   float c = fminf(fmaxf(g, lo), hi);
+  return (g != g) ? g : c;
+}
+
+// The same clamp as one median-of-three (v_med3_f32 takes no care of NaN) and a select that puts a NaN back.
+// For lo <= hi and any non-NaN g, including the infinities and both zeros, the median is min(max(g, lo), hi).
+__device__ __forceinline__ float clamp_median_keep_nan(float g, float lo, float hi) {
+  const float c = __builtin_amdgcn_fmed3f(g, lo, hi);
   return (g != g) ? g : c;
 }
 

@@ -48,12 +48,12 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
     auto one_element = [&](uint64_t off) {
       float p = Elem<PD>::load(P, off);
       const float ge = combine(Elem<GD>::load(G, off), kHasG2 ? Elem<G2D>::load(G2P, off) : 0.0f);
-      float m = Math::kM ? M[off] : 0.0f;
-      float v = read_v ? V[off] : 0.0f;
+      float m = Math::kM ? Elem<MXOPT_F32>::load(M, off) : 0.0f;
+      float v = read_v ? Elem<MXOPT_F32>::load(V, off) : 0.0f;
       math(p, ge, m, v, bc1, bc2, flags);
       Elem<OD>::store(PO, off, p);
-      if (Math::kM) M[off] = m;
-      if (use_v) V[off] = v;
+      if (Math::kM) Elem<MXOPT_F32>::store(M, off, m);
+      if (use_v) Elem<MXOPT_F32>::store(V, off, v);
     };
 
     if (cv.fast) {
@@ -114,10 +114,11 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 // add != 0: g_out = g_out + prep(g) (one float32 add, rounded to g_out's dtype by the store): the
 // engines' "clamp, clip-norm, then accumulate" (grpo/engine.rs:636-661) without materialising the
 // clipped gradient.
-template <int GD, int OD, bool NT>
+template <int GD, int OD, bool NT, bool ADD>
 __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __restrict__ T,
                                                              const DevChunk* __restrict__ C, DevTensor one,
-                                                             uint32_t nchunks, DevPrep prep, int add) {
+                                                             uint32_t nchunks, DevPrep prep) {
+  constexpr bool add = ADD;
   constexpr int E = (GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
   if (skip_requested(prep)) return;
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
         if (clamp_then_scale) {
 #pragma unroll
           for (int e = 0; e < E; ++e) {
-            g[j][e] = clamp_keep_nan(g[j][e], pr.pre_lo, pr.pre_hi) * pr.scale;
+            g[j][e] = clamp_median_keep_nan(g[j][e], pr.pre_lo, pr.pre_hi) * pr.scale;
             if (add) g[j][e] = a[j][e] + g[j][e];
           }
         } else {
@@ -309,18 +310,21 @@ bool launch_sgd_plain(int pd, int gd, int od, const Launch& L, float lr_p, float
   return false;
 }
 
+template <int GD, int OD>
+static void launch_transform_t(const Launch& L, const DevPrep& prep, int add) {
+  if (L.nontemporal) {
+    if (add) MXOPT_LAUNCH((transform_kernel<GD, OD, true, true>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, OD, true, false>), L, prep);
+  } else {
+    if (add) MXOPT_LAUNCH((transform_kernel<GD, OD, false, true>), L, prep);
+    else MXOPT_LAUNCH((transform_kernel<GD, OD, false, false>), L, prep);
+  }
+}
+
 template <int GD>
 static bool transform_for_gd(int od, const Launch& L, const DevPrep& prep, int add) {
-  if (od == MXOPT_F32) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, true>), L, prep, add);
-    else MXOPT_LAUNCH((transform_kernel<GD, MXOPT_F32, false>), L, prep, add);
-    return true;
-  }
-  if (od == GD) {
-    if (L.nontemporal) MXOPT_LAUNCH((transform_kernel<GD, GD, true>), L, prep, add);
-    else MXOPT_LAUNCH((transform_kernel<GD, GD, false>), L, prep, add);
-    return true;
-  }
+  if (od == MXOPT_F32) { launch_transform_t<GD, MXOPT_F32>(L, prep, add); return true; }
+  if (od == GD) { launch_transform_t<GD, GD>(L, prep, add); return true; }
   return false;
 }
 

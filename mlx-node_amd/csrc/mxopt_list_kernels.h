@@ -108,12 +108,12 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
 #pragma unroll
       for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? Elem<XD>::load(ps.x[k], off) : 0.0f;
       const float ge = gradient(Elem<GD>::load(G, off), xs);
-      float m = Math::kM ? M[off] : 0.0f;
-      float v = read_v ? V[off] : 0.0f;
+      float m = Math::kM ? Elem<MXOPT_F32>::load(M, off) : 0.0f;
+      float v = read_v ? Elem<MXOPT_F32>::load(V, off) : 0.0f;
       math(p, ge, m, v, bc1, bc2, flags);
       Elem<PD>::store(PO, off, p);
-      if (Math::kM) M[off] = m;
-      if (use_v) V[off] = v;
+      if (Math::kM) Elem<MXOPT_F32>::store(M, off, m);
+      if (use_v) Elem<MXOPT_F32>::store(V, off, v);
     };
 
     if (cv.fast && KMAX > 3) {
@@ -154,6 +154,8 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
         if (Math::kM) load_group<MXOPT_F32, E, false>(M, off, m[j]);
         if (read_v) load_group<MXOPT_F32, E, false>(V, off, v[j]);
       }
+      // One group at a time: its results are stored before the next group's values are unpacked, so that
+      // only the loaded words of the later groups stay live (fewer registers, one more wave per SIMD).
 #pragma unroll
       for (int j = 0; j < U; ++j) {
 #pragma unroll
@@ -163,9 +165,6 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
           for (int k = 0; k < KMAX; ++k) xs[k] = k < kx ? x[k][j][e] : 0.0f;
           math(p[j][e], gradient(g[j][e], xs), m[j][e], v[j][e], bc1, bc2, flags);
         }
-      }
-#pragma unroll
-      for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
         store_group<PD, E, false>(PO, off, p[j]);
         if (Math::kM) store_group<MXOPT_F32, E, false>(M, off, m[j]);

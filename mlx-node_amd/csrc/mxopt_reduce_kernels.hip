@@ -213,7 +213,8 @@ __global__ __launch_bounds__(kThreads) void sumsq_kernel(const DevTensor* __rest
       // instead of two widenings and two multiply-adds; with twice the elements per byte the widening path
       // is bound by instruction issue (6.3 against 6.8 TB/s).  The norm is held to 1e-5, not bitwise; NaN
       // and Inf propagate into the partial sum as before.
-      const u32x4* q = (const u32x4*)((const uint16_t*)Chunk::squared_stream(cv) + cv.start) + tid;
+      const MXOPT_GLOBAL u32x4* q =
+          global_ptr<u32x4>((const void*)((const uint16_t*)Chunk::squared_stream(cv) + cv.start)) + tid;
       u32x4 r[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) r[j] = NT ? __builtin_nontemporal_load(q + j * kThreads) : q[j * kThreads];
