@@ -77,22 +77,22 @@ int mxopt_synchronize(mxopt_ctx* ctx);
 int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value);
 int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
 
-/* ---- HBM placement -------------------------------------------------------------------
- * Kernels that walk several streams at once (every update kernel here) run 5 - 12 % faster on this
- * part in most runs when the buffers' physical pages are interleaved with unrelated memory instead of
- * lying in one compact run -- what a process gets by default when it is the first to use the GPU.  The library
- * never owns the caller's buffers, so it cannot place them; this pair lets a host do it at start-up:
+/* ---- HBM placement (the older, luck-based way; see the region-interleaved pool below) -------------
+ * Why placement matters at all is told at the pool: device memory consists of three physical regions and
+ * a kernel that reads and writes wants its traffic in at least two of them.  This pair only raises the odds
+ * of that for hosts that cannot route their allocations through a pool:
  *
  *   mxopt_hbm_spread_begin(ctx, 0, 0, &s);    all free device memory is taken in blocks, then two of
  *   ... allocate parameters, moments, ...      every three blocks are released: what is allocated now
  *   mxopt_hbm_spread_end(s);                   fills those gaps; end() releases the rest
  *
- * block_bytes = 0: 64 MiB; keep_one_in = 0: every third block is kept (>= 2: every keep_one_in-th).
- * The defaults suit buffer sets of tens of GB (Qwen3-1.7B ... 8B lists); the 0.6B list wanted 256 MiB
- * blocks, so a host with unusual sizes should time one step per candidate.
- * Between the two calls about (1 - 1/keep_one_in) of the free memory can be allocated.  Both calls
- * synchronise with the device and are meant for start-up, not for the training loop.  No counterpart
- * in the reference. */
+ * What is allocated in between lands in pieces all over the free memory instead of one compact run, which
+ * usually -- not always, the driver decides -- means pieces of more than one region (measured over 17 fresh
+ * processes on the Qwen3-8B list: 79.7 - 86.2 ms per step, against 84.6 - 85.8 ms without and 77.1 ms from
+ * the pool).  block_bytes = 0: 64 MiB; keep_one_in = 0: every third block is kept (>= 2: every
+ * keep_one_in-th).  Between the two calls about (1 - 1/keep_one_in) of the free memory can be allocated.
+ * Both calls synchronise with the device and are meant for start-up, not for the training loop.  No
+ * counterpart in the reference. */
 typedef struct mxopt_hbm_spread mxopt_hbm_spread;
 int mxopt_hbm_spread_begin(mxopt_ctx* ctx, size_t block_bytes, int keep_one_in, mxopt_hbm_spread** out);
 int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
@@ -135,13 +135,42 @@ typedef struct mxopt_hbm_pool_info {
   double scan_seconds;                                   /* ... and timing probes to find the regions */
   int32_t probes;                                        /* probe measurements taken */
   int32_t reserved2_;
+  uint64_t interleaved_bytes;  /* arena bytes [0, this) alternate between regions chunk by chunk; what lies behind
+                                  comes from one region at a time (MXOPT_HBM_ONE_REGION allocations) */
 } mxopt_hbm_pool_info;
 int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
                           mxopt_hbm_pool** out);
+/* The same with every knob.  Zero-fill the struct first; a field left 0 takes its default.
+ * While it scans, creation holds the device's free memory (all of it by default: memory far from what a small
+ * allocation would get can only be reached by holding what lies in between) and times kernels on it, so the
+ * process needs the GPU to itself for those seconds: another process's, or another thread's, allocation can
+ * fail with out-of-memory meanwhile, and a co-tenant's traffic disturbs the timing.  max_take_bytes bounds what
+ * is held (never less than the arena itself); with a bound below the free memory the scan sees less, possibly
+ * one region only.  slab_bytes is the unit of classification (a power of two in [128 MiB, 4 GiB], default
+ * 1 GiB): smaller slabs follow fragmented free memory more closely at about the same scan time. */
+typedef struct mxopt_hbm_pool_options {
+  size_t capacity_bytes;
+  size_t chunk_bytes;      /* 0: 64 MiB */
+  int    max_regions;      /* 0: all regions found */
+  int    reserved_;
+  size_t max_take_bytes;   /* 0: all free memory but 1 GiB */
+  size_t slab_bytes;       /* 0: 1 GiB */
+} mxopt_hbm_pool_options;
+int mxopt_hbm_pool_create_ex(mxopt_ctx* ctx, const mxopt_hbm_pool_options* options, mxopt_hbm_pool** out);
 /* Refused (MXOPT_ERR_INVALID_ARG, nothing happens) while allocations from the pool are live: their memory would
  * be unmapped under whoever still uses it. */
 int mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool);
 int mxopt_hbm_pool_alloc(mxopt_hbm_pool* pool, size_t bytes, void** out);
+/* Where in the arena: MXOPT_HBM_INTERLEAVED (what mxopt_hbm_pool_alloc gives) for buffers a kernel writes or
+ * reads together with ones it writes; MXOPT_HBM_ONE_REGION for buffers that are only ever read (gradients):
+ * the part of the arena behind the alternation, when the arena is large enough to have one (info.capacity_bytes
+ * > info.interleaved_bytes), else anywhere.  Read-only passes are 3 % (two regions) to 10 % (three) faster on
+ * memory of one region. */
+enum { MXOPT_HBM_INTERLEAVED = 0, MXOPT_HBM_ONE_REGION = 1 };
+int mxopt_hbm_pool_alloc_kind(mxopt_hbm_pool* pool, size_t bytes, int kind, void** out);
+/* Gives the range back.  Like every pool free (the hook's and the library's own included) this does NOT
+ * synchronise with the device the way hipFree does: a caller that frees memory which kernels on another stream
+ * may still use, or reuses it from another stream, orders that itself. */
 int mxopt_hbm_pool_free(mxopt_hbm_pool* pool, void* ptr);
 int mxopt_hbm_pool_owns(const mxopt_hbm_pool* pool, const void* ptr);   /* 1 if ptr lies inside the arena */
 int mxopt_hbm_pool_get_info(mxopt_hbm_pool* pool, mxopt_hbm_pool_info* out);
@@ -154,21 +183,9 @@ int mxopt_set_state_pool(mxopt_ctx* ctx, mxopt_hbm_pool* pool);
  * signatures): allocations on the target pool's device come from its arena while it has room and from
  * hipMalloc otherwise; frees find their way back by address. */
 int mxopt_hbm_pool_set_hook_target(mxopt_hbm_pool* pool);
+int mxopt_hbm_pool_set_hook_kind(int kind);   /* kind of the hook's allocations from now on (process-wide) */
 void* mxopt_hbm_pool_hook_alloc(ptrdiff_t size, int device, void* stream);
 void mxopt_hbm_pool_hook_free(void* ptr, ptrdiff_t size, int device, void* stream);
-
-/* ---- bare streaming probes ------------------------------------------------------------
- * The measured ceilings the update kernels are compared with: float32 buffers of n_elems elements
- * (a positive multiple of 4096, 16-byte aligned), no table, no tails, no arithmetic to speak of.
- *   MXOPT_PROBE_READ   reads a                       MXOPT_PROBE_WRITE  writes a
- *   MXOPT_PROBE_COPY   reads a, writes b             MXOPT_PROBE_MIX43  reads a, b, c, d and writes a, c, d
- * (MIX43 is float32 AdamW's byte mix, 28 B/elem.)  One launch on the context's stream. */
-enum { MXOPT_PROBE_READ = 0, MXOPT_PROBE_WRITE = 1, MXOPT_PROBE_COPY = 2, MXOPT_PROBE_MIX43 = 3 };
-int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n_elems);
-/* The byte mix of the update over k un-summed 16-bit micro-batches (mxopt_adam_with_pending_list) without its
- * arithmetic: g[0..k) and p are 2-byte streams of n_elems elements, m and v 4-byte ones; p, m and v are
- * rewritten in place (2k + 20 B/elem).  k in [1, 8], n_elems a positive multiple of 4096. */
-int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k, uint64_t n_elems);
 
 /* ---- tensor table ------------------------------------------------------------------
  * One descriptor per tensor.  Which fields a kernel reads is listed at that kernel;
@@ -446,31 +463,6 @@ int mxopt_accumulate_norm_only(mxopt_ctx* ctx, const mxopt_table* t, const mxopt
  * add, rounded once to dtype(g_out).  Honours prep->d_skip_if_nonzero: a micro-batch flagged
  * non-finite by mxopt_global_norm leaves the buffer untouched (grpo/engine.rs:561-562). */
 int mxopt_accumulate_transformed(mxopt_ctx* ctx, const mxopt_table* t, int first, const mxopt_grad_prep* prep);
-
-/* ---- synthetic data for benchmarks and parity tests ----------------------------------
- * out[i] = f(hash(seed, first_index + i)), hash = splitmix64 finaliser of seed + (index+1)*golden:
- *   MXOPT_SYNTH_NORMAL          (sum of four 16-bit fields of the hash - 131070) * f32(a / sqrt((65536^2-1)/3)):
- *                               mean 0, standard deviation a, bell shaped, |x| <= 3.46 a
- *   MXOPT_SYNTH_NORMAL_OUTLIERS the same, and on average every 100th element (second hash % 100 == 0) times f32(b)
- *   MXOPT_SYNTH_UNIFORM         f32(top 24 bits) * f32((b - a) / 2^24) + f32(a): uniform on [a, b)
- *   MXOPT_SYNTH_GAUSSIAN        normal with standard deviation a and true tails: bit 63 of the hash is the sign,
- *                               bits 31..62 a uniform u that stands for the two-sided tail probability
- *                               (u + 0.5) / 2^32 of |x|; u is split like a floating-point number (leading zeros:
- *                               octave, next 5 bits: sub-interval, 16 more bits: linear interpolation) into a
- *                               committed 32 x 33 table of float32 quantiles, so |x| reaches 6.3 a with the same
- *                               relative resolution everywhere; then * f32(a)
- *   MXOPT_SYNTH_GAUSSIAN_OUTLIERS  the same, and on average every 100th element times f32(b)
- * then rounded once to out's dtype.  Only integer arithmetic, exact conversions and at most two rounded
- * float32 operations (three and a table look-up for the Gaussian modes): a host program regenerates any slice bit for bit (as the CPU checker in this
- * repository does), so inputs never have to be copied or read back to compare results at full size.
- * No counterpart in the reference (its tests build inputs on the host). */
-enum { MXOPT_SYNTH_NORMAL = 0, MXOPT_SYNTH_NORMAL_OUTLIERS = 1, MXOPT_SYNTH_UNIFORM = 2, MXOPT_SYNTH_GAUSSIAN = 3,
-       MXOPT_SYNTH_GAUSSIAN_OUTLIERS = 4 };
-int mxopt_fill_synthetic(mxopt_ctx* ctx, void* out, uint64_t n, int dtype, uint64_t seed, uint64_t first_index,
-                         int distribution, double a, double b);
-/* The stream key used by this repository's benchmark and tests:
- * splitmix64(seed ^ config ^ step << 32 ^ micro_batch << 48 ^ tensor_index).  Host only. */
-uint64_t mxopt_synthetic_key(uint64_t seed, uint64_t config, uint64_t step, uint64_t micro_batch, uint64_t tensor_index);
 
 /* ---- small host<->device helpers (each synchronises the context's stream) --------- */
 int mxopt_read_norm_result(mxopt_ctx* ctx, const mxopt_norm_result* d_result, mxopt_norm_result* host_out);

@@ -17,6 +17,8 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
+# mxopt_diagnostics.h (probes, data generator, the pool scan on synthetic rates) is for benchmarks and tests only:
+# no call site of the reference binds it, so it gets no Rust declarations.
 HEADERS = ["mxopt.h", "mxopt_optimizers.h", "mxopt_engine.h"]
 OUT = os.path.join(HERE, "mxopt_sys.rs")
 

@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmxopt.so")
 
 SOURCES = ["mxopt_kernels.hip", "mxopt_reduce_kernels.hip", "mxopt_list_kernels.hip", "mxopt_list_kernels_sgd_rmsprop.hip", "mxopt_hbm_pool.hip",
-           "mxopt_api.cpp",
+           "mxopt_api.cpp", "mxopt_region_scan.cpp",
            "mxopt_optimizers.cpp", "mxopt_engine.cpp", "mxopt_checkpoint.cpp"]
 
 FLAGS = [

@@ -23,6 +23,7 @@
 #include <vector>
 
 #include "mxopt_internal.h"
+#include "mxopt_region_scan.h"
 
 namespace mxopt {
 
@@ -182,6 +183,7 @@ struct mxopt_hbm_pool {
   char* base = nullptr;
   size_t capacity = 0;
   std::map<size_t, size_t> free_list;                    // offset -> bytes, coalesced
+  size_t one_region_begin = 0;                           // arena bytes from here on lie in one region at a time
   std::unordered_map<size_t, size_t> live;               // offset -> bytes
   std::mutex mu;
   mxopt_hbm_pool_info info{};
@@ -190,7 +192,9 @@ struct mxopt_hbm_pool {
 namespace {
 
 constexpr size_t kAlign = 512;
-constexpr size_t kSlabChunksBytes = (size_t)1 << 30;  // chunks are classified in groups of this many bytes
+constexpr size_t kSlabChunksBytes = (size_t)1 << 30;  // chunks are classified in groups of this many bytes by default
+// The driver limits the live allocations of a process (about 60 000 were seen to succeed) and maps fewer still.
+constexpr size_t kMaxChunks = 24000;
 
 struct Builder {  // everything pool creation holds until it either succeeds or fails
   mxopt_ctx* ctx;
@@ -236,6 +240,7 @@ std::mutex g_pools_mu;
 std::vector<mxopt_hbm_pool*> g_pools;
 std::mutex g_hook_mu;
 mxopt_hbm_pool* g_hook_pool = nullptr;
+int g_hook_kind = MXOPT_HBM_INTERLEAVED;
 
 mxopt_hbm_pool* pool_of(const void* ptr) {
   std::lock_guard<std::mutex> all(g_pools_mu);
@@ -289,12 +294,28 @@ int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* cons
 
 int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
                           mxopt_hbm_pool** out) {
+  mxopt_hbm_pool_options o;
+  std::memset(&o, 0, sizeof o);
+  o.capacity_bytes = capacity_bytes;
+  o.chunk_bytes = chunk_bytes;
+  o.max_regions = max_regions;
+  return mxopt_hbm_pool_create_ex(ctx, &o, out);
+}
+
+int mxopt_hbm_pool_create_ex(mxopt_ctx* ctx, const mxopt_hbm_pool_options* options, mxopt_hbm_pool** out) {
   const char* op = "mxopt_hbm_pool_create";
-  if (!ctx || !out) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
+  if (!ctx || !out || !options) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null argument");
   *out = nullptr;
+  const size_t capacity_bytes = options->capacity_bytes;
+  size_t chunk_bytes = options->chunk_bytes;
+  const int max_regions = options->max_regions;
+  size_t slab_bytes = options->slab_bytes ? options->slab_bytes : kSlabChunksBytes;
   if (chunk_bytes == 0) chunk_bytes = (size_t)64 << 20;
   if (chunk_bytes < ((size_t)2 << 20) || (chunk_bytes & (chunk_bytes - 1)) || chunk_bytes > kSlabChunksBytes)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": chunk_bytes must be a power of two in [2 MiB, 1 GiB]");
+  if ((slab_bytes & (slab_bytes - 1)) || slab_bytes < ((size_t)128 << 20) || slab_bytes > ((size_t)4 << 30))
+    return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": slab_bytes must be a power of two in [128 MiB, 4 GiB]");
+  if (slab_bytes < chunk_bytes) slab_bytes = chunk_bytes;
   if (capacity_bytes == 0) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": capacity_bytes is 0");
   if (max_regions < 0) return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": max_regions is negative");
   const auto t_begin = std::chrono::steady_clock::now();
@@ -304,15 +325,18 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
   HIP_TRY(ctx, hipMemGetInfo(&free_b, &total_b));
   const size_t margin = (size_t)1 << 30;  // left to the runtime
   const size_t want_chunks = (capacity_bytes + chunk_bytes - 1) / chunk_bytes;
-  const size_t avail_chunks = free_b > margin ? (free_b - margin) / chunk_bytes : 0;
+  size_t avail_chunks = free_b > margin ? (free_b - margin) / chunk_bytes : 0;
   if (want_chunks > avail_chunks)
     return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": " + std::to_string(capacity_bytes >> 20) + " MiB wanted, " +
                                         std::to_string(free_b >> 20) + " MiB free");
-  if (avail_chunks > 24000)  // the driver limits the number of live allocations of a process, and maps fewer still
+  // A caller that shares the device bounds what creation may hold while it scans (never less than the arena).
+  if (options->max_take_bytes)
+    avail_chunks = std::min(avail_chunks, std::max(want_chunks, options->max_take_bytes / chunk_bytes));
+  if (avail_chunks > kMaxChunks)  // the driver limits the number of live allocations of a process, and maps fewer still
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": chunk_bytes too small for this much free memory");
 
-  // 1. All free memory as physical chunks: memory far from what a small allocation would get can
-  //    only be reached by holding what lies in between.
+  // 1. The free memory as physical chunks: memory far from what a small allocation would get can only be
+  //    reached by holding what lies in between.
   Builder b{ctx};
   const hipMemAllocationProp prop = device_prop(ctx->device);
   b.all.reserve(avail_chunks);
@@ -326,42 +350,50 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
   }
   b.released.assign(b.all.size(), 0);
   const auto t_created = std::chrono::steady_clock::now();
-  int probes = 0;
   if (b.all.size() < want_chunks)
     return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": the driver handed out fewer chunks than the capacity needs");
 
-  // 2. Which chunks share a region?  Chunks are judged in creation-order groups of 1 GiB ("slabs"):
-  //    the 4-read/3-write probe runs with two of its streams in a reference slab and two in the slab
-  //    under test; it is slow when both lie in one region.
-  const size_t per_slab = kSlabChunksBytes / chunk_bytes;
+  // 2. Which chunks share a region?  Chunks are judged in creation-order groups ("slabs"): the 4-read/3-write
+  //    probe runs with two of its streams in a reference slab and two in the slab under test; it is slow when
+  //    both lie in one region.  The decisions are classify_slabs' (mxopt_region_scan.cpp), this function only
+  //    measures.
+  const size_t per_slab = slab_bytes / chunk_bytes;
   const size_t nslab = b.all.size() / per_slab;
-  std::vector<int> slab_region(nslab, 0);
-  int nregions = 1;
-  double same_gbps = 0.0, cross_gbps = 0.0;
-  if (nslab >= 4) {
+  ScanResult scan;
+  scan.slab_region.assign(nslab, 0);
+  const ScanLimits limits;
+  if (nslab >= limits.min_region_slabs) {
     const hipMemAccessDesc acc = rw_access(ctx->device);
-    b.probe_bytes = 2 * kSlabChunksBytes;
+    b.probe_bytes = 2 * slab_bytes;
     HIP_TRY(ctx, hipMemAddressReserve(&b.probe_va, b.probe_bytes, 0, nullptr, 0));
     HIP_TRY(ctx, hipEventCreate(&b.ev0));
     HIP_TRY(ctx, hipEventCreate(&b.ev1));
     char* va_ref = (char*)b.probe_va;
-    char* va_x = va_ref + kSlabChunksBytes;
-    const uint64_t stream_elems = kSlabChunksBytes / 2 / 4;  // two streams per slab
+    char* va_x = va_ref + slab_bytes;
+    const uint64_t stream_elems = slab_bytes / 2 / 4;  // two streams per slab
     auto map_slab = [&](char* va, size_t slab) -> hipError_t {
       for (size_t k = 0; k < per_slab; ++k) {
         hipError_t e = hipMemMap(va + k * chunk_bytes, chunk_bytes, 0, b.all[slab * per_slab + k], 0);
         if (e != hipSuccess) return e;
       }
-      return hipMemSetAccess(va, kSlabChunksBytes, &acc, 1);
+      return hipMemSetAccess(va, slab_bytes, &acc, 1);
     };
-    // Rate of the probe with streams p, g in the (already mapped) reference slab and m, v in slab x.
-    auto probe_against_ref = [&](int x, double* out) -> int {
+    int mapped_ref = -1;
+    // Rate of the probe with streams p, g in the reference slab and m, v in slab x.
+    const SlabProbe probe = [&](int ref, int x, double* out_gbps) -> int {
+      if (mapped_ref != ref) {
+        if (mapped_ref >= 0) HIP_TRY(ctx, hipMemUnmap(va_ref, slab_bytes));
+        mapped_ref = -1;
+        hipError_t me = map_slab(va_ref, (size_t)ref);
+        if (me != hipSuccess) return hip_fail(ctx, me, "mxopt_hbm_pool_create: mapping a slab");
+        mapped_ref = ref;
+      }
       hipError_t e = map_slab(va_x, (size_t)x);
       if (e != hipSuccess) return hip_fail(ctx, e, "mxopt_hbm_pool_create: mapping a slab");
       void* p = va_ref;
-      void* g = va_ref + kSlabChunksBytes / 2;
+      void* g = va_ref + slab_bytes / 2;
       void* m = va_x;
-      void* v = va_x + kSlabChunksBytes / 2;
+      void* v = va_x + slab_bytes / 2;
       int rc = launch_probe(ctx, MXOPT_PROBE_MIX43, p, g, m, v, stream_elems);
       if (rc) return rc;
       HIP_TRY(ctx, hipEventRecord(b.ev0, ctx->stream));
@@ -371,133 +403,24 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
       HIP_TRY(ctx, hipEventSynchronize(b.ev1));
       float ms = 0.f;
       HIP_TRY(ctx, hipEventElapsedTime(&ms, b.ev0, b.ev1));
-      *out = 2.0 * 7.0 * (double)(kSlabChunksBytes / 2) / 1e9 / ((double)ms * 1e-3);
-      ++probes;
-      HIP_TRY(ctx, hipMemUnmap(va_x, kSlabChunksBytes));
+      *out_gbps = 2.0 * 7.0 * (double)(slab_bytes / 2) / 1e9 / ((double)ms * 1e-3);
+      HIP_TRY(ctx, hipMemUnmap(va_x, slab_bytes));
       return MXOPT_OK;
     };
-    std::vector<int> todo(nslab);
-    for (size_t i = 0; i < nslab; ++i) todo[i] = (int)i;
-    std::vector<double> rate(nslab);
-    double abs_thr = 0.0;  // rate that separates "same region" from "another region", once one scan has shown both
-    int region = 0, attempts = 0;
-    while (!todo.empty() && region < MXOPT_HBM_MAX_REGIONS) {
-      if (todo.size() < 4) {  // a few boundary slabs are no region of their own
-        for (int x : todo) slab_region[x] = std::max(region - 1, 0);
-        todo.clear();
-        break;
-      }
-      // The reference must lie inside one region; a slab that straddles a boundary makes everything look
-      // fast.  First try the first slab, after a suspicious scan one further into the list.
-      const size_t ref_pos = std::min(todo.size() - 1, todo.size() * (size_t)attempts / 4);
-      const int ref = todo[ref_pos];
-      std::vector<int> others;
-      for (size_t i = 0; i < todo.size(); ++i) if (i != ref_pos) others.push_back(todo[i]);
-      hipError_t me = map_slab(va_ref, (size_t)ref);
-      if (me != hipSuccess) return hip_fail(ctx, me, "mxopt_hbm_pool_create: mapping a slab");
-      // Coarse scan (creation order is close to physical order, regions are long runs), refined below
-      // wherever two scanned neighbours disagree.
-      const size_t stride = 4;
-      std::vector<char> probed(others.size(), 0);
-      double lo = 1e30, hi = 0.0;
-      auto scan = [&](size_t k) -> int {
-        if (probed[k]) return MXOPT_OK;
-        int rc = probe_against_ref(others[k], &rate[others[k]]);
-        if (rc) return rc;
-        probed[k] = 1;
-        lo = std::min(lo, rate[others[k]]);
-        hi = std::max(hi, rate[others[k]]);
-        return MXOPT_OK;
-      };
-      for (size_t k = 0; k < others.size(); k += stride) { int rc = scan(k); if (rc) return rc; }
-      { int rc = scan(others.size() - 1); if (rc) return rc; }
-      const bool uniform = hi < lo * 1.07;
-      const double level = 0.5 * (lo + hi);
-      if (uniform) {
-        HIP_TRY(ctx, hipMemUnmap(va_ref, kSlabChunksBytes));
-        const bool straddler = abs_thr > 0.0 ? level > abs_thr : attempts < 2;
-        if (straddler && attempts < 3) {
-          if (abs_thr > 0.0) {  // known to be fast against everything: a boundary slab, lumped with its predecessors
-            slab_region[ref] = std::max(region - 1, 0);
-            todo.erase(todo.begin() + (ptrdiff_t)ref_pos);
-          }
-          ++attempts;
-          continue;
-        }
-        for (int x : todo) slab_region[x] = region;  // they all share the reference's region
-        if (abs_thr == 0.0) same_gbps = level;
-        ++region;
-        todo.clear();
-        break;
-      }
-      const double thr = abs_thr > 0.0 ? abs_thr : level;
-      for (size_t k = 0; k + 1 < others.size();) {  // refine between scanned neighbours that disagree
-        size_t k2 = k + 1;
-        while (!probed[k2]) ++k2;
-        if ((rate[others[k]] < thr) != (rate[others[k2]] < thr))
-          for (size_t q = k + 1; q < k2; ++q) { int rc = scan(q); if (rc) return rc; }
-        k = k2;
-      }
-      HIP_TRY(ctx, hipMemUnmap(va_ref, kSlabChunksBytes));
-      if (log_level() >= 2) {
-        std::string line = "hbm pool scan: reference slab " + std::to_string(ref) + ", threshold " + std::to_string((int)thr) + ":";
-        for (size_t k = 0; k < others.size(); ++k)
-          if (probed[k]) line += " " + std::to_string(others[k]) + "=" + std::to_string((int)rate[others[k]]);
-        std::fprintf(stderr, "mxopt: %s\n", line.c_str());  // longer than log_line's buffer
-      }
-      if (abs_thr == 0.0) { abs_thr = thr; same_gbps = lo; cross_gbps = hi; }
-      std::vector<int> rest;
-      bool same = true;
-      for (size_t k = 0; k < others.size(); ++k) {
-        if (probed[k]) same = rate[others[k]] < thr;  // slabs between two agreeing neighbours inherit
-        if (same) slab_region[others[k]] = region;
-        else rest.push_back(others[k]);
-      }
-      slab_region[ref] = region;
-      ++region;
-      attempts = 0;
-      todo.swap(rest);
-    }
-    nregions = std::max(region, 1);
-    for (int s : todo) slab_region[s] = nregions - 1;  // more groups than MXOPT_HBM_MAX_REGIONS: lumped together
+    const int rc = classify_slabs(nslab, probe, limits, &scan);
+    if (mapped_ref >= 0) (void)hipMemUnmap(va_ref, slab_bytes);
+    if (rc) return rc;
+    if (log_level() >= 2) std::fprintf(stderr, "mxopt: hbm pool %s", scan.trace.c_str());  // longer than log_line's buffer
   }
-
+  const int nregions = scan.regions;
+  const double same_gbps = scan.same_region_gbps, cross_gbps = scan.cross_region_gbps;
+  const int probes = scan.probes;
   const auto t_scanned = std::chrono::steady_clock::now();
 
   // 3. The arena: consecutive chunks alternate between the regions for as long as each has chunks.
-  std::vector<std::vector<size_t>> by_region(nregions);
-  for (size_t i = 0; i < b.all.size(); ++i) {
-    const size_t slab = i / per_slab;
-    by_region[slab < nslab ? slab_region[slab] : slab_region.empty() ? 0 : slab_region[nslab - 1]].push_back(i);
-  }
-  // Regions by free memory, largest first.  Groups holding under a tenth of the chunks are leftovers of the
-  // scan (slabs whose chunks straddle regions when the free memory was fragmented): they serve last and
-  // are not counted.  With max_regions, only that many of the largest take part in the alternation.
-  std::vector<int> rank(nregions);
-  for (int r = 0; r < nregions; ++r) rank[r] = r;
-  std::stable_sort(rank.begin(), rank.end(), [&](int a, int c) { return by_region[a].size() > by_region[c].size(); });
-  int real_regions = 0;
-  for (int k = 0; k < nregions; ++k)
-    if (by_region[rank[k]].size() * 10 >= b.all.size()) ++real_regions;
-  real_regions = std::max(real_regions, 1);
-  const int active = max_regions > 0 ? std::min(max_regions, real_regions) : real_regions;
-  std::vector<size_t> order;
-  order.reserve(want_chunks);
-  std::vector<size_t> next(nregions, 0);
-  for (int lo_rank = 0; lo_rank < nregions && order.size() < want_chunks;) {
-    const int hi_rank = lo_rank == 0 ? active : nregions;  // first the alternation, then whatever is left
-    for (bool any = true; any && order.size() < want_chunks;) {
-      any = false;
-      for (int k = lo_rank; k < hi_rank && order.size() < want_chunks; ++k) {
-        const int r = rank[k];
-        if (next[r] < by_region[r].size()) {
-          order.push_back(by_region[r][next[r]++]);
-          any = true;
-        }
-      }
-    }
-    lo_rank = hi_rank;
-  }
+  const ArenaPlan plan = plan_arena(scan.slab_region, nregions, per_slab, b.all.size(), want_chunks, max_regions);
+  const std::vector<size_t>& order = plan.order;
+  const int real_regions = plan.real_regions;
   if (order.size() < want_chunks) return fail(ctx, MXOPT_ERR_OOM, std::string(op) + ": ran out of chunks");
 
   mxopt_hbm_pool* pool = new (std::nothrow) mxopt_hbm_pool();
@@ -529,13 +452,16 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
     b.released[order[k]] = 1;  // now owned by the pool; everything else goes back to the driver with `b`
   }
   pool->free_list[0] = pool->capacity;
+  // With one region in the alternation nothing is interleaved: the whole arena is "one region at a time".
+  pool->one_region_begin = plan.active > 1 ? plan.interleaved_chunks * chunk_bytes : 0;
   mxopt_hbm_pool_info& info = pool->info;
   info.capacity_bytes = pool->capacity;
   info.chunk_bytes = chunk_bytes;
   info.regions = real_regions;
+  info.interleaved_bytes = pool->one_region_begin;
   for (int k = 0; k < nregions && k < MXOPT_HBM_MAX_REGIONS; ++k) {  // largest first; entries past `regions` are leftovers
-    info.region_free_bytes[k] = by_region[rank[k]].size() * chunk_bytes;
-    info.region_arena_bytes[k] = next[rank[k]] * chunk_bytes;
+    info.region_free_bytes[k] = plan.region_chunks[(size_t)k] * chunk_bytes;
+    info.region_arena_bytes[k] = plan.region_used[(size_t)k] * chunk_bytes;
   }
   info.probe_same_region_gbps = same_gbps;
   info.probe_cross_region_gbps = cross_gbps;
@@ -591,24 +517,37 @@ int mxopt_hbm_pool_destroy(mxopt_hbm_pool* pool) {
   return MXOPT_OK;
 }
 
-// First fit; NULL when no free range is large enough.
-static void* pool_try_alloc(mxopt_hbm_pool* pool, size_t bytes) {
+// First fit; NULL when no free range is large enough.  MXOPT_HBM_ONE_REGION looks at the part of the arena that
+// lies behind the alternation first (consecutive chunks of one region), then anywhere.
+static void* pool_try_alloc(mxopt_hbm_pool* pool, size_t bytes, int kind = MXOPT_HBM_INTERLEAVED) {
   const size_t need = std::max<size_t>((bytes + kAlign - 1) / kAlign * kAlign, kAlign);
   std::lock_guard<std::mutex> lock(pool->mu);
-  for (auto it = pool->free_list.begin(); it != pool->free_list.end(); ++it) {
-    if (it->second < need) continue;
-    const size_t off = it->first, left = it->second - need;
-    pool->free_list.erase(it);
-    if (left) pool->free_list[off + need] = left;
-    pool->live[off] = need;
-    return pool->base + off;
+  const size_t zone = kind == MXOPT_HBM_ONE_REGION ? pool->one_region_begin : 0;
+  for (int pass = zone ? 0 : 1; pass < 2; ++pass) {
+    const size_t from = pass == 0 ? zone : 0;
+    for (auto it = pool->free_list.begin(); it != pool->free_list.end(); ++it) {
+      const size_t off = it->first, len = it->second;
+      const size_t begin = std::max(off, from);
+      if (begin >= off + len || off + len - begin < need) continue;
+      pool->free_list.erase(it);
+      if (begin > off) pool->free_list[off] = begin - off;
+      if (off + len > begin + need) pool->free_list[begin + need] = off + len - begin - need;
+      pool->live[begin] = need;
+      return pool->base + begin;
+    }
   }
   return nullptr;
 }
 
 int mxopt_hbm_pool_alloc(mxopt_hbm_pool* pool, size_t bytes, void** out) {
+  return mxopt_hbm_pool_alloc_kind(pool, bytes, MXOPT_HBM_INTERLEAVED, out);
+}
+
+int mxopt_hbm_pool_alloc_kind(mxopt_hbm_pool* pool, size_t bytes, int kind, void** out) {
   if (!pool || !out) return fail(pool ? pool->ctx : nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_alloc: null argument");
-  *out = pool_try_alloc(pool, bytes);
+  if (kind != MXOPT_HBM_INTERLEAVED && kind != MXOPT_HBM_ONE_REGION)
+    return fail(pool->ctx, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_alloc: unknown kind");
+  *out = pool_try_alloc(pool, bytes, kind);
   if (*out) return MXOPT_OK;
   return fail(pool->ctx, MXOPT_ERR_OOM, "mxopt_hbm_pool_alloc: the arena has no free range of " + std::to_string(bytes) + " bytes");
 }
@@ -654,6 +593,42 @@ int mxopt_hbm_pool_get_info(mxopt_hbm_pool* pool, mxopt_hbm_pool_info* out) {
   return MXOPT_OK;
 }
 
+int mxopt_hbm_classify_regions(int n_slabs, mxopt_slab_probe_fn probe, void* user, int* slab_region,
+                               mxopt_hbm_scan_report* report) {
+  if (n_slabs < 0 || !probe || (n_slabs && !slab_region))
+    return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_classify_regions: null argument");
+  ScanResult r;
+  const SlabProbe fn = [&](int ref, int x, double* gbps) { return probe(user, ref, x, gbps); };
+  const int rc = classify_slabs((size_t)n_slabs, fn, ScanLimits{}, &r);
+  if (rc) return rc;
+  for (int i = 0; i < n_slabs; ++i) slab_region[i] = r.slab_region[(size_t)i];
+  if (report) {
+    report->regions = r.regions;
+    report->probes = r.probes;
+    report->same_region_gbps = r.same_region_gbps;
+    report->cross_region_gbps = r.cross_region_gbps;
+  }
+  return MXOPT_OK;
+}
+
+int mxopt_hbm_plan_arena(int n_slabs, const int* slab_region, int regions, int chunks_per_slab, int total_chunks,
+                         int want_chunks, int max_regions, int* order, mxopt_hbm_arena_report* report) {
+  if (n_slabs < 0 || chunks_per_slab < 1 || total_chunks < 0 || want_chunks < 0 || (n_slabs && !slab_region) ||
+      (want_chunks && !order))
+    return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_plan_arena: bad argument");
+  const std::vector<int> sr(slab_region, slab_region + n_slabs);
+  const ArenaPlan plan = plan_arena(sr, regions, (size_t)chunks_per_slab, (size_t)total_chunks, (size_t)want_chunks, max_regions);
+  if (plan.order.size() < (size_t)want_chunks)
+    return fail(nullptr, MXOPT_ERR_OOM, "mxopt_hbm_plan_arena: fewer chunks than wanted");
+  for (int i = 0; i < want_chunks; ++i) order[i] = (int)plan.order[(size_t)i];
+  if (report) {
+    report->real_regions = plan.real_regions;
+    report->active_regions = plan.active;
+    report->interleaved_chunks = (int)plan.interleaved_chunks;
+  }
+  return MXOPT_OK;
+}
+
 int mxopt_set_state_pool(mxopt_ctx* ctx, mxopt_hbm_pool* pool) {
   if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_set_state_pool: null context");
   if (pool && pool->ctx->device != ctx->device)
@@ -670,15 +645,25 @@ int mxopt_hbm_pool_set_hook_target(mxopt_hbm_pool* pool) {
   return MXOPT_OK;
 }
 
+int mxopt_hbm_pool_set_hook_kind(int kind) {
+  if (kind != MXOPT_HBM_INTERLEAVED && kind != MXOPT_HBM_ONE_REGION)
+    return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_hbm_pool_set_hook_kind: unknown kind");
+  std::lock_guard<std::mutex> lock(g_hook_mu);
+  g_hook_kind = kind;
+  return MXOPT_OK;
+}
+
 void* mxopt_hbm_pool_hook_alloc(ptrdiff_t size, int device, void* stream) {
   (void)stream;
   mxopt_hbm_pool* pool;
+  int kind;
   {
     std::lock_guard<std::mutex> lock(g_hook_mu);
     pool = g_hook_pool;
+    kind = g_hook_kind;
   }
   void* p = nullptr;
-  if (pool && pool->ctx->device == device && (p = pool_try_alloc(pool, (size_t)size)) != nullptr) return p;
+  if (pool && pool->ctx->device == device && (p = pool_try_alloc(pool, (size_t)size, kind)) != nullptr) return p;
   int prev = -1;                              // arena full, or no pool: plain device memory
   (void)hipGetDevice(&prev);
   if (prev != device) (void)hipSetDevice(device);

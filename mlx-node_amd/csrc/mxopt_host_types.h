@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "mxopt.h"
+#include "mxopt_diagnostics.h"
 
 namespace mxopt {
 

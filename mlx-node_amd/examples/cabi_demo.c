@@ -18,6 +18,7 @@
 #include <time.h>
 
 #include "mxopt_engine.h"
+#include "mxopt_diagnostics.h"   /* the bare probes */
 
 #define CHECK_HIP(call)                                                                  \
   do {                                                                                   \

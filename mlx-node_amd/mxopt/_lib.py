@@ -71,7 +71,26 @@ class HbmPoolInfo(C.Structure):
                 ("region_arena_bytes", C.c_uint64 * HBM_MAX_REGIONS),
                 ("probe_same_region_gbps", C.c_double), ("probe_cross_region_gbps", C.c_double),
                 ("setup_seconds", C.c_double), ("create_seconds", C.c_double), ("scan_seconds", C.c_double),
-                ("probes", C.c_int32), ("reserved2_", C.c_int32)]
+                ("probes", C.c_int32), ("reserved2_", C.c_int32), ("interleaved_bytes", C.c_uint64)]
+
+
+class HbmPoolOptions(C.Structure):
+    _fields_ = [("capacity_bytes", C.c_size_t), ("chunk_bytes", C.c_size_t), ("max_regions", C.c_int),
+                ("reserved_", C.c_int), ("max_take_bytes", C.c_size_t), ("slab_bytes", C.c_size_t)]
+
+
+class HbmScanReport(C.Structure):
+    _fields_ = [("regions", C.c_int32), ("probes", C.c_int32), ("same_region_gbps", C.c_double),
+                ("cross_region_gbps", C.c_double)]
+
+
+class HbmArenaReport(C.Structure):
+    _fields_ = [("real_regions", C.c_int32), ("active_regions", C.c_int32), ("interleaved_chunks", C.c_int32),
+                ("reserved_", C.c_int32)]
+
+
+SLAB_PROBE_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_double))
+HBM_INTERLEAVED, HBM_ONE_REGION = 0, 1
 
 
 class RmspropHp(C.Structure):
@@ -106,7 +125,14 @@ SIGNATURES = {
     "mxopt_hbm_spread_begin": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
     "mxopt_hbm_spread_end": (C.c_int, [C.c_void_p]),
     "mxopt_hbm_pool_create": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
+    "mxopt_hbm_pool_create_ex": (C.c_int, [C.c_void_p, C.POINTER(HbmPoolOptions), C.POINTER(C.c_void_p)]),
     "mxopt_hbm_pool_destroy": (C.c_int, [C.c_void_p]),
+    "mxopt_hbm_pool_alloc_kind": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_void_p)]),
+    "mxopt_hbm_pool_set_hook_kind": (C.c_int, [C.c_int]),
+    "mxopt_hbm_classify_regions": (C.c_int, [C.c_int, SLAB_PROBE_FN, C.c_void_p, C.POINTER(C.c_int),
+                                             C.POINTER(HbmScanReport)]),
+    "mxopt_hbm_plan_arena": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                       C.POINTER(C.c_int), C.POINTER(HbmArenaReport)]),
     "mxopt_hbm_pool_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
     "mxopt_hbm_pool_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "mxopt_hbm_pool_owns": (C.c_int, [C.c_void_p, C.c_void_p]),

@@ -297,22 +297,29 @@ class HbmPool:
     MAX_REGIONS = L.HBM_MAX_REGIONS
     _torch_allocator = None   # one per process: torch keeps the function pointers
 
-    def __init__(self, ctx: "Context", capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0):
+    def __init__(self, ctx: "Context", capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0,
+                 max_take_bytes: int = 0, slab_bytes: int = 0):
         self.ctx = ctx
         self.handle = C.c_void_p()
         torch.cuda.empty_cache()     # what torch caches is not free memory to the driver
-        L.check(ctx.lib.mxopt_hbm_pool_create(ctx.handle, capacity_bytes, chunk_bytes, max_regions,
-                                              C.byref(self.handle)), ctx.handle)
+        opts = L.HbmPoolOptions(capacity_bytes=capacity_bytes, chunk_bytes=chunk_bytes, max_regions=max_regions,
+                                max_take_bytes=max_take_bytes, slab_bytes=slab_bytes)
+        L.check(ctx.lib.mxopt_hbm_pool_create_ex(ctx.handle, C.byref(opts), C.byref(self.handle)), ctx.handle)
 
     def info(self) -> L.HbmPoolInfo:
         out = L.HbmPoolInfo()
         L.check(self.ctx.lib.mxopt_hbm_pool_get_info(self.handle, C.byref(out)), self.ctx.handle)
         return out
 
-    def alloc(self, nbytes: int) -> int:
+    def alloc(self, nbytes: int, kind: int = L.HBM_INTERLEAVED) -> int:
         p = C.c_void_p()
-        L.check(self.ctx.lib.mxopt_hbm_pool_alloc(self.handle, nbytes, C.byref(p)), self.ctx.handle)
+        L.check(self.ctx.lib.mxopt_hbm_pool_alloc_kind(self.handle, nbytes, kind, C.byref(p)), self.ctx.handle)
         return p.value
+
+    @staticmethod
+    def hook_kind(kind: int) -> None:
+        """What torch's allocations through torch_pool() get from now on: HBM_INTERLEAVED or HBM_ONE_REGION."""
+        L.check(L.load().mxopt_hbm_pool_set_hook_kind(kind))
 
     def free(self, ptr: int) -> None:
         L.check(self.ctx.lib.mxopt_hbm_pool_free(self.handle, C.c_void_p(ptr)), self.ctx.handle)
@@ -341,8 +348,32 @@ class HbmPool:
             self.handle = C.c_void_p()
 
 
-def _hbm_pool(self, capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0) -> HbmPool:
-    return HbmPool(self, capacity_bytes, chunk_bytes, max_regions)
+def _hbm_pool(self, capacity_bytes: int, chunk_bytes: int = 0, max_regions: int = 0, max_take_bytes: int = 0,
+              slab_bytes: int = 0) -> HbmPool:
+    return HbmPool(self, capacity_bytes, chunk_bytes, max_regions, max_take_bytes, slab_bytes)
+
+
+def classify_regions(n_slabs: int, probe):
+    """mxopt_hbm_classify_regions on a Python callable probe(ref_slab, slab) -> GB/s: (regions per slab, report)."""
+    def thunk(_user, ref, slab, out):
+        out[0] = float(probe(ref, slab))
+        return 0
+    fn = L.SLAB_PROBE_FN(thunk)
+    regions = (C.c_int * max(n_slabs, 1))()
+    report = L.HbmScanReport()
+    L.check(L.load().mxopt_hbm_classify_regions(n_slabs, fn, None, regions, C.byref(report)))
+    return list(regions[:n_slabs]), report
+
+
+def plan_arena(slab_region, regions: int, chunks_per_slab: int, total_chunks: int, want_chunks: int, max_regions: int = 0):
+    """mxopt_hbm_plan_arena: (physical chunk of every arena chunk, report)."""
+    n = len(slab_region)
+    sr = (C.c_int * max(n, 1))(*slab_region)
+    order = (C.c_int * max(want_chunks, 1))()
+    report = L.HbmArenaReport()
+    L.check(L.load().mxopt_hbm_plan_arena(n, sr, regions, chunks_per_slab, total_chunks, want_chunks, max_regions, order,
+                                          C.byref(report)))
+    return list(order[:want_chunks]), report
 
 
 def _probe_stream(self, kind: int, a, b=None, c=None, d=None) -> None:

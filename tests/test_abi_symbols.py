@@ -16,7 +16,7 @@ sys.path.insert(0, os.path.join(ROOT, "mlx-node_amd"))
 
 import mxopt_oracle as O
 
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("mxopt.h", "mxopt_optimizers.h", "mxopt_engine.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("mxopt.h", "mxopt_optimizers.h", "mxopt_engine.h", "mxopt_diagnostics.h")]
 
 
 @pytest.fixture(scope="module")
@@ -50,6 +50,7 @@ def test_ctypes_structs_match_c_layout(L, tmp_path):
 #include <stdio.h>
 #include <stddef.h>
 #include "mxopt_engine.h"
+#include "mxopt_diagnostics.h"
 #define S(T) printf(#T " %zu\n", sizeof(T))
 #define F(T, f) printf(#T "." #f " %zu\n", offsetof(T, f))
 #define V(name) printf("=" #name " %ld\n", (long)(name))
