@@ -99,6 +99,10 @@ def parse_args():
                          "(`verified` in the line); default: cfg5 only")
     ap.add_argument("--pool-regions", type=int, default=2, help="--placement pool: regions to alternate between (0 = all found)")
     ap.add_argument("--pool-chunk-mb", type=int, default=0, help="--placement pool: chunk size (0 = the library's 64)")
+    ap.add_argument("--pool-slab-mb", type=int, default=0, help="--placement pool: unit of the region scan, 512 ... 4096 (0 = the library's 1024)")
+    ap.add_argument("--grads-one-region", type=int, default=0,
+                    help="--placement pool: 1 = gradient buffers (read only in every kernel) come from the part of the "
+                         "arena behind the alternation, i.e. from one region")
     ap.add_argument("--others", type=int, default=-1,
                     help="1: after the main workload, run BASELINE's configs 1-4 for a few steps each and report them as "
                          "other_configs; default: only when the workload is cfg5 at full scale")
@@ -171,11 +175,23 @@ class Workload:
             getattr(self, "_setup_" + args.workload.replace("-", "_"))()
             torch.cuda.synchronize()
 
+    @contextlib.contextmanager
     def _window(self, kind):
         """Where buffers of this kind ("param", "grad", "state") are allocated."""
-        if kind in self.arena_kinds:
-            return self.torch.cuda.use_mem_pool(self.mem_pool)
-        return contextlib.nullcontext()
+        if kind not in self.arena_kinds:
+            yield
+            return
+        # gradient buffers are only ever read: with --grads-one-region they come from the part of the arena that
+        # lies behind the alternation (one region at a time), where read-only passes run a few per cent faster
+        one_region = kind == "grad" and getattr(self.args, "grads_one_region", 0)
+        if one_region:
+            self.mx.HbmPool.hook_kind(self.mx.HBM_ONE_REGION)
+        try:
+            with self.torch.cuda.use_mem_pool(self.mem_pool):
+                yield
+        finally:
+            if one_region:
+                self.mx.HbmPool.hook_kind(self.mx.HBM_INTERLEAVED)
 
     def free_bytes(self, kind="state"):
         """Device memory this workload may still take for buffers of that kind."""
@@ -978,7 +994,7 @@ def child_leg(args, placement, steps=5, warmup=2):
     cmd = [sys.executable, os.path.abspath(__file__), "--workload", args.workload, "--placement", placement,
            "--steps", str(steps), "--warmup", str(warmup), "--cpu-sample", "0", "--others", "0", "--placements", "0",
            "--verify", "0", "--ceiling", "0", "--variants", "0", "--fold-last", str(args.fold_last),
-           "--scale", str(args.scale), "--alloc", args.alloc]
+           "--scale", str(args.scale), "--alloc", args.alloc, "--micro", str(args.micro)]
     try:
         proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
         line = [l for l in proc.stdout.splitlines() if l.startswith("{")][-1]
@@ -1028,7 +1044,8 @@ def main():
         if three_placements or args.placement == "state-pool":
             host_side = sum(sizes) * 2 * 5 + (4 << 30) if args.workload == "cfg5" else free // 2
         try:
-            pool = ctx.hbm_pool(free - (8 << 30) - host_side, args.pool_chunk_mb << 20, args.pool_regions)
+            pool = ctx.hbm_pool(free - (8 << 30) - host_side, args.pool_chunk_mb << 20, args.pool_regions,
+                                slab_bytes=args.pool_slab_mb << 20)
         except mxopt.MxoptError as e:
             # e.g. another process holds most of the device: measure in plain memory and say so in the line
             print(f"bench.py: no region-interleaved arena ({e}); buffers come from plain device memory", file=sys.stderr)
@@ -1042,6 +1059,8 @@ def main():
                      "chunk_mib": i.chunk_bytes >> 20, "regions_found": i.regions,
                      "regions_used": min(args.pool_regions, i.regions) if args.pool_regions else i.regions,
                      "arena_gib": round(i.capacity_bytes / 2**30, 1),
+                     "interleaved_gib": round(i.interleaved_bytes / 2**30, 1),
+                     "gradients": "one region (behind the alternation)" if args.grads_one_region else "interleaved",
                      "region_free_gib": [round(x / 2**30, 1) for x in i.region_free_bytes[:i.regions]],
                      "probe_same_region_gbps": round(i.probe_same_region_gbps, 1),
                      "probe_cross_region_gbps": round(i.probe_cross_region_gbps, 1),

@@ -73,7 +73,10 @@ int mxopt_synchronize(mxopt_ctx* ctx);
 /* Tuning knobs, by name: "grid_blocks_per_cu" (persistent grid = CUs x this),
  * "persistent" (0: one workgroup per chunk for the update kernels), "persistent_accumulate" (1: the
  * persistent grid also for accumulation passes after the first that take no norm), "nontemporal" /
- * "nontemporal_reduce" (streaming-hint memory instructions in the read-write / read-only kernels). */
+ * "nontemporal_reduce" (streaming-hint memory instructions in the read-write / read-only kernels),
+ * "pipelined_norm" (the plain norm of a 16-bit stream: 0 = the general reduction kernel always; 2 (default)
+ * or 4 = a kernel that takes that many chunks per trip, for tables whose chunks are under 90 % full on
+ * average, i.e. many small tensors; 1 = that kernel, two chunks per trip, for every table). */
 int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value);
 int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value);
 
@@ -146,8 +149,9 @@ int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_by
  * process needs the GPU to itself for those seconds: another process's, or another thread's, allocation can
  * fail with out-of-memory meanwhile, and a co-tenant's traffic disturbs the timing.  max_take_bytes bounds what
  * is held (never less than the arena itself); with a bound below the free memory the scan sees less, possibly
- * one region only.  slab_bytes is the unit of classification (a power of two in [128 MiB, 4 GiB], default
- * 1 GiB): smaller slabs follow fragmented free memory more closely at about the same scan time. */
+ * one region only.  slab_bytes is the unit of classification (a power of two in [512 MiB, 4 GiB], default
+ * 1 GiB): 512 MiB slabs follow fragmented free memory more closely for twice the probes at about the same scan
+ * time; smaller ones would let the probe's working set sit in the last-level cache and hide the regions. */
 typedef struct mxopt_hbm_pool_options {
   size_t capacity_bytes;
   size_t chunk_bytes;      /* 0: 64 MiB */

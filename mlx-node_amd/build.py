@@ -49,6 +49,23 @@ def _headers_mtime() -> float:
     return max(os.path.getmtime(os.path.join(d, f)) for d in dirs for f in os.listdir(d) if f.endswith(".h"))
 
 
+def build_variant(out: str, defines, verbose: bool = False) -> str:
+    """The library alone, compiled with extra -D definitions into `out` (for A/B measurements of one build
+    against another on the same machine); objects go to a directory of their own."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    obj_dir = os.path.join(HERE, "bin", "obj_" + os.path.basename(out))
+    os.makedirs(obj_dir, exist_ok=True)
+    jobs = []
+    for s in SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(s)[0] + ".o")
+        jobs.append(([hipcc] + FLAGS + ["-D" + d for d in defines] + ["-x", "hip", "-c", os.path.join(CSRC, s), "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+        list(pool.map(lambda j: _run(j[0], verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + [obj for _, obj in jobs] + ["-o", out], verbose)
+    return out
+
+
 def build(verbose: bool = False, incremental: bool = False) -> str:
     """Every translation unit is compiled by its own hipcc process (they are independent and the three
     kernel files take about as long as each other), then linked.  incremental: a unit whose object file is
@@ -142,7 +159,10 @@ def build_sanitized(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    if "--sanitize" in sys.argv:
+    if "--variant" in sys.argv:   # --variant OUT.so [NAME=VALUE ...]
+        i = sys.argv.index("--variant")
+        print(build_variant(os.path.abspath(sys.argv[i + 1]), [a for a in sys.argv[i + 2:] if "=" in a]))
+    elif "--sanitize" in sys.argv:
         print(build_sanitized(verbose=True))
     else:
         print(build(verbose=True, incremental="--incremental" in sys.argv))

@@ -155,6 +155,9 @@ Launch make_launch(const mxopt_ctx* ctx, const mxopt_table* t, const Group& g, b
   L.grid = persistent ? persistent_grid(ctx, g.nchunks) : g.nchunks;
   L.stream = ctx->stream;
   L.nontemporal = ctx->nontemporal;
+  L.pipelined_norm = ctx->pipelined_norm;
+  L.any_unaligned = g.any_unaligned;
+  L.partial_chunks = g.elems * 10 < (uint64_t)g.nchunks * kChunkElems * 9;
   return L;
 }
 
@@ -268,6 +271,9 @@ Launch make_single_launch(const mxopt_ctx* ctx, const mxopt_tensor& t, bool pers
   L.grid = persistent ? persistent_grid(ctx, L.nchunks) : L.nchunks;
   L.stream = ctx->stream;
   L.nontemporal = ctx->nontemporal;
+  L.pipelined_norm = ctx->pipelined_norm;
+  L.any_unaligned = (L.one.flags & kTfUnaligned) != 0;
+  L.partial_chunks = L.one.n * 10 < (uint64_t)L.nchunks * kChunkElems * 9;
   return L;
 }
 
@@ -346,6 +352,8 @@ int mxopt_set_option(mxopt_ctx* ctx, const char* name, int64_t value) {
     ctx->nontemporal_reduce = value != 0;
   } else if (n == "persistent_accumulate") {
     ctx->persistent_accumulate = value != 0;
+  } else if (n == "pipelined_norm") {
+    ctx->pipelined_norm = (int)value;  // 0: the general kernel; 2 or 4: chunks per trip of the 16-bit norm kernel
   } else {
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_set_option: unknown option " + n);
   }
@@ -360,6 +368,7 @@ int mxopt_get_option(const mxopt_ctx* ctx, const char* name, int64_t* value) {
   else if (n == "nontemporal") *value = ctx->nontemporal;
   else if (n == "nontemporal_reduce") *value = ctx->nontemporal_reduce;
   else if (n == "persistent_accumulate") *value = ctx->persistent_accumulate;
+  else if (n == "pipelined_norm") *value = ctx->pipelined_norm;
   else if (n == "num_cus") *value = ctx->num_cus;
   else return MXOPT_ERR_INVALID_ARG;
   return MXOPT_OK;
@@ -463,6 +472,8 @@ int mxopt_table_build(mxopt_ctx* ctx, const mxopt_tensor* tensors, size_t n, mxo
     g.pd = (kv.first >> 24) & 0xff; g.gd = (kv.first >> 16) & 0xff; g.pod = (kv.first >> 8) & 0xff; g.god = kv.first & 0xff;
     g.chunk_begin = (uint32_t)chunks.size();
     for (uint32_t ti : kv.second) {
+      g.any_unaligned = g.any_unaligned || (t->dev[ti].flags & kTfUnaligned) != 0;
+      g.elems += t->dev[ti].n;
       const uint64_t nc = chunks_of(t->dev[ti]);
       for (uint64_t c = 0; c < nc; ++c) chunks.push_back(DevChunk{ti, (uint32_t)c});
     }

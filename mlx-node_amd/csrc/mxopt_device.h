@@ -32,6 +32,30 @@ __device__ __forceinline__ MXOPT_GLOBAL T* global_ptr(void* p) {
   return (MXOPT_GLOBAL T*)(uintptr_t)p;
 }
 
+// Tables (descriptors, chunk lists, pending-stream pointers) and the device scalars a kernel is handed are
+// written before the launch and never during it.  Read through the constant address space, a load whose
+// address is the same for the whole wavefront becomes a scalar load: it lands in scalar registers, goes
+// through the scalar cache, and is counted apart from the vector loads, so that waiting for a descriptor
+// never means waiting for the data loads already in flight.
+#define MXOPT_CONSTANT __attribute__((address_space(4)))
+template <class T>
+__device__ __forceinline__ const MXOPT_CONSTANT T* constant_ptr(const void* p) {
+  return (const MXOPT_CONSTANT T*)(uintptr_t)p;
+}
+
+// Element `index` of an array of plain structs, read word by word through the constant address space (the
+// compiler merges the words into s_load_dwordx2 ... x16).
+template <class S>
+__device__ __forceinline__ S load_constant(const void* array, size_t index) {
+  static_assert(sizeof(S) % 4 == 0 && alignof(S) >= 4, "whole 32-bit words");
+  struct Words { uint32_t w[sizeof(S) / 4]; };
+  const MXOPT_CONSTANT uint32_t* src = constant_ptr<uint32_t>(array) + index * (sizeof(S) / 4);
+  Words tmp;
+#pragma unroll
+  for (size_t i = 0; i < sizeof(S) / 4; ++i) tmp.w[i] = src[i];
+  return __builtin_bit_cast(S, tmp);
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

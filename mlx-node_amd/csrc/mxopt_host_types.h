@@ -69,6 +69,8 @@ struct StreamScales {
 struct Group {
   int pd, gd, pod, god;
   uint32_t chunk_begin, nchunks;
+  bool any_unaligned = false;  // some tensor of the group takes the element-wise path
+  uint64_t elems = 0;          // elements of the group's tensors (chunks * kChunkElems when every chunk is full)
 };
 
 }  // namespace mxopt
@@ -85,6 +87,7 @@ struct mxopt_ctx {
   int nontemporal = 0;          // streaming-hint loads/stores in update, transform, accumulate kernels
   int nontemporal_reduce = 1;   // streaming-hint loads in the read-only reduction kernels
   int persistent_accumulate = 0;  // bounded grid also for accumulation passes that take no norm
+  int pipelined_norm = 2;         // plain 16-bit norms: the software-pipelined kernel
   double* d_partial_sum = nullptr;            // one float64 partial per workgroup of a reduction
   size_t partial_cap = 0;
   double* d_static_partials = nullptr;        // this device's copy of the library's fixed partial-sum array

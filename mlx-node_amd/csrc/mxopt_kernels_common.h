@@ -144,9 +144,9 @@ __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, con
                                             const DevTensor& one, uint32_t c) {
   ChunkView cv;
   uint32_t index;
-  if (C != nullptr) {  // table walk
-    const DevChunk ch = C[c];
-    cv.t = T[ch.tensor];
+  if (C != nullptr) {  // table walk: two dependent scalar loads
+    const DevChunk ch = load_constant<DevChunk>(C, c);
+    cv.t = load_constant<DevTensor>(T, ch.tensor);
     cv.tensor = ch.tensor;
     index = ch.index;
   } else {             // a single tensor described in the kernel arguments: chunk c of `one`

@@ -25,7 +25,7 @@ __device__ __forceinline__ PendingStreams<KMAX> pending_of(const void* const* __
                                                      int kx) {
   PendingStreams<KMAX> ps;
 #pragma unroll
-  for (int j = 0; j < KMAX; ++j) ps.x[j] = j < kx ? X[(size_t)j * ntensors + row] : nullptr;
+  for (int j = 0; j < KMAX; ++j) ps.x[j] = j < kx ? (const void*)load_constant<uint64_t>(X, (size_t)j * ntensors + row) : nullptr;
   return ps;
 }
 

@@ -277,14 +277,14 @@ def test_pool_created_after_the_process_held_and_released_most_of_the_device(mx,
 
 
 def test_smaller_slabs_classify_the_same_memory(mx, ctx):
-    """slab_bytes = 256 MiB: four times the slabs, a quarter of the bytes per probe; the regions found must agree
-    with the default's to within a few slabs."""
+    """slab_bytes = 512 MiB: twice the slabs, half the bytes per probe; the regions found must agree with the
+    default's to within a few GiB (slabs that straddle two regions go to either)."""
     import torch
     torch.cuda.empty_cache()
     if torch.cuda.mem_get_info()[0] < 200 * GiB:
         pytest.skip("needs a nearly empty device")
     sizes = []
-    for slab in (0, 256 << 20):
+    for slab in (0, 512 << 20):
         p = ctx.hbm_pool(16 * GiB, 0, 2, slab_bytes=slab)
         i = p.info()
         sizes.append(sorted(i.region_free_bytes[:i.regions], reverse=True))
@@ -292,6 +292,6 @@ def test_smaller_slabs_classify_the_same_memory(mx, ctx):
         p.close()
     assert len(sizes[0]) == len(sizes[1])
     for a, b in zip(sizes[0], sizes[1]):
-        assert abs(a - b) <= 4 * GiB
+        assert abs(a - b) <= 12 * GiB
     with pytest.raises(mx.InvalidArg, match="slab_bytes"):
-        ctx.hbm_pool(GiB, slab_bytes=100 << 20)
+        ctx.hbm_pool(GiB, slab_bytes=256 << 20)
