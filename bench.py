@@ -1064,6 +1064,7 @@ def main():
                      "region_free_gib": [round(x / 2**30, 1) for x in i.region_free_bytes[:i.regions]],
                      "probe_same_region_gbps": round(i.probe_same_region_gbps, 1),
                      "probe_cross_region_gbps": round(i.probe_cross_region_gbps, 1),
+                     "probe_on_arena_gbps": round(i.arena_probe_gbps, 1),
                      "setup_s": round(i.setup_seconds, 2), "scan_s": round(i.scan_seconds, 2), "probes": i.probes}
     elif args.placement == "spread":
         placement = (f"buffers allocated between mxopt_hbm_spread_begin and _end ({args.spread_block_mb or 64} MiB "

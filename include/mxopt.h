@@ -120,7 +120,14 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * either way).  Allocations are 512-byte
  * aligned, first fit, thread-safe; contents are not cleared.  A pointer goes back to the pool it came
  * from whichever pool a context or the hooks point at by then.  Destroy the pool after everything that
- * allocated from it and before its context.  No counterpart in the reference (MLX owns its allocator there). */
+ * allocated from it and before its context.
+ * One pool per process, made at start-up.  The scan reads the regions off runs of consecutively created
+ * chunks: a process's first pool sees such runs (on a fresh device, after other processes came and went, after
+ * the process itself allocated and freed tens of GB), but once a pool has taken all memory chunk by chunk and
+ * given most of it back, chunks come in no physical order any more: a second pool made by the same process
+ * finds mixtures (every pair of 1 GiB groups answers at an in-between rate), reports whatever grouping the
+ * rates suggest, and its arena is interleaved by accident rather than by design.
+ * No counterpart in the reference (MLX owns its allocator there). */
 #define MXOPT_HBM_MAX_REGIONS 8
 typedef struct mxopt_hbm_pool mxopt_hbm_pool;
 typedef struct mxopt_hbm_pool_info {
@@ -140,6 +147,9 @@ typedef struct mxopt_hbm_pool_info {
   int32_t reserved2_;
   uint64_t interleaved_bytes;  /* arena bytes [0, this) alternate between regions chunk by chunk; what lies behind
                                   comes from one region at a time (MXOPT_HBM_ONE_REGION allocations) */
+  double arena_probe_gbps;     /* the 4-read/3-write probe over four pieces spread across the finished arena: what
+                                  was built, measured (compare with the two probe levels above; 0 for an arena
+                                  under 256 MiB) */
 } mxopt_hbm_pool_info;
 int mxopt_hbm_pool_create(mxopt_ctx* ctx, size_t capacity_bytes, size_t chunk_bytes, int max_regions,
                           mxopt_hbm_pool** out);

@@ -84,7 +84,9 @@ int mxopt_optimizer_update_many(mxopt_optimizer* opt, size_t n, const char* cons
  * GradientUtils::clip_grad_norm (optimizers/mod.rs:67-107; clip_mode as in mxopt_global_norm) of
  * that gradient's global norm, then the optimizer's own update (any of the four kinds) with
  * update_many's per-call step counting.  Two launches per dtype group, no accumulation buffer,
- * no host synchronisation.  k >= 1.  The kernels read MXOPT_MAX_PENDING + 1 streams: with a larger
+ * no host synchronisation.  k >= 1; with k = 1, no prep and no clip nothing is added or multiplied and
+ * the call is update_many (the lone gradient reaches the optimizer in its own dtype, so a 16-bit
+ * gradient's square is 16-bit there, mlx.cpp:2016-2020).  The kernels read MXOPT_MAX_PENDING + 1 streams: with a larger
  * k the oldest micro-batches are first added, in order, into a float32 buffer per parameter that
  * the optimizer keeps with its state (4 B/elem, freed by reset), and that buffer stands in for
  * them.  Of the streams the kernels read, the second to the last share one dtype and the first has

@@ -467,6 +467,31 @@ int mxopt_hbm_pool_create_ex(mxopt_ctx* ctx, const mxopt_hbm_pool_options* optio
   }
   info.probe_same_region_gbps = same_gbps;
   info.probe_cross_region_gbps = cross_gbps;
+  // What was built, measured: the 4-read/3-write probe over four pieces spread across the arena.  Whatever
+  // the scan concluded -- and when the free memory came in no physical order its grouping means little --
+  // this is the rate a kernel will see on memory from here.
+  info.arena_probe_gbps = 0.0;
+  if (pool->capacity >= 4 * ((size_t)64 << 20) && b.ev0 == nullptr) {
+    (void)hipEventCreate(&b.ev0);
+    (void)hipEventCreate(&b.ev1);
+  }
+  if (pool->capacity >= 4 * ((size_t)64 << 20) && b.ev0 && b.ev1) {
+    const size_t quarter = pool->capacity / 4 / kAlign * kAlign;
+    const size_t piece = std::min<size_t>(quarter, (size_t)1 << 30) / (kProbeTileElems * 4) * (kProbeTileElems * 4);
+    void* q[4];
+    for (int k = 0; k < 4; ++k) q[k] = pool->base + (size_t)k * quarter;
+    const uint64_t elems = piece / 4;
+    int rc = launch_probe(ctx, MXOPT_PROBE_MIX43, q[0], q[1], q[2], q[3], elems);
+    if (!rc && hipEventRecord(b.ev0, ctx->stream) == hipSuccess) {
+      for (int rep = 0; rep < 2 && !rc; ++rep) rc = launch_probe(ctx, MXOPT_PROBE_MIX43, q[0], q[1], q[2], q[3], elems);
+      float ms = 0.f;
+      if (!rc && hipEventRecord(b.ev1, ctx->stream) == hipSuccess && hipEventSynchronize(b.ev1) == hipSuccess &&
+          hipEventElapsedTime(&ms, b.ev0, b.ev1) == hipSuccess && ms > 0.f)
+        info.arena_probe_gbps = 2.0 * 7.0 * (double)piece / 1e9 / ((double)ms * 1e-3);
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipGetLastError();
+  }
   for (size_t i = 0; i < b.all.size(); ++i)   // what the arena does not use goes back to the driver now
     if (!b.released[i]) { (void)hipMemRelease(b.all[i]); b.released[i] = 1; }
   const auto t_end = std::chrono::steady_clock::now();
@@ -474,8 +499,10 @@ int mxopt_hbm_pool_create_ex(mxopt_ctx* ctx, const mxopt_hbm_pool_options* optio
   info.create_seconds = std::chrono::duration<double>(t_created - t_begin).count();
   info.scan_seconds = std::chrono::duration<double>(t_scanned - t_created).count();
   info.probes = probes;
-  MXOPT_DEBUG("hbm pool: %zu MiB arena of %zu MiB chunks over %d region(s); probe %.0f GB/s inside one region, %.0f across; %.2f s",
-              pool->capacity >> 20, chunk_bytes >> 20, nregions, same_gbps, cross_gbps, info.setup_seconds);
+  MXOPT_DEBUG("hbm pool: %zu MiB arena of %zu MiB chunks over %d region(s); probe %.0f GB/s inside one region, %.0f across, "
+              "%.0f on the arena; %.2f s",
+              pool->capacity >> 20, chunk_bytes >> 20, nregions, same_gbps, cross_gbps, info.arena_probe_gbps,
+              info.setup_seconds);
   {
     std::lock_guard<std::mutex> all(g_pools_mu);
     g_pools.push_back(pool);

@@ -71,7 +71,8 @@ class HbmPoolInfo(C.Structure):
                 ("region_arena_bytes", C.c_uint64 * HBM_MAX_REGIONS),
                 ("probe_same_region_gbps", C.c_double), ("probe_cross_region_gbps", C.c_double),
                 ("setup_seconds", C.c_double), ("create_seconds", C.c_double), ("scan_seconds", C.c_double),
-                ("probes", C.c_int32), ("reserved2_", C.c_int32), ("interleaved_bytes", C.c_uint64)]
+                ("probes", C.c_int32), ("reserved2_", C.c_int32), ("interleaved_bytes", C.c_uint64),
+                ("arena_probe_gbps", C.c_double)]
 
 
 class HbmPoolOptions(C.Structure):
