@@ -93,6 +93,12 @@ def parse_args():
                          "before this one touches the GPU: the first allocations of a fresh process) and with "
                          "--placement state-pool, and config.placement carries the three AdamW rates; default: only "
                          "for cfg5 at full scale on the arena")
+    ap.add_argument("--plain-leg", default="first", choices=["first", "last"],
+                    help="--placements: when the child process with --placement plain runs.  first: before this process "
+                         "touches the GPU (on a fresh box: the first allocations of a fresh process, one compact physical "
+                         "run -- and this process then finds the free memory in the order the child left it); last: "
+                         "after this process has given all its memory back (the child then gets pieces from all over the device, "
+                         "a matter of luck: 5.73 TB/s was measured that way against 5.34 first)")
     ap.add_argument("--verify", type=int, default=-1,
                     help="1: after the timed steps, seeded windows of parameters and moments are recomputed on the host "
                          "by the C twin of the oracle for exactly the steps that ran and compared bit for bit "
@@ -1018,8 +1024,8 @@ def main():
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
     full_default = args.workload == "cfg5" and args.scale == 1.0
     three_placements = args.placement == "pool" and (args.placements == 1 or (args.placements == -1 and full_default))
-    # before anything here touches the GPU: the plain leg wants to be the first allocations of a fresh process
-    plain_leg = child_leg(args, "plain") if three_placements else None
+    # first: before anything here touches the GPU, so that on a fresh box the child's are the first allocations
+    plain_leg = child_leg(args, "plain") if three_placements and args.plain_leg == "first" else None
 
     import torch
     import mxopt
@@ -1129,12 +1135,12 @@ def main():
         w3 = Workload(a, torch, mxopt, ctx, pool)
         state_pool_leg = leg_summary(measure(w3, 5, 2), w3, 5)
         w3.close()
-        placement["legs"] = {
+        placement["plain_leg_ran"] = args.plain_leg
+        legs = placement["legs"] = {
             "arena (every buffer from the pool; the headline)": main_leg,
             "state_pool (moments and accumulation buffers from the pool, parameters and gradients from torch's allocator)":
                 state_pool_leg,
-            "plain (torch's allocator for everything; child process run first, so the first allocations of a fresh process)":
-                plain_leg}
+            "plain (torch's allocator for everything; a child process)": plain_leg}
         placement["adamw_gbps"] = {"arena": main_leg["dominant_kernel_gbps"],
                                    "state_pool": state_pool_leg["dominant_kernel_gbps"],
                                    "plain": (plain_leg or {}).get("dominant_kernel_gbps")}
@@ -1162,6 +1168,22 @@ def main():
             w2.close()
         if args.cpu_sample > 0:
             others["cfg1"]["cpu_baseline"] = cpu_baseline_cfg1_full()
+
+    if three_placements and pool is not None and args.plain_leg == "last":
+        # everything this process held goes back to the driver first; the child then allocates as any host would
+        # that starts on a device other processes have used
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            pool.close()
+            pool = None
+        except mxopt.MxoptError as e:      # something still lives in the arena: the child gets what is left
+            placement["arena_not_released"] = str(e)
+        torch.cuda.empty_cache()
+        plain_leg = child_leg(args, "plain")
+        placement["legs"]["plain (torch's allocator for everything; a child process)"] = plain_leg
+        placement["adamw_gbps"]["plain"] = plain_leg.get("dominant_kernel_gbps")
 
     no_cpu_leg = ("copy", "probes", "grpo-engine", "sft-engine")
     cpu = cpu_baseline(args, n) if args.cpu_sample > 0 and args.workload not in no_cpu_leg else None

@@ -203,7 +203,9 @@ __device__ __forceinline__ PrepRegs load_prep(const DevPrep& p) {
   r.pre_mul = p.pre_mul; r.pre_lo = p.pre_lo; r.pre_hi = p.pre_hi;
   r.post_lo = p.post_lo; r.post_hi = p.post_hi; r.flags = p.flags;
   r.has_scale = p.d_scale != nullptr;
-  r.scale = r.has_scale ? *p.d_scale : 1.0f;
+  // A scalar load: every workgroup of the launch reads this one word, and as a vector load that is one request
+  // per wavefront to a single L2 channel (millions of them beside that channel's share of the streams).
+  r.scale = r.has_scale ? *constant_ptr<float>(p.d_scale) : 1.0f;
   return r;
 }
 

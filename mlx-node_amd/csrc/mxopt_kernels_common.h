@@ -167,7 +167,7 @@ __device__ __forceinline__ ChunkView locate(const DevTensor* __restrict__ T, con
 // Bit 0 of mxopt_norm_result.nonfinite is "some element was a NaN or an infinity"; bit 1 (finite elements
 // whose squares overflowed) does not stop a step: the reference clips such gradients to zero and goes on.
 __device__ __forceinline__ bool skip_requested(const DevPrep& prep) {
-  return prep.d_skip_if_nonzero != nullptr && (*prep.d_skip_if_nonzero & 1ull) != 0ull;
+  return prep.d_skip_if_nonzero != nullptr && (*constant_ptr<unsigned long long>(prep.d_skip_if_nonzero) & 1ull) != 0ull;
 }
 
 // A value clamp would turn +-Inf into a finite bound and hide it from the sum-based validity

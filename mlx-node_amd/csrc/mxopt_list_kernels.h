@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kThreads) void update_list_kernel(const DevTensor* 
     ps_regs[j] = pr;
     const bool has = each && j <= kx && scales.s[j] != nullptr;
     ps_regs[j].has_scale = has;
-    ps_regs[j].scale = has ? *scales.s[j] : 1.0f;
+    ps_regs[j].scale = has ? *constant_ptr<float>(scales.s[j]) : 1.0f;
   }
   if (pr.flags & kPrepFirstIsSum) {  // a buffer of earlier micro-batches, each prepared before it was added
     ps_regs[0].flags = 0;
