@@ -73,7 +73,9 @@ int mxopt_synchronize(mxopt_ctx* ctx);
 /* Tuning knobs, by name: "grid_blocks_per_cu" (persistent grid = CUs x this),
  * "persistent" (0: one workgroup per chunk for the update kernels), "persistent_accumulate" (1: the
  * persistent grid also for accumulation passes after the first that take no norm), "nontemporal" /
- * "nontemporal_reduce" (streaming-hint memory instructions in the read-write / read-only kernels),
+ * "nontemporal_reduce" (both 1 by default: streaming-hint memory instructions in the read-write / read-only
+ * kernels -- on every load that fetches whole 32-byte sectors, and on stores to lines the kernel has read;
+ * 0 = plain loads and stores; the list kernels of deferred accumulation always stream),
  * "pipelined_norm" (the plain norm of a 16-bit stream: 0 = the general reduction kernel always; 2 (default)
  * or 4 = a kernel that takes that many chunks per trip, for tables whose chunks are under 90 % full on
  * average, i.e. many small tensors; 1 = that kernel, two chunks per trip, for every table). */

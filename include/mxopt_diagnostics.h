@@ -21,12 +21,16 @@ extern "C" {
  * (a positive multiple of 4096, 16-byte aligned), no table, no tails, no arithmetic to speak of.
  *   MXOPT_PROBE_READ   reads a                       MXOPT_PROBE_WRITE  writes a
  *   MXOPT_PROBE_COPY   reads a, writes b             MXOPT_PROBE_MIX43  reads a, b, c, d and writes a, c, d
- * (MIX43 is float32 AdamW's byte mix, 28 B/elem.)  One launch on the context's stream. */
+ * (MIX43 is float32 AdamW's byte mix, 28 B/elem.)  One launch on the context's stream.
+ * kind | MXOPT_PROBE_STREAMING: the same streams with streaming-hint loads and stores, which is how the update
+ * kernels access memory by default (READ always streams; the pool's own region scan uses plain MIX43). */
 enum { MXOPT_PROBE_READ = 0, MXOPT_PROBE_WRITE = 1, MXOPT_PROBE_COPY = 2, MXOPT_PROBE_MIX43 = 3 };
+#define MXOPT_PROBE_STREAMING 0x100
 int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n_elems);
 /* The byte mix of the update over k un-summed 16-bit micro-batches (mxopt_adam_with_pending_list) without its
  * arithmetic: g[0..k) and p are 2-byte streams of n_elems elements, m and v 4-byte ones; p, m and v are
- * rewritten in place (2k + 20 B/elem).  k in [1, 8], n_elems a positive multiple of 4096. */
+ * rewritten in place (2k + 20 B/elem).  k in [1, 8], n_elems a positive multiple of 4096.
+ * k | MXOPT_PROBE_STREAMING: the 2-byte streams with streaming-hint loads and stores (the list kernels' way). */
 int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k, uint64_t n_elems);
 
 /* ---- synthetic data for benchmarks and parity tests ----------------------------------

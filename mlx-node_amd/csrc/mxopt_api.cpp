@@ -42,7 +42,14 @@ void log_line(const char* fmt, ...) {
   std::fprintf(stderr, "mxopt: %s\n", buf);
 }
 
-int fail(mxopt_ctx* ctx, int code, const std::string& msg) {
+int fail(mxopt_ctx* ctx, int code, const std::string& text) {
+  // Messages quote names out of files and arguments the caller supplied: what is not printable ASCII becomes
+  // '?', so that the message is valid UTF-8 for every binding that decodes it.
+  std::string msg = text;
+  for (char& ch : msg) {
+    const unsigned char u = (unsigned char)ch;
+    if ((u < 0x20 && ch != '\n' && ch != '\t') || u >= 0x7f) ch = '?';
+  }
   if (ctx) ctx->err = msg;
   g_thread_error = msg;
   if (log_level() >= 1) log_line("error %d: %s", code, msg.c_str());

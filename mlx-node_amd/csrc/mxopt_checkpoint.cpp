@@ -226,6 +226,9 @@ int read_header(mxopt_ctx* ctx, FILE* f, std::string* optimizer, int64_t* step,
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: not an optimizer-state checkpoint");
   const Json* kind = meta->get("optimizer");
   *optimizer = kind ? kind->string : "";
+  for (char ch : *optimizer)  // the name goes back to the caller as a C string: plain identifiers only
+    if (!((ch >= 'a' && ch <= 'z') || (ch >= 'A' && ch <= 'Z') || (ch >= '0' && ch <= '9') || ch == '_' || ch == '-'))
+      return fail(ctx, MXOPT_ERR_INVALID_ARG, "load_file: the optimizer name in the metadata is not a plain identifier");
   const Json* st = meta->get("step");
   if (step) *step = st ? std::strtoll(st->string.c_str(), nullptr, 10) : 0;
   if (std::fseek(f, 0, SEEK_END) != 0) return fail(ctx, MXOPT_ERR_FAILURE, "load_file: seek failed");

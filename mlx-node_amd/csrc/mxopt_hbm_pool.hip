@@ -47,30 +47,40 @@ __global__ __launch_bounds__(kProbeThreads) void probe_read_kernel(const pu32x4*
   if (s == 0x9E3779B9u && sink != nullptr) *sink = s;  // keeps the loads alive
 }
 
+// NT (the MXOPT_PROBE_STREAMING bit of the kind): streaming-hint stores, and loads where the plain form has plain
+// loads; what the update kernels do by default.
+template <bool NT, class T>
+__device__ __forceinline__ T probe_ld(const T* q) { return NT ? __builtin_nontemporal_load(q) : *q; }
+template <bool NT, class T>
+__device__ __forceinline__ void probe_st(T* q, T v) { if (NT) __builtin_nontemporal_store(v, q); else *q = v; }
+
 // One write stream.
+template <bool NT>
 __global__ __launch_bounds__(kProbeThreads) void probe_write_kernel(pu32x4* __restrict__ a, uint32_t ntiles) {
   for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
     const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
     const pu32x4 r = {t, t, t, t};
 #pragma unroll
-    for (int j = 0; j < kProbeVecs; ++j) a[b + j * kProbeThreads] = r;
+    for (int j = 0; j < kProbeVecs; ++j) probe_st<NT>(a + b + j * kProbeThreads, r);
   }
 }
 
 // One read and one write stream.
+template <bool NT>
 __global__ __launch_bounds__(kProbeThreads) void probe_copy_kernel(const pu32x4* __restrict__ a, pu32x4* __restrict__ o,
                                                                   uint32_t ntiles) {
   for (uint32_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
     const size_t b = (size_t)t * (kProbeThreads * kProbeVecs) + threadIdx.x;
     pu32x4 r[kProbeVecs];
 #pragma unroll
-    for (int j = 0; j < kProbeVecs; ++j) r[j] = a[b + j * kProbeThreads];
+    for (int j = 0; j < kProbeVecs; ++j) r[j] = probe_ld<NT>(a + b + j * kProbeThreads);
 #pragma unroll
-    for (int j = 0; j < kProbeVecs; ++j) o[b + j * kProbeThreads] = r[j];
+    for (int j = 0; j < kProbeVecs; ++j) probe_st<NT>(o + b + j * kProbeThreads, r[j]);
   }
 }
 
 // AdamW's float32 byte mix without its arithmetic: reads a, b, c, d; writes a, c, d in place.
+template <bool NT>
 __global__ __launch_bounds__(kProbeThreads) void probe_mix43_kernel(pu32x4* __restrict__ a, const pu32x4* __restrict__ g,
                                                                    pu32x4* __restrict__ c, pu32x4* __restrict__ d,
                                                                    uint32_t ntiles) {
@@ -79,14 +89,14 @@ __global__ __launch_bounds__(kProbeThreads) void probe_mix43_kernel(pu32x4* __re
     pu32x4 ra[kProbeVecs], rg[kProbeVecs], rc[kProbeVecs], rd[kProbeVecs];
 #pragma unroll
     for (int j = 0; j < kProbeVecs; ++j) {
-      ra[j] = a[b + j * kProbeThreads]; rg[j] = g[b + j * kProbeThreads];
-      rc[j] = c[b + j * kProbeThreads]; rd[j] = d[b + j * kProbeThreads];
+      ra[j] = probe_ld<NT>(a + b + j * kProbeThreads); rg[j] = probe_ld<NT>(g + b + j * kProbeThreads);
+      rc[j] = probe_ld<NT>(c + b + j * kProbeThreads); rd[j] = probe_ld<NT>(d + b + j * kProbeThreads);
     }
 #pragma unroll
     for (int j = 0; j < kProbeVecs; ++j) {
-      a[b + j * kProbeThreads] = ra[j] ^ rg[j];
-      c[b + j * kProbeThreads] = rc[j] + rg[j];
-      d[b + j * kProbeThreads] = rd[j] ^ (rg[j] >> 1);
+      probe_st<NT>(a + b + j * kProbeThreads, ra[j] ^ rg[j]);
+      probe_st<NT>(c + b + j * kProbeThreads, rc[j] + rg[j]);
+      probe_st<NT>(d + b + j * kProbeThreads, rd[j] ^ (rg[j] >> 1));
     }
   }
 }
@@ -94,8 +104,10 @@ __global__ __launch_bounds__(kProbeThreads) void probe_mix43_kernel(pu32x4* __re
 // The byte mix of the update over un-summed 16-bit micro-batches (deferred accumulation) without its
 // arithmetic: per element K + 1 two-byte reads (the gradient streams and the parameter), two four-byte
 // reads (the moments); the parameter and the moments are written back in place.  One workgroup per
-// 4096-element tile, every load of the tile issued before the first store, as in the update kernels.
-template <int K>
+// 4096-element tile, every load of the tile issued before the first store, as in the update kernels.  NT: the
+// 2-byte streams use streaming loads and stores; the 4-byte ones, whose two 16-byte pieces per lane share their
+// sectors, stay plain (the list kernels' rule).
+template <int K, bool NT>
 __global__ __launch_bounds__(kProbeThreads) void probe_list_kernel(pu32x4* __restrict__ p, pu32x4* __restrict__ m,
                                                                   pu32x4* __restrict__ v,
                                                                   const pu32x4* __restrict__ g0, const pu32x4* __restrict__ g1,
@@ -112,8 +124,8 @@ __global__ __launch_bounds__(kProbeThreads) void probe_list_kernel(pu32x4* __res
 #pragma unroll
     for (int j = 0; j < U; ++j) {
 #pragma unroll
-      for (int k = 0; k < K; ++k) rg[k][j] = gs[k][b16 + j * kProbeThreads];
-      rp[j] = p[b16 + j * kProbeThreads];
+      for (int k = 0; k < K; ++k) rg[k][j] = probe_ld<NT>(gs[k] + b16 + j * kProbeThreads);
+      rp[j] = probe_ld<NT>(p + b16 + j * kProbeThreads);
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         rm[j][h] = m[b32 + (2 * j + h) * kProbeThreads];
@@ -125,7 +137,7 @@ __global__ __launch_bounds__(kProbeThreads) void probe_list_kernel(pu32x4* __res
       pu32x4 s = rg[0][j];
 #pragma unroll
       for (int k = 1; k < K; ++k) s += rg[k][j];
-      p[b16 + j * kProbeThreads] = rp[j] ^ s;
+      probe_st<NT>(p + b16 + j * kProbeThreads, rp[j] ^ s);
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         m[b32 + (2 * j + h) * kProbeThreads] = rm[j][h] + s;
@@ -135,15 +147,17 @@ __global__ __launch_bounds__(kProbeThreads) void probe_list_kernel(pu32x4* __res
   }
 }
 
-template <int K>
+template <int K, bool NT>
 static void launch_probe_list_k(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, uint32_t ntiles) {
   const pu32x4* q[8];
   for (int k = 0; k < 8; ++k) q[k] = (const pu32x4*)g[k < K ? k : 0];
-  hipLaunchKernelGGL(probe_list_kernel<K>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)p, (pu32x4*)m,
+  hipLaunchKernelGGL((probe_list_kernel<K, NT>), dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)p, (pu32x4*)m,
                      (pu32x4*)v, q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], ntiles);
 }
 
-static int launch_probe(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void* d, uint64_t n) {
+static int launch_probe(mxopt_ctx* ctx, int kind_and_flags, void* a, void* b, void* c, void* d, uint64_t n) {
+  const bool nt = (kind_and_flags & MXOPT_PROBE_STREAMING) != 0;
+  const int kind = kind_and_flags & ~MXOPT_PROBE_STREAMING;
   const uint32_t ntiles = (uint32_t)(n / kProbeTileElems);
   const uint32_t bounded = (uint32_t)std::min<uint64_t>(ntiles, (uint64_t)ctx->num_cus * 16u);
   switch (kind) {
@@ -152,15 +166,20 @@ static int launch_probe(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, voi
                          (uint32_t*)nullptr);
       break;
     case MXOPT_PROBE_WRITE:
-      hipLaunchKernelGGL(probe_write_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a, ntiles);
+      if (nt) hipLaunchKernelGGL(probe_write_kernel<true>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a, ntiles);
+      else hipLaunchKernelGGL(probe_write_kernel<false>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a, ntiles);
       break;
     case MXOPT_PROBE_COPY:
-      hipLaunchKernelGGL(probe_copy_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (const pu32x4*)a,
-                         (pu32x4*)b, ntiles);
+      if (nt) hipLaunchKernelGGL(probe_copy_kernel<true>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (const pu32x4*)a,
+                                 (pu32x4*)b, ntiles);
+      else hipLaunchKernelGGL(probe_copy_kernel<false>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (const pu32x4*)a,
+                              (pu32x4*)b, ntiles);
       break;
     case MXOPT_PROBE_MIX43:
-      hipLaunchKernelGGL(probe_mix43_kernel, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a,
-                         (const pu32x4*)b, (pu32x4*)c, (pu32x4*)d, ntiles);
+      if (nt) hipLaunchKernelGGL(probe_mix43_kernel<true>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a,
+                                 (const pu32x4*)b, (pu32x4*)c, (pu32x4*)d, ntiles);
+      else hipLaunchKernelGGL(probe_mix43_kernel<false>, dim3(ntiles), dim3(kProbeThreads), 0, ctx->stream, (pu32x4*)a,
+                              (const pu32x4*)b, (pu32x4*)c, (pu32x4*)d, ntiles);
       break;
     default:
       return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: unknown kind");
@@ -257,7 +276,8 @@ int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void
   if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: null context");
   if (n_elems == 0 || n_elems % kProbeTileElems != 0 || n_elems / kProbeTileElems > 0xffffffffull)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, "mxopt_probe_stream: n_elems must be a positive multiple of 4096");
-  const int need = kind == MXOPT_PROBE_MIX43 ? 4 : kind == MXOPT_PROBE_COPY ? 2 : 1;
+  const int base_kind = kind & ~MXOPT_PROBE_STREAMING;
+  const int need = base_kind == MXOPT_PROBE_MIX43 ? 4 : base_kind == MXOPT_PROBE_COPY ? 2 : 1;
   void* ptrs[4] = {a, b, c, d};
   for (int i = 0; i < need; ++i)
     if (!ptrs[i] || (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u))
@@ -266,8 +286,11 @@ int mxopt_probe_stream(mxopt_ctx* ctx, int kind, void* a, void* b, void* c, void
   return launch_probe(ctx, kind, a, b, c, d, n_elems);
 }
 
-int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k, uint64_t n_elems) {
+int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* const* g, int k_and_flags,
+                     uint64_t n_elems) {
   const char* op = "mxopt_probe_list";
+  const bool nt = (k_and_flags & MXOPT_PROBE_STREAMING) != 0;
+  const int k = k_and_flags & ~MXOPT_PROBE_STREAMING;
   if (!ctx) return fail(nullptr, MXOPT_ERR_INVALID_ARG, std::string(op) + ": null context");
   if (n_elems == 0 || n_elems % 4096 != 0 || n_elems / 4096 > 0xffffffffull)
     return fail(ctx, MXOPT_ERR_INVALID_ARG, std::string(op) + ": n_elems must be a positive multiple of 4096");
@@ -280,14 +303,14 @@ int mxopt_probe_list(mxopt_ctx* ctx, void* p, void* m, void* v, const void* cons
   DeviceGuard guard(ctx->device);
   const uint32_t ntiles = (uint32_t)(n_elems / 4096);
   switch (k) {
-    case 1: launch_probe_list_k<1>(ctx, p, m, v, g, ntiles); break;
-    case 2: launch_probe_list_k<2>(ctx, p, m, v, g, ntiles); break;
-    case 3: launch_probe_list_k<3>(ctx, p, m, v, g, ntiles); break;
-    case 4: launch_probe_list_k<4>(ctx, p, m, v, g, ntiles); break;
-    case 5: launch_probe_list_k<5>(ctx, p, m, v, g, ntiles); break;
-    case 6: launch_probe_list_k<6>(ctx, p, m, v, g, ntiles); break;
-    case 7: launch_probe_list_k<7>(ctx, p, m, v, g, ntiles); break;
-    default: launch_probe_list_k<8>(ctx, p, m, v, g, ntiles); break;
+    case 1: nt ? launch_probe_list_k<1, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<1, false>(ctx, p, m, v, g, ntiles); break;
+    case 2: nt ? launch_probe_list_k<2, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<2, false>(ctx, p, m, v, g, ntiles); break;
+    case 3: nt ? launch_probe_list_k<3, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<3, false>(ctx, p, m, v, g, ntiles); break;
+    case 4: nt ? launch_probe_list_k<4, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<4, false>(ctx, p, m, v, g, ntiles); break;
+    case 5: nt ? launch_probe_list_k<5, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<5, false>(ctx, p, m, v, g, ntiles); break;
+    case 6: nt ? launch_probe_list_k<6, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<6, false>(ctx, p, m, v, g, ntiles); break;
+    case 7: nt ? launch_probe_list_k<7, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<7, false>(ctx, p, m, v, g, ntiles); break;
+    default: nt ? launch_probe_list_k<8, true>(ctx, p, m, v, g, ntiles) : launch_probe_list_k<8, false>(ctx, p, m, v, g, ntiles); break;
   }
   return check_launch(ctx, op);
 }

@@ -84,7 +84,7 @@ struct mxopt_ctx {
   int num_cus = 0;
   int grid_blocks_per_cu = 16;  // bounded grids (reductions, accumulation): workgroups per CU
   int persistent = 0;           // update kernels: 0 = one workgroup per chunk, 1 = bounded grid
-  int nontemporal = 0;          // streaming-hint loads/stores in update, transform, accumulate kernels
+  int nontemporal = 1;          // streaming-hint loads/stores in update, transform, accumulate kernels
   int nontemporal_reduce = 1;   // streaming-hint loads in the read-only reduction kernels
   int persistent_accumulate = 0;  // bounded grid also for accumulation passes that take no norm
   int pipelined_norm = 2;         // plain 16-bit norms: the software-pipelined kernel

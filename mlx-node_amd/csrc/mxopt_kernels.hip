@@ -78,7 +78,8 @@ __global__ __launch_bounds__(kThreads) void update_kernel(const DevTensor* __res
 #pragma unroll
       for (int j = 0; j < U; ++j) {
         const uint64_t off = start + (uint64_t)(j * kThreads + tid) * E;
-        store_group<OD, E, NT>(PO, off, p[j]);
+        if (PO == P) store_group<OD, E, NT>(PO, off, p[j]);  // streaming only where the line was read
+        else store_group<OD, E, false>(PO, off, p[j]);
         if (Math::kM) store_group<MXOPT_F32, E, NT>(M, off, m[j]);
         if (use_v) store_group<MXOPT_F32, E, NT>(V, off, v[j]);
       }
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
             if (add) g[j][e] = a[j][e] + g[j][e];
           }
         }
-        store_group<OD, E, NT>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);
+        store_group<OD, E, NT && ADD>(GO, start + (uint64_t)(j * kThreads + tid) * E, g[j]);  // streaming only where the line was read
       }
     } else {
       const uint32_t ngroups = (cv.t.flags & kTfUnaligned) ? 0u : cv.len / E;

@@ -19,7 +19,7 @@ struct Launch {
   uint32_t nchunks = 0;
   uint32_t grid = 0;                 // workgroups (<= nchunks)
   hipStream_t stream = nullptr;
-  int nontemporal = 0;               // non-zero: streaming-hint loads and stores
+  int nontemporal = 1;               // non-zero: streaming-hint loads and stores
   int pipelined_norm = 2;            // plain 16-bit norms take the software-pipelined kernel
   bool any_unaligned = false;        // some tensor of the launch takes the element-wise path
   bool partial_chunks = false;       // the chunks are under 90 % full on average (many small tensors)

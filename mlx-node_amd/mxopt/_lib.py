@@ -62,6 +62,7 @@ class SgdHp(C.Structure):
 
 HBM_MAX_REGIONS = 8
 PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_MIX43 = 0, 1, 2, 3
+PROBE_STREAMING = 0x100
 
 
 class HbmPoolInfo(C.Structure):

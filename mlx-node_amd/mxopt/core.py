@@ -388,11 +388,13 @@ def _hbm_spread(self, block_bytes: int = 0, keep_one_in: int = 0) -> _HbmSpread:
 
 Context.hbm_spread = _hbm_spread
 Context.hbm_pool = _hbm_pool
-def _probe_list(self, p, m, v, grads) -> None:
-    """One launch of the bare byte mix of the update over un-summed 16-bit micro-batches (mxopt_probe_list)."""
+def _probe_list(self, p, m, v, grads, streaming: bool = False) -> None:
+    """One launch of the bare byte mix of the update over un-summed 16-bit micro-batches (mxopt_probe_list);
+    streaming: the 2-byte streams with streaming-hint loads and stores, as the list kernels access them."""
     arr = (C.c_void_p * len(grads))(*[_dev_ptr(g) for g in grads])
+    k = len(grads) | (L.PROBE_STREAMING if streaming else 0)
     L.check(self.lib.mxopt_probe_list(self.handle, C.c_void_p(_dev_ptr(p)), C.c_void_p(_dev_ptr(m)),
-                                      C.c_void_p(_dev_ptr(v)), arr, len(grads), p.numel()), self.handle)
+                                      C.c_void_p(_dev_ptr(v)), arr, k, p.numel()), self.handle)
 
 
 Context.probe_stream = _probe_stream

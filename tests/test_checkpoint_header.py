@@ -65,6 +65,8 @@ def test_refuses_malformed_files(lib, tmp_path):
         "not json": (b"{not json" + b" " * 7, b""),
         "deep nesting": (b"[" * 200 + b"]" * 200, b""),
         "unterminated string": (b'{"abc', b""),
+        "optimizer name with a byte that is no text": (ok_header.replace(b'"adamw"', b'"\x80damw"'), b"\0" * 16),
+        "optimizer name with a control character": (ok_header.replace(b'"adamw"', b'"ada\\nw"'), b"\0" * 16),
     }
     for name, spec in cases.items():
         path = tmp_path / "bad"
