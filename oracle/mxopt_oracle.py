@@ -30,6 +30,10 @@ What pins each function (see tests/test_oracle_*.py)
   agreement with torch.optim / torch.nn.utils (a library that is not the
   reference) to ~1e-6 relative, plus float64 brute force on small inputs.
 * f32<->bf16 conversion: bit-exact against torch's CPU conversion.
+* GradientUtils.clip_grad_value_and_norm (clamp, norm of the clamped values, scale; max_norm=None
+  returns the clamped values: optimizers/mod.rs:174-226) and clip_gradients_by_value with a one-sided
+  bound through inf (gradients/mod.rs:299-312, mlx.cpp:469-481): closed forms worked by hand in
+  tests/test_oracle_kat.py.
 
 PARITY UNPINNED (no reference test, fixture or buildable reference covers it):
 * bf16 inputs through any optimizer (promotion to float32 by the scalar multiplies and
