@@ -158,26 +158,29 @@ def test_optimizer_state_comes_from_the_pool(mx, ctx, pool):
     del opt
 
 
-def test_probes_move_the_bytes_they_claim(mx, ctx):
+@pytest.mark.parametrize("streaming", [0, 1])
+def test_probes_move_the_bytes_they_claim(mx, ctx, streaming):
+    """Both forms of every probe (plain accesses; MXOPT_PROBE_STREAMING: streaming-hint loads and stores)."""
     import torch
+    flag = mx.PROBE_STREAMING if streaming else 0
     n = 4096 * 37
     rng = np.random.default_rng(13)
     host = [rng.integers(0, 2**31 - 1, n, dtype=np.int64).astype(np.int32) for _ in range(4)]
     a, b, c, d = [torch.from_numpy(h.copy()).cuda().view(torch.float32) for h in host]
     before = [t.clone() for t in (a, b, c, d)]
-    ctx.probe_stream(mx.PROBE_READ, a)
+    ctx.probe_stream(mx.PROBE_READ | flag, a)
     torch.cuda.synchronize()
     assert torch.equal(a.view(torch.int32), before[0].view(torch.int32))
-    ctx.probe_stream(mx.PROBE_COPY, a, b)
+    ctx.probe_stream(mx.PROBE_COPY | flag, a, b)
     torch.cuda.synchronize()
     assert torch.equal(b.view(torch.int32), a.view(torch.int32))
     a0, g0, c0, d0 = [t.view(torch.int32).cpu().numpy().astype(np.uint32) for t in (a, b, c, d)]
-    ctx.probe_stream(mx.PROBE_MIX43, a, b, c, d)
+    ctx.probe_stream(mx.PROBE_MIX43 | flag, a, b, c, d)
     torch.cuda.synchronize()
     got = [t.view(torch.int32).cpu().numpy().astype(np.uint32) for t in (a, b, c, d)]
     assert np.array_equal(got[0], a0 ^ g0) and np.array_equal(got[1], g0)
     assert np.array_equal(got[2], c0 + g0) and np.array_equal(got[3], d0 ^ (g0 >> 1))
-    ctx.probe_stream(mx.PROBE_WRITE, a)
+    ctx.probe_stream(mx.PROBE_WRITE | flag, a)
     torch.cuda.synchronize()
     w = a.view(torch.int32).cpu().numpy()
     assert np.array_equal(w, np.repeat(np.arange(n // 4096, dtype=np.int32), 4096))   # every element written, by its tile
@@ -186,7 +189,36 @@ def test_probes_move_the_bytes_they_claim(mx, ctx):
     with pytest.raises(mx.InvalidArg, match="non-NULL"):
         ctx.probe_stream(mx.PROBE_COPY, a)
     with pytest.raises(mx.InvalidArg, match="unknown kind"):
-        ctx.probe_stream(9, a)
+        ctx.probe_stream(9 | flag, a)
+
+
+@pytest.mark.parametrize("k,streaming", [(1, False), (4, False), (4, True), (8, True)])
+def test_list_probe_moves_the_bytes_it_claims(mx, ctx, k, streaming):
+    """mxopt_probe_list: per 4096-element tile and lane, two 16-byte pieces of every 2-byte stream and four of every
+    4-byte stream; s = the word-wise sum of the gradient pieces, p ^= s, m += s, v ^= s >> 1 (both 16-byte halves of a
+    moment group get the s of their parameter piece)."""
+    import torch
+    tiles = 9
+    n = 4096 * tiles
+    rng = np.random.default_rng(k + 100 * streaming)
+    words = lambda count: rng.integers(0, 2**32, count, dtype=np.uint64).astype(np.uint32)
+    g_h = [words(n // 2) for _ in range(k)]                  # 2 bytes per element
+    p_h, m_h, v_h = words(n // 2), words(n), words(n)
+    dev = lambda h: torch.from_numpy(h.view(np.int32).copy()).cuda()
+    gs, p, m, v = [dev(h).view(torch.bfloat16) for h in g_h], dev(p_h).view(torch.bfloat16), dev(m_h).view(torch.float32), dev(v_h).view(torch.float32)
+    ctx.probe_list(p, m, v, gs, streaming=streaming)
+    torch.cuda.synchronize()
+    back = lambda t: t.view(torch.int32).cpu().numpy().view(np.uint32)
+    S = np.zeros((tiles, 2, 256, 4), np.uint32)
+    for h in g_h:
+        S = S + h.reshape(tiles, 2, 256, 4)
+    assert np.array_equal(back(p).reshape(tiles, 2, 256, 4), p_h.reshape(tiles, 2, 256, 4) ^ S)
+    assert np.array_equal(back(m).reshape(tiles, 2, 2, 256, 4), m_h.reshape(tiles, 2, 2, 256, 4) + S[:, :, None])
+    assert np.array_equal(back(v).reshape(tiles, 2, 2, 256, 4), v_h.reshape(tiles, 2, 2, 256, 4) ^ (S >> 1)[:, :, None])
+    for g, h in zip(gs, g_h):
+        assert np.array_equal(back(g), h)                   # read only
+    with pytest.raises(mx.InvalidArg, match="1 to 8"):
+        ctx.probe_list(p, m, v, gs * 9)
 
 
 def test_one_region_kind_without_such_a_part_changes_nothing(mx, pool):
