@@ -55,7 +55,9 @@ struct SumsqChunk {
   }
 
   // The new sum of group j.  A streaming store pays off where the pass has just read the line it writes; the
-  // first pass of a cycle writes lines nobody read (acc = widen(g)), and there it costs 60 % more time.
+  // first pass of a cycle writes lines nobody read (acc = widen(g)), and there streaming stores cost 60 % more
+  // time (measured on the bf16 -> float32 pass, whose float32 stores come in sector-sharing pairs that
+  // store_group no longer streams anyway; single-piece stores were not measured on their own).
   static __device__ __forceinline__ void store_sum(const ChunkView& cv, uint32_t tid, int j, bool first,
                                                    const float (&v)[E]) {
     const uint64_t off = cv.start + (uint64_t)(j * kThreads + tid) * E;
