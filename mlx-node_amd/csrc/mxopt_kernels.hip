@@ -128,7 +128,10 @@ __global__ __launch_bounds__(kThreads) void transform_kernel(const DevTensor* __
                                                              const DevChunk* __restrict__ C, DevTensor one,
                                                              uint32_t nchunks, DevPrep prep) {
   constexpr bool add = ADD;
-  constexpr int E = (GD != MXOPT_F32 || OD != MXOPT_F32) ? 8 : 4;
+  // Elements per lane and group: 4 when the kernel adds into g_out (every access then covers whole sectors and
+  // streams: the GRPO engine's accumulate of clamp * scale, bf16 into float32, 13.0 against 13.4 ms on the
+  // Qwen3-8B list), 8 when a 16-bit stream is only converted (the first micro-batch: 8 was not slower there).
+  constexpr int E = ((GD != MXOPT_F32 || OD != MXOPT_F32) && !ADD) ? 8 : 4;
   constexpr int U = kElemsPerLane / E;
   if (skip_requested(prep)) return;
   const PrepRegs pr = load_prep(prep);
