@@ -71,6 +71,8 @@ int main(void) {
   V(MXOPT_SYNTH_NORMAL); V(MXOPT_SYNTH_NORMAL_OUTLIERS); V(MXOPT_SYNTH_UNIFORM);
   V(MXOPT_ENGINE_GRPO); V(MXOPT_ENGINE_SFT); V(MXOPT_ENGINE_APPLY_SGD); V(MXOPT_ENGINE_APPLY_ADAMW);
   V(MXOPT_F32); V(MXOPT_F16); V(MXOPT_BF16);
+  V(MXOPT_PROBE_READ); V(MXOPT_PROBE_WRITE); V(MXOPT_PROBE_COPY); V(MXOPT_PROBE_MIX43); V(MXOPT_PROBE_STREAMING);
+  V(MXOPT_HBM_INTERLEAVED); V(MXOPT_HBM_ONE_REGION);
   return 0;
 }''')
     exe = tmp_path / "layout"
