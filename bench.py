@@ -94,16 +94,26 @@ def parse_args():
                          "--placement state-pool, and config.placement carries the three AdamW rates; default: only "
                          "for cfg5 at full scale on the arena")
     ap.add_argument("--plain-leg", default="first", choices=["first", "last"],
-                    help="--placements: when the child process with --placement plain runs.  first: before this process "
-                         "touches the GPU (on a fresh box: the first allocations of a fresh process, one compact physical "
-                         "run -- and this process then finds the free memory in the order the child left it); last: "
-                         "after this process has given all its memory back (the child then gets pieces from all over the device, "
-                         "a matter of luck: 5.73 TB/s was measured that way against 5.34 first)")
+                    help="--placements: when the child process with --placement plain runs.  first (default): before this "
+                         "process touches the GPU; on a fresh box the child's are then the first allocations of a fresh "
+                         "process, one compact physical run in one region, the worst case (5.37 TB/s in every run); this "
+                         "process then waits --settle-s before it looks at the device.  last: after this process has given "
+                         "all its memory back; the child then gets pieces from all over the device, which is what a host "
+                         "sees on a GPU other processes have used (5.5 - 6.05 TB/s measured)")
     ap.add_argument("--verify", type=int, default=-1,
                     help="1: after the timed steps, seeded windows of parameters and moments are recomputed on the host "
                          "by the C twin of the oracle for exactly the steps that ran and compared bit for bit "
                          "(`verified` in the line); default: cfg5 only")
     ap.add_argument("--pool-regions", type=int, default=2, help="--placement pool: regions to alternate between (0 = all found)")
+    ap.add_argument("--pool-gib", type=float, default=0.0,
+                    help="--placement pool: size of the arena in GiB (0 = all free memory but a margin, less what the "
+                         "state-pool leg keeps in plain memory)")
+    ap.add_argument("--settle-s", type=float, default=-1.0,
+                    help="seconds to wait after device memory went back to the driver (an arena smaller than the free "
+                         "memory; a child process that has exited) before anything is measured or probed: for about 3 s "
+                         "after a release of tens of GB every kernel runs 0.7 %% slower (75.44 against 74.92 ms per step "
+                         "with 80 GiB released, fresh machines, twice each; 74.94 after 3 s).  -1: 4 s after the arena, "
+                         "8 s after a child that held the whole workload")
     ap.add_argument("--pool-chunk-mb", type=int, default=0, help="--placement pool: chunk size (0 = the library's 64)")
     ap.add_argument("--pool-slab-mb", type=int, default=0, help="--placement pool: unit of the region scan, 512 ... 4096 (0 = the library's 1024)")
     ap.add_argument("--grads-one-region", type=int, default=0,
@@ -1038,6 +1048,8 @@ def main():
     three_placements = args.placement == "pool" and (args.placements == 1 or (args.placements == -1 and full_default))
     # first: before anything here touches the GPU, so that on a fresh box the child's are the first allocations
     plain_leg = child_leg(args, "plain") if three_placements and args.plain_leg == "first" else None
+    if plain_leg is not None:
+        time.sleep(8.0 if args.settle_s < 0 else args.settle_s)   # the child's memory is on its way back to the driver
 
     import torch
     import mxopt
@@ -1062,12 +1074,18 @@ def main():
         if three_placements or args.placement == "state-pool":
             host_side = sum(sizes) * 2 * 5 + (4 << 30) if args.workload == "cfg5" else free // 2
         try:
-            pool = ctx.hbm_pool(free - (8 << 30) - host_side, args.pool_chunk_mb << 20, args.pool_regions,
+            want = int(args.pool_gib * 2**30) if args.pool_gib > 0 else free - (8 << 30) - host_side
+            pool = ctx.hbm_pool(want, args.pool_chunk_mb << 20, args.pool_regions,
                                 slab_bytes=args.pool_slab_mb << 20)
         except mxopt.MxoptError as e:
             # e.g. another process holds most of the device: measure in plain memory and say so in the line
             print(f"bench.py: no region-interleaved arena ({e}); buffers come from plain device memory", file=sys.stderr)
             placement = {"kind": "plain", "arena_refused": str(e)}
+    if pool is not None:
+        gave_back = free - pool.info().capacity_bytes > (16 << 30)
+        settle = args.settle_s if args.settle_s >= 0 else (4.0 if gave_back else 0.0)
+        if settle > 0:
+            time.sleep(settle)
     if pool is not None:
         pool.use_for_state()
         i = pool.info()
@@ -1148,6 +1166,8 @@ def main():
         w3 = Workload(a, torch, mxopt, ctx, pool)
         state_pool_leg = leg_summary(measure(w3, 5, 2), w3, 5)
         w3.close()
+        # that leg's parameters and gradients (80 GB of plain memory) have just gone back to the driver
+        time.sleep(4.0 if args.settle_s < 0 else args.settle_s)
         placement["plain_leg_ran"] = args.plain_leg
         legs = placement["legs"] = {
             "arena (every buffer from the pool; the headline)": main_leg,

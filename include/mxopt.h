@@ -123,12 +123,17 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * aligned, first fit, thread-safe; contents are not cleared.  A pointer goes back to the pool it came
  * from whichever pool a context or the hooks point at by then.  Destroy the pool after everything that
  * allocated from it and before its context.
- * One pool per process, made at start-up.  The scan reads the regions off runs of consecutively created
- * chunks: a process's first pool sees such runs (on a fresh device, after other processes came and went, after
- * the process itself allocated and freed tens of GB), but once a pool has taken all memory chunk by chunk and
- * given most of it back, chunks come in no physical order any more: a second pool made by the same process
- * finds mixtures (every pair of 1 GiB groups answers at an in-between rate), reports whatever grouping the
- * rates suggest, and its arena is interleaved by accident rather than by design.
+ * One pool per device at a time, made at start-up, and not within about ten seconds of a large release of
+ * device memory.  The driver takes released memory back asynchronously: for a few seconds after tens of GB were
+ * freed (a pool destroyed, this function's own hand-back of what the arena does not need, another process that
+ * has just exited) every kernel on the device runs about 0.7 % slower, taking memory chunk by chunk is several
+ * times slower, and a scan made in that time reads rates that belong to nothing: a second pool created right
+ * after the first was destroyed found four groups and interleaved 138 of 200 GiB in 8.8 s, ten seconds later
+ * three regions and 192 GiB in 1.8 s.  So wait before creating a pool after such a release, and allow about
+ * three seconds after this function before timing anything.  A pool created while another pool or another
+ * large allocation is alive only sees what is left, in pieces smaller than its 1 GiB groups: every pair of
+ * groups answers at an in-between rate, it reports whatever grouping the rates suggest, and its arena is
+ * interleaved by accident rather than by design.
  * No counterpart in the reference (MLX owns its allocator there). */
 #define MXOPT_HBM_MAX_REGIONS 8
 typedef struct mxopt_hbm_pool mxopt_hbm_pool;
