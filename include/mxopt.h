@@ -129,8 +129,10 @@ int mxopt_hbm_spread_end(mxopt_hbm_spread* s);
  * has just exited) every kernel on the device runs about 0.7 % slower, taking memory chunk by chunk is several
  * times slower, and a scan made in that time reads rates that belong to nothing: a second pool created right
  * after the first was destroyed found four groups and interleaved 138 of 200 GiB in 8.8 s, ten seconds later
- * three regions and 192 GiB in 1.8 s.  So wait before creating a pool after such a release, and allow about
- * three seconds after this function before timing anything.  A pool created while another pool or another
+ * three regions and 192 GiB in 1.8 s.  This function notices by the slow creation of its chunks, hands everything
+ * back, waits four seconds and takes the memory again, at most twice (create_seconds then reads 10 - 15 s); a
+ * host does better to wait by itself before creating a pool after such a release.  Allow about three seconds
+ * after this function before timing anything: it hands back what the arena does not need.  A pool created while another pool or another
  * large allocation is alive only sees what is left, in pieces smaller than its 1 GiB groups: every pair of
  * groups answers at an in-between rate, it reports whatever grouping the rates suggest, and its arena is
  * interleaved by accident rather than by design.

@@ -19,6 +19,7 @@
 #include <map>
 #include <mutex>
 #include <new>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -215,6 +216,17 @@ constexpr size_t kSlabChunksBytes = (size_t)1 << 30;  // chunks are classified i
 // The driver limits the live allocations of a process (about 60 000 were seen to succeed) and maps fewer still.
 constexpr size_t kMaxChunks = 24000;
 
+// Taking the free memory as chunks, measured on 286 GiB: 0.08 - 0.13 s as 4,566 chunks of 64 MiB and 0.56 - 2.06 s as
+// 18,266 of 16 MiB on a quiet device (under 0.5 ms per GiB plus 0.03 - 0.11 ms per chunk), 3.9 s as 64 MiB chunks
+// (13.6 ms per GiB) while the driver is still taking back memory released a moment ago.  Slower than this bound the
+// call hands everything back, waits and starts over.  (With 16 MiB chunks the sign is weaker -- 2.2 - 4.6 s busy
+// against 0.6 - 2.1 s quiet -- and the bound only catches the worse cases; 64 MiB is the default for more than one
+// reason.)
+constexpr double kBusyCreateSecondsPerGiB = 0.004;
+constexpr double kBusyCreateSecondsPerChunk = 0.00015;
+constexpr int kMaxTakeAttempts = 3;
+constexpr int kBusyWaitMs = 4000;
+
 struct Builder {  // everything pool creation holds until it either succeeds or fails
   mxopt_ctx* ctx;
   std::vector<hipMemGenericAllocationHandle_t> all;
@@ -362,16 +374,35 @@ int mxopt_hbm_pool_create_ex(mxopt_ctx* ctx, const mxopt_hbm_pool_options* optio
 
   // 1. The free memory as physical chunks: memory far from what a small allocation would get can only be
   //    reached by holding what lies in between.
+  //    The driver takes released memory back asynchronously: within seconds of a large release (a pool that was
+  //    just destroyed, a process that has just exited) chunk creation is thirty times slower than on a quiet
+  //    device, and a scan made then reads rates that mean nothing (measured: four groups, 138 of
+  //    200 GiB interleaved, against three regions and 192 GiB ten seconds later).  Creation that slow is taken as
+  //    the sign: everything goes back, the call waits and takes the memory again, at most twice.
   Builder b{ctx};
   const hipMemAllocationProp prop = device_prop(ctx->device);
   b.all.reserve(avail_chunks);
-  for (size_t i = 0; i < avail_chunks; ++i) {
-    hipMemGenericAllocationHandle_t h;
-    if (hipMemCreate(&h, chunk_bytes, &prop, 0) != hipSuccess) {
-      (void)hipGetLastError();
-      break;
+  int take_attempts = 0;
+  for (;;) {
+    ++take_attempts;
+    const auto t_take = std::chrono::steady_clock::now();
+    for (size_t i = 0; i < avail_chunks; ++i) {
+      hipMemGenericAllocationHandle_t h;
+      if (hipMemCreate(&h, chunk_bytes, &prop, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        break;
+      }
+      b.all.push_back(h);
     }
-    b.all.push_back(h);
+    const double took = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_take).count();
+    const double gib = (double)b.all.size() * (double)chunk_bytes / (double)((size_t)1 << 30);
+    const bool busy = gib >= 16.0 && took > kBusyCreateSecondsPerGiB * gib + kBusyCreateSecondsPerChunk * (double)b.all.size();
+    MXOPT_DEBUG("hbm pool: %zu chunks taken in %.2f s (%.1f ms per GiB)%s", b.all.size(), took,
+                gib > 0 ? took * 1e3 / gib : 0.0, busy ? ": the driver is busy taking memory back" : "");
+    if (!busy || take_attempts >= kMaxTakeAttempts) break;
+    for (hipMemGenericAllocationHandle_t h : b.all) (void)hipMemRelease(h);
+    b.all.clear();
+    std::this_thread::sleep_for(std::chrono::milliseconds(kBusyWaitMs));
   }
   b.released.assign(b.all.size(), 0);
   const auto t_created = std::chrono::steady_clock::now();
