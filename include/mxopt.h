@@ -150,7 +150,7 @@ typedef struct mxopt_hbm_pool_info {
   double probe_same_region_gbps;                         /* the probe with all four streams in one region */
   double probe_cross_region_gbps;                        /* ... with two of them in another (0 if regions == 1) */
   double setup_seconds;                                  /* whole of mxopt_hbm_pool_create */
-  double create_seconds;                                 /* ... of which taking the free memory as chunks */
+  double create_seconds;                                 /* ... of which taking the free memory as chunks (with the waits and retakes when the driver was busy) */
   double scan_seconds;                                   /* ... and timing probes to find the regions */
   int32_t probes;                                        /* probe measurements taken */
   int32_t reserved2_;
